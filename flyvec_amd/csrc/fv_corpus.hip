@@ -1,0 +1,324 @@
+// Host half of the window sampler, done on the device: window count, window-start table and
+// inverse unigram frequency.  Restates flyvec/src/prune_input.cpp:64-122 and
+// flyvec/src/model_arrays.cu:396-424 as data-parallel passes:
+//   * the running sum of chunk lengths the reference keeps (prune_input.cpp:103-115) telescopes
+//     to offsets[s] - offsets[0] (uint64 arithmetic, wrap-around included), so a window start
+//     is offsets[s] - offsets[0] + i;
+//   * the output slot of a chunk's first window is an exclusive prefix sum of per-chunk window
+//     counts (three-pass scan: block totals, scan of totals, rescan + expansion);
+//   * the reference counts occurrences in an fp32 accumulator, which stops at 2^24; an integer
+//     histogram clamped to 2^24 gives the same value.
+#include "fv_internal.h"
+
+#define FV_MAXLEN 214ull  // flyvec/src/prune_input.cpp:7
+#define FV_SCAN_THREADS 256
+#define FV_SCAN_ITEMS 8
+#define FV_SCAN_TILE (FV_SCAN_THREADS * FV_SCAN_ITEMS)
+
+__device__ __forceinline__ uint64_t fv_chunk_windows(const uint64_t *__restrict__ off, uint64_t s,
+                                                     uint64_t n_chunks, uint64_t w) {
+  if (s >= n_chunks) return 0;
+  uint64_t len = off[s + 1] - off[s];
+  return (len >= w && len < FV_MAXLEN) ? len - w + 1 : 0;
+}
+
+__device__ __forceinline__ uint64_t fv_block_sum_u64(uint64_t v, uint64_t *smem /*4*/) {
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_down(v, d, 64);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __syncthreads();
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  return smem[0] + smem[1] + smem[2] + smem[3];
+}
+
+// Pass 1: total number of windows of each tile of FV_SCAN_TILE chunks.
+__global__ __launch_bounds__(FV_SCAN_THREADS) void fv_tile_totals_kernel(
+    const uint64_t *__restrict__ off, uint64_t n_chunks, uint64_t w, uint64_t *__restrict__ totals) {
+  __shared__ uint64_t smem[4];
+  const uint64_t base = (uint64_t)blockIdx.x * FV_SCAN_TILE + (uint64_t)threadIdx.x * FV_SCAN_ITEMS;
+  uint64_t v = 0;
+#pragma unroll
+  for (int j = 0; j < FV_SCAN_ITEMS; ++j) v += fv_chunk_windows(off, base + j, n_chunks, w);
+  uint64_t t = fv_block_sum_u64(v, smem);
+  if (threadIdx.x == 0) totals[blockIdx.x] = t;
+}
+
+// Pass 2: exclusive scan of the tile totals by one block; totals[n_tiles] receives the sum.
+__global__ __launch_bounds__(FV_SCAN_THREADS) void fv_scan_totals_kernel(uint64_t *totals,
+                                                                         uint64_t n_tiles) {
+  __shared__ uint64_t part[FV_SCAN_THREADS];
+  __shared__ uint64_t carry;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (uint64_t b0 = 0; b0 < n_tiles; b0 += FV_SCAN_THREADS) {
+    uint64_t i = b0 + threadIdx.x;
+    uint64_t v = i < n_tiles ? totals[i] : 0;
+    part[threadIdx.x] = v;
+    __syncthreads();
+    for (int d = 1; d < FV_SCAN_THREADS; d <<= 1) {  // Hillis-Steele inclusive scan
+      uint64_t add = threadIdx.x >= (unsigned)d ? part[threadIdx.x - d] : 0;
+      __syncthreads();
+      part[threadIdx.x] += add;
+      __syncthreads();
+    }
+    uint64_t incl = part[threadIdx.x];
+    uint64_t c = carry;
+    if (i < n_tiles) totals[i] = c + incl - v;
+    __syncthreads();
+    if (threadIdx.x == FV_SCAN_THREADS - 1) carry = c + incl;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) totals[n_tiles] = carry;
+}
+
+// Pass 3: each thread rescans its FV_SCAN_ITEMS chunks and writes their window starts.
+__global__ __launch_bounds__(FV_SCAN_THREADS) void fv_expand_starts_kernel(
+    const uint64_t *__restrict__ off, uint64_t n_chunks, uint64_t w,
+    const uint64_t *__restrict__ tile_base, uint64_t *__restrict__ starts, uint64_t n_windows) {
+  __shared__ uint64_t part[FV_SCAN_THREADS];
+  const uint64_t base = (uint64_t)blockIdx.x * FV_SCAN_TILE + (uint64_t)threadIdx.x * FV_SCAN_ITEMS;
+  uint64_t cnt[FV_SCAN_ITEMS];
+  uint64_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < FV_SCAN_ITEMS; ++j) {
+    cnt[j] = fv_chunk_windows(off, base + j, n_chunks, w);
+    mine += cnt[j];
+  }
+  part[threadIdx.x] = mine;
+  __syncthreads();
+  for (int d = 1; d < FV_SCAN_THREADS; d <<= 1) {
+    uint64_t add = threadIdx.x >= (unsigned)d ? part[threadIdx.x - d] : 0;
+    __syncthreads();
+    part[threadIdx.x] += add;
+    __syncthreads();
+  }
+  uint64_t out = tile_base[blockIdx.x] + part[threadIdx.x] - mine;
+  const uint64_t off0 = off[0];
+#pragma unroll
+  for (int j = 0; j < FV_SCAN_ITEMS; ++j) {
+    if (cnt[j]) {
+      uint64_t first = off[base + j] - off0;
+      for (uint64_t i = 0; i < cnt[j]; ++i)
+        if (out + i < n_windows) starts[out + i] = first + i;
+      out += cnt[j];
+    }
+  }
+}
+
+static int fv_scan_windows(const uint64_t *offsets_dev, uint64_t n_chunks, uint64_t w,
+                           uint64_t **out_tile_base, uint64_t *out_total, hipStream_t stream) {
+  const uint64_t n_tiles = (n_chunks + FV_SCAN_TILE - 1) / FV_SCAN_TILE;
+  FV_REQUIRE(n_tiles < (1ull << 31), FV_ERR_INVALID, "too many chunks (%llu)",
+             (unsigned long long)n_chunks);
+  uint64_t *totals = nullptr;
+  FV_HIP(hipMalloc((void **)&totals, (n_tiles + 1) * sizeof(uint64_t)));
+  if (n_tiles)
+    hipLaunchKernelGGL(fv_tile_totals_kernel, dim3((unsigned)n_tiles), dim3(FV_SCAN_THREADS), 0,
+                       stream, offsets_dev, n_chunks, w, totals);
+  hipLaunchKernelGGL(fv_scan_totals_kernel, dim3(1), dim3(FV_SCAN_THREADS), 0, stream, totals,
+                     n_tiles);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(out_total, totals + n_tiles, sizeof(uint64_t), hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) {
+    (void)hipFree(totals);
+    return fv_fail(FV_ERR_HIP, "window scan failed: %s", hipGetErrorString(e));
+  }
+  if (out_tile_base)
+    *out_tile_base = totals;
+  else
+    (void)hipFree(totals);
+  return FV_OK;
+}
+
+int fv_dev_count_windows(const uint64_t *offsets_dev, uint64_t n_chunks, uint64_t w,
+                         uint64_t *out_count_host, hipStream_t stream) {
+  return fv_scan_windows(offsets_dev, n_chunks, w, nullptr, out_count_host, stream);
+}
+
+int fv_dev_build_window_starts(const uint64_t *offsets_dev, uint64_t n_chunks, uint64_t w,
+                               uint64_t *starts_dev, uint64_t n_windows, hipStream_t stream) {
+  uint64_t *tile_base = nullptr;
+  uint64_t total = 0;
+  FV_TRY(fv_scan_windows(offsets_dev, n_chunks, w, &tile_base, &total, stream));
+  int rc = FV_OK;
+  if (total != n_windows) {
+    rc = fv_fail(FV_ERR_INVALID, "window table capacity %llu does not match the %llu windows found",
+                 (unsigned long long)n_windows, (unsigned long long)total);
+  } else if (n_chunks) {
+    const uint64_t n_tiles = (n_chunks + FV_SCAN_TILE - 1) / FV_SCAN_TILE;
+    hipLaunchKernelGGL(fv_expand_starts_kernel, dim3((unsigned)n_tiles), dim3(FV_SCAN_THREADS), 0,
+                       stream, offsets_dev, n_chunks, w, tile_base, starts_dev, n_windows);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "window expansion failed: %s", hipGetErrorString(e));
+  }
+  (void)hipFree(tile_base);
+  return rc;
+}
+
+// ---- inverse unigram frequency ---------------------------------------------------------
+#define FV_HIST_LDS 12288  // ids below this are counted in LDS first (Zipf head), the rest in HBM
+
+__global__ __launch_bounds__(256) void fv_histogram_kernel(const int32_t *__restrict__ corpus,
+                                                           uint64_t n_tokens, uint32_t vocab,
+                                                           uint32_t *__restrict__ counts,
+                                                           int32_t *__restrict__ minmax) {
+  __shared__ uint32_t hist[FV_HIST_LDS];
+  for (int i = threadIdx.x; i < FV_HIST_LDS; i += 256) hist[i] = 0;
+  __syncthreads();
+  int32_t lo = 0x7fffffff, hi = -0x7fffffff - 1;
+  const uint64_t stride = (uint64_t)gridDim.x * 256;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n_tokens; i += stride) {
+    int32_t t = corpus[i];
+    lo = t < lo ? t : lo;
+    hi = t > hi ? t : hi;
+    if (t >= 0 && (uint32_t)t < vocab) {
+      if (t < FV_HIST_LDS)
+        atomicAdd(&hist[t], 1u);
+      else
+        atomicAdd(&counts[t], 1u);
+    }
+  }
+  __syncthreads();
+  const uint32_t lim = vocab < FV_HIST_LDS ? vocab : FV_HIST_LDS;
+  for (uint32_t i = threadIdx.x; i < lim; i += 256)
+    if (hist[i]) atomicAdd(&counts[i], hist[i]);
+  for (int d = 32; d >= 1; d >>= 1) {
+    int32_t ol = __shfl_down(lo, d, 64), oh = __shfl_down(hi, d, 64);
+    lo = ol < lo ? ol : lo;
+    hi = oh > hi ? oh : hi;
+  }
+  if ((threadIdx.x & 63) == 0 && lo <= hi) {
+    atomicMin(&minmax[0], lo);
+    atomicMax(&minmax[1], hi);
+  }
+}
+
+__global__ void fv_invert_counts_kernel(const uint32_t *__restrict__ counts, uint32_t vocab,
+                                        float *__restrict__ invf) {
+  uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= vocab) return;
+  uint32_t c = counts[i];
+  if (c > (1u << 24)) c = 1u << 24;  // where the reference's fp32 counter stops
+  invf[i] = c ? (float)(1.0 / (double)(float)c) : 0.0f;
+}
+
+int fv_dev_inverse_frequency(const int32_t *corpus_dev, uint64_t n_tokens, uint64_t vocab,
+                             float *invf_dev, int32_t *out_min_host, int32_t *out_max_host,
+                             hipStream_t stream) {
+  FV_REQUIRE(vocab > 0 && vocab < (1ull << 30), FV_ERR_INVALID, "vocabulary size %llu out of range",
+             (unsigned long long)vocab);
+  FV_REQUIRE(n_tokens < (1ull << 32), FV_ERR_INVALID, "corpus of %llu tokens exceeds 2^32",
+             (unsigned long long)n_tokens);
+  uint32_t *counts = nullptr;
+  FV_HIP(hipMalloc((void **)&counts, vocab * sizeof(uint32_t) + 2 * sizeof(int32_t)));
+  int32_t *minmax = (int32_t *)(counts + vocab);
+  int32_t init[2] = {0x7fffffff, -0x7fffffff - 1};
+  hipError_t e = hipMemsetAsync(counts, 0, vocab * sizeof(uint32_t), stream);
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(minmax, init, sizeof init, hipMemcpyHostToDevice, stream);
+  if (e == hipSuccess && n_tokens) {
+    uint64_t want = (n_tokens + 256 * 16 - 1) / (256 * 16);
+    unsigned blocks = (unsigned)(want < 1 ? 1 : (want > 2048 ? 2048 : want));
+    hipLaunchKernelGGL(fv_histogram_kernel, dim3(blocks), dim3(256), 0, stream, corpus_dev, n_tokens,
+                       (uint32_t)vocab, counts, minmax);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess) {
+    hipLaunchKernelGGL(fv_invert_counts_kernel, dim3((unsigned)((vocab + 255) / 256)), dim3(256), 0,
+                       stream, counts, (uint32_t)vocab, invf_dev);
+    e = hipGetLastError();
+  }
+  int32_t mm[2] = {0, 0};
+  if (e == hipSuccess) e = hipMemcpyAsync(mm, minmax, sizeof mm, hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  (void)hipFree(counts);
+  if (e != hipSuccess) return fv_fail(FV_ERR_HIP, "inverse frequency failed: %s", hipGetErrorString(e));
+  if (out_min_host) *out_min_host = mm[0];
+  if (out_max_host) *out_max_host = mm[1];
+  return FV_OK;
+}
+
+// ---- C ABI on host buffers ---------------------------------------------------------------
+
+static int fv_upload_offsets(const uint64_t *offsets, uint64_t n_chunks, uint64_t **out_dev) {
+  FV_HIP(hipMalloc((void **)out_dev, (n_chunks + 1) * sizeof(uint64_t)));
+  hipError_t e = hipMemcpy(*out_dev, offsets, (n_chunks + 1) * sizeof(uint64_t), hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipFree(*out_dev);
+    *out_dev = nullptr;
+    return fv_fail(FV_ERR_HIP, "offset upload failed: %s", hipGetErrorString(e));
+  }
+  return FV_OK;
+}
+
+extern "C" int fv_count_windows(const uint64_t *offsets, uint64_t n_chunks, uint64_t w,
+                                uint64_t *out_count) {
+  FV_REQUIRE(out_count, FV_ERR_INVALID, "fv_count_windows: null output");
+  *out_count = 0;
+  if (n_chunks == 0) return FV_OK;
+  FV_REQUIRE(offsets, FV_ERR_INVALID, "fv_count_windows: null offsets");
+  FV_REQUIRE(w >= 1, FV_ERR_INVALID, "fv_count_windows: window length must be >= 1");
+  uint64_t *d = nullptr;
+  FV_TRY(fv_upload_offsets(offsets, n_chunks, &d));
+  int rc = fv_dev_count_windows(d, n_chunks, w, out_count, 0);
+  (void)hipFree(d);
+  return rc;
+}
+
+extern "C" int fv_build_window_starts(const uint64_t *offsets, uint64_t n_chunks, uint64_t w,
+                                      uint64_t *out_starts, uint64_t capacity) {
+  if (n_chunks == 0) return FV_OK;
+  FV_REQUIRE(offsets, FV_ERR_INVALID, "fv_build_window_starts: null offsets");
+  FV_REQUIRE(w >= 1, FV_ERR_INVALID, "fv_build_window_starts: window length must be >= 1");
+  uint64_t *d = nullptr, *s = nullptr;
+  FV_TRY(fv_upload_offsets(offsets, n_chunks, &d));
+  uint64_t total = 0;
+  int rc = fv_dev_count_windows(d, n_chunks, w, &total, 0);
+  if (rc == FV_OK && total > capacity)
+    rc = fv_fail(FV_ERR_INVALID, "fv_build_window_starts: %llu windows do not fit capacity %llu",
+                 (unsigned long long)total, (unsigned long long)capacity);
+  if (rc == FV_OK && total) {
+    FV_REQUIRE(out_starts, FV_ERR_INVALID, "fv_build_window_starts: null output");
+    hipError_t e = hipMalloc((void **)&s, total * sizeof(uint64_t));
+    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "hipMalloc failed: %s", hipGetErrorString(e));
+    if (rc == FV_OK) rc = fv_dev_build_window_starts(d, n_chunks, w, s, total, 0);
+    if (rc == FV_OK) {
+      e = hipMemcpy(out_starts, s, total * sizeof(uint64_t), hipMemcpyDeviceToHost);
+      if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
+    }
+  }
+  (void)hipFree(d);
+  (void)hipFree(s);
+  return rc;
+}
+
+extern "C" int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, uint64_t vocab,
+                                    float *out_invf) {
+  FV_REQUIRE(out_invf, FV_ERR_INVALID, "fv_inverse_frequency: null output");
+  FV_REQUIRE(corpus || n_tokens == 0, FV_ERR_INVALID, "fv_inverse_frequency: null corpus");
+  int32_t *dc = nullptr;
+  float *df = nullptr;
+  FV_HIP(hipMalloc((void **)&df, vocab * sizeof(float)));
+  int rc = FV_OK;
+  hipError_t e = hipSuccess;
+  if (n_tokens) {
+    e = hipMalloc((void **)&dc, n_tokens * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMemcpy(dc, corpus, n_tokens * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "corpus upload failed: %s", hipGetErrorString(e));
+  }
+  int32_t lo = 0, hi = 0;
+  if (rc == FV_OK) rc = fv_dev_inverse_frequency(dc, n_tokens, vocab, df, &lo, &hi, 0);
+  if (rc == FV_OK && n_tokens && hi >= 0 && (uint64_t)hi >= vocab)
+    rc = fv_fail(FV_ERR_DATA, "token id %d is outside the vocabulary of %llu", hi,
+                 (unsigned long long)vocab);
+  if (rc == FV_OK) {
+    e = hipMemcpy(out_invf, df, vocab * sizeof(float), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
+  }
+  (void)hipFree(dc);
+  (void)hipFree(df);
+  return rc;
+}

@@ -1,0 +1,463 @@
+// Batched top-k hashing: FlyVec.get_sparse_embedding (flyvec/core.py:139-163) for many target
+// ids or many context windows at once.
+//
+// One wavefront per window.  The activation (fp32 sum of the window's token rows, in window
+// order) lives in registers, neuron h = lane + 64 j in register j of its lane.  The reference
+// sorts all K activations (core.py:155) but only uses the k-th and (k+1)-th largest:
+//     thr = fl32(a[k-1] + a[k]) / 2;  code = act > thr            (core.py:157-158)
+// so the kernel selects instead of sorting: a bit-by-bit search from the most significant bit of
+// an order-preserving integer key finds the largest threshold with at least k keys at or above
+// it; each probe is one compare per register and a population count of the resulting lane mask.
+// The search stops as soon as exactly k keys pass (the top-k set is then known; its minimum and
+// the maximum of the rest are the two order statistics) and otherwise ends on the exact k-th key,
+// with ties at the boundary counted with multiplicity as the sort does.  A compare's lane mask is
+// also exactly one 64-bit word of the packed code, so bit packing costs nothing.
+#include <math.h>
+#include <string.h>
+
+#include <vector>
+
+#include "fv_internal.h"
+
+struct fv_hasher {
+  uint32_t K, ldk;
+  uint64_t N;
+  hipStream_t stream;
+  float *Wt;
+  uint32_t *err;  // device flag: a column index outside [-1, N) was met
+  unsigned max_blocks;
+};
+
+struct fv_hash_args {
+  const float *Wt;
+  const int32_t *idx;
+  uint64_t n;
+  uint32_t w, k, K, ldk, n_cols;
+  int32_t shift;  // added to every index (V for target ids, 0 for window columns)
+  uint64_t *out_bits;
+  int8_t *out_codes;
+  uint32_t *err;
+};
+
+template <int NV, int RB>
+__device__ __forceinline__ void fv_hash_gather(const float *__restrict__ Wt, uint32_t ldk, uint32_t K,
+                                               int lane, int w, int32_t idx_lane, float (&acc)[NV]) {
+  for (int c0 = 0; c0 < w; c0 += RB) {
+    float v[RB][NV];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      const int c = c0 + b;
+      const int32_t i = (int32_t)fv_readlane((uint32_t)idx_lane, c < 63 ? c : 63);
+      const bool ok = (c < w) && (i >= 0);
+      const float *row = Wt + (uint64_t)(ok ? i : 0) * ldk + lane;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const bool in = ok && (j < NV - 1 || (uint32_t)(lane + 64 * j) < K);
+        v[b][j] = in ? row[64 * j] : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+      for (int j = 0; j < NV; ++j) acc[j] = __fadd_rn(acc[j], v[b][j]);
+  }
+}
+
+template <int NV>
+__global__ __launch_bounds__(256) void fv_hash_kernel(fv_hash_args a) {
+  constexpr int RB = NV <= 2 ? 16 : NV <= 4 ? 8 : NV <= 8 ? 4 : NV <= 16 ? 2 : 1;
+  const int lane = threadIdx.x & 63;
+  const uint64_t n_waves = (uint64_t)gridDim.x * 4;
+  for (uint64_t r = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6); r < a.n; r += n_waves) {
+    int32_t idx = -1;
+    if (lane < (int)a.w) {
+      const int32_t raw = a.idx[r * a.w + lane];
+      if (raw != -1 || a.shift != 0) {
+        const int64_t col = (int64_t)raw + a.shift;
+        if (raw >= 0 && col < (int64_t)a.n_cols)
+          idx = (int32_t)col;
+        else
+          atomicOr(a.err, 1u);
+      }
+    }
+
+    float acc[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) acc[j] = 0.0f;
+    fv_hash_gather<NV, RB>(a.Wt, a.ldk, a.K, lane, (int)a.w, idx, acc);
+
+    uint32_t key[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const bool valid = (j < NV - 1) || (uint32_t)(lane + 64 * j) < a.K;
+      key[j] = valid ? fv_ord_key(acc[j]) : 0u;  // pads sort below every real value
+    }
+
+    // largest cand with count(key >= cand) >= k, built from the top bit down
+    uint32_t cand = 0, c_at = 0;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t t = cand | (1u << bit);
+      uint32_t c = 0;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) c += (uint32_t)__popcll(__ballot(key[j] >= t));
+      if (c >= a.k) {
+        cand = t;
+        c_at = c;
+        if (c == a.k) break;
+      }
+    }
+    uint32_t lo = 0xffffffffu, hi = 0u;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      if (key[j] >= cand) lo = key[j] < lo ? key[j] : lo;
+      else hi = key[j] > hi ? key[j] : hi;
+    }
+    const float a_k = fv_ord_unkey(fv_wave_min_u32(lo));  // k-th largest
+    const float a_k1 = c_at > a.k ? a_k : fv_ord_unkey(fv_wave_max_u32(hi));  // (k+1)-th largest
+    const float thr = __fmul_rn(__fadd_rn(a_k, a_k1), 0.5f);
+
+    uint64_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const bool valid = (j < NV - 1) || (uint32_t)(lane + 64 * j) < a.K;
+      const bool on = valid && acc[j] > thr;
+      const uint64_t m = __ballot(on);
+      if (lane == j) mine = m;
+      if (a.out_codes && valid) a.out_codes[r * a.K + lane + 64 * j] = on ? 1 : 0;
+    }
+    if (a.out_bits && lane < NV) a.out_bits[r * NV + lane] = mine;
+  }
+}
+
+template <int NV>
+static void fv_launch_hash(const fv_hash_args &a, unsigned blocks, hipStream_t stream) {
+  hipLaunchKernelGGL(fv_hash_kernel<NV>, dim3(blocks), dim3(256), 0, stream, a);
+}
+
+static int fv_enqueue_hash(fv_hasher *h, const int32_t *idx_dev, uint64_t n, uint32_t w, uint32_t k,
+                           int32_t shift, uint64_t *bits_dev, int8_t *codes_dev) {
+  if (n == 0) return FV_OK;
+  fv_hash_args a;
+  a.Wt = h->Wt;
+  a.idx = idx_dev;
+  a.n = n;
+  a.w = w;
+  a.k = k;
+  a.K = h->K;
+  a.ldk = h->ldk;
+  a.n_cols = (uint32_t)h->N;
+  a.shift = shift;
+  a.out_bits = bits_dev;
+  a.out_codes = codes_dev;
+  a.err = h->err;
+  uint64_t want = (n + 3) / 4;
+  unsigned blocks = (unsigned)(want < h->max_blocks ? want : h->max_blocks);
+  switch ((h->K + 63) / 64) {
+#define FV_CASE(NV) case NV: fv_launch_hash<NV>(a, blocks, h->stream); break;
+    FV_CASE(1) FV_CASE(2) FV_CASE(3) FV_CASE(4) FV_CASE(5) FV_CASE(6) FV_CASE(7) FV_CASE(8)
+    FV_CASE(9) FV_CASE(10) FV_CASE(11) FV_CASE(12) FV_CASE(13) FV_CASE(14) FV_CASE(15) FV_CASE(16)
+    FV_CASE(17) FV_CASE(18) FV_CASE(19) FV_CASE(20) FV_CASE(21) FV_CASE(22) FV_CASE(23) FV_CASE(24)
+    FV_CASE(25) FV_CASE(26) FV_CASE(27) FV_CASE(28) FV_CASE(29) FV_CASE(30) FV_CASE(31) FV_CASE(32)
+#undef FV_CASE
+    default:
+      return fv_fail(FV_ERR_INVALID, "hid = %u not supported", h->K);
+  }
+  FV_HIP(hipGetLastError());
+  return FV_OK;
+}
+
+static int fv_check_hash_args(fv_hasher *h, uint32_t w, uint32_t k) {
+  FV_REQUIRE(h, FV_ERR_INVALID, "null hasher");
+  FV_REQUIRE(w >= 1 && w <= FV_MAX_WINDOW, FV_ERR_INVALID, "window = %u is outside 1..%d", w,
+             FV_MAX_WINDOW);
+  FV_REQUIRE(k >= 1 && k < h->K, FV_ERR_INVALID,
+             "hash length k = %u must satisfy 0 < k < %u (the k-th and (k+1)-th largest are read)", k,
+             h->K);
+  return FV_OK;
+}
+
+extern "C" int fv_hasher_destroy(fv_hasher *h) {
+  if (!h) return FV_OK;
+  if (h->stream) (void)hipStreamSynchronize(h->stream);
+  (void)hipFree(h->Wt);
+  (void)hipFree(h->err);
+  if (h->stream) (void)hipStreamDestroy(h->stream);
+  delete h;
+  return FV_OK;
+}
+
+extern "C" int fv_hasher_create(const float *W, uint32_t hid, uint64_t n_columns, fv_hasher **out_hasher) {
+  FV_REQUIRE(W && out_hasher, FV_ERR_INVALID, "fv_hasher_create: null argument");
+  *out_hasher = nullptr;
+  FV_REQUIRE(hid >= 2 && hid <= FV_MAX_HID, FV_ERR_INVALID, "hid = %u is outside 2..%d", hid, FV_MAX_HID);
+  FV_REQUIRE(n_columns >= 1 && n_columns < (1ull << 31), FV_ERR_INVALID, "n_columns = %llu out of range",
+             (unsigned long long)n_columns);
+  fv_hasher *h = new fv_hasher();
+  memset(h, 0, sizeof *h);
+  h->K = hid;
+  h->ldk = fv_ldk(hid);
+  h->N = n_columns;
+  int cus = 0;
+  int rc = fv_device_info(nullptr, 0, &cus, nullptr);
+  h->max_blocks = (unsigned)(cus > 0 ? cus : 256) * 8;
+  hipError_t e = hipSuccess;
+  if (rc == FV_OK) {
+    e = hipStreamCreate(&h->stream);
+    if (e == hipSuccess) e = hipMalloc((void **)&h->Wt, (size_t)h->N * h->ldk * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc((void **)&h->err, sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMemsetAsync(h->err, 0, sizeof(uint32_t), h->stream);
+    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "hasher allocation failed: %s", hipGetErrorString(e));
+  }
+  if (rc == FV_OK) rc = fv_upload_weights(W, h->Wt, h->K, h->N, h->ldk, h->stream);
+  if (rc != FV_OK) {
+    fv_hasher_destroy(h);
+    return rc;
+  }
+  *out_hasher = h;
+  return FV_OK;
+}
+
+extern "C" int fv_hasher_get_weights(fv_hasher *h, float *out_W) {
+  FV_REQUIRE(h && out_W, FV_ERR_INVALID, "null argument");
+  return fv_download_weights(h->Wt, out_W, h->K, h->N, h->ldk, h->stream);
+}
+
+extern "C" int fv_hasher_sync(fv_hasher *h) {
+  FV_REQUIRE(h, FV_ERR_INVALID, "null hasher");
+  FV_HIP(hipStreamSynchronize(h->stream));
+  uint32_t err = 0;
+  FV_HIP(hipMemcpy(&err, h->err, sizeof err, hipMemcpyDeviceToHost));
+  if (err) {
+    FV_HIP(hipMemset(h->err, 0, sizeof err));
+    return fv_fail(FV_ERR_DATA, "a column index outside [-1, %llu) was met; its position was skipped",
+                   (unsigned long long)h->N);
+  }
+  return FV_OK;
+}
+
+extern "C" int fv_hash_windows_dev(fv_hasher *h, const int32_t *idx_dev, uint64_t n, uint32_t w, uint32_t k,
+                                   uint64_t *out_bits_dev, int8_t *out_codes_dev) {
+  FV_TRY(fv_check_hash_args(h, w, k));
+  FV_REQUIRE(idx_dev || n == 0, FV_ERR_INVALID, "null index buffer");
+  return fv_enqueue_hash(h, idx_dev, n, w, k, 0, out_bits_dev, out_codes_dev);
+}
+
+static int fv_hash_host(fv_hasher *h, const int32_t *idx, uint64_t n, uint32_t w, uint32_t k, int32_t shift,
+                        uint64_t *out_bits, int8_t *out_codes) {
+  if (n == 0) return FV_OK;
+  FV_REQUIRE(idx, FV_ERR_INVALID, "null index buffer");
+  const uint32_t words = (h->K + 63) / 64;
+  int32_t *d_idx = nullptr;
+  uint64_t *d_bits = nullptr;
+  int8_t *d_codes = nullptr;
+  int rc = FV_OK;
+  hipError_t e = hipMalloc((void **)&d_idx, n * w * sizeof(int32_t));
+  if (e == hipSuccess && out_bits) e = hipMalloc((void **)&d_bits, n * words * sizeof(uint64_t));
+  if (e == hipSuccess && out_codes) e = hipMalloc((void **)&d_codes, n * (uint64_t)h->K);
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(d_idx, idx, n * w * sizeof(int32_t), hipMemcpyHostToDevice, h->stream);
+  if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "hash staging failed: %s", hipGetErrorString(e));
+  if (rc == FV_OK) rc = fv_enqueue_hash(h, d_idx, n, w, k, shift, d_bits, d_codes);
+  if (rc == FV_OK && out_bits) {
+    e = hipMemcpyAsync(out_bits, d_bits, n * words * sizeof(uint64_t), hipMemcpyDeviceToHost, h->stream);
+    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
+  }
+  if (rc == FV_OK && out_codes) {
+    e = hipMemcpyAsync(out_codes, d_codes, n * (uint64_t)h->K, hipMemcpyDeviceToHost, h->stream);
+    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
+  }
+  int rs = fv_hasher_sync(h);
+  if (rc == FV_OK) rc = rs;
+  (void)hipFree(d_idx);
+  (void)hipFree(d_bits);
+  (void)hipFree(d_codes);
+  return rc;
+}
+
+extern "C" int fv_hash_windows(fv_hasher *h, const int32_t *idx, uint64_t n, uint32_t w, uint32_t k,
+                               uint64_t *out_bits, int8_t *out_codes) {
+  FV_TRY(fv_check_hash_args(h, w, k));
+  return fv_hash_host(h, idx, n, w, k, 0, out_bits, out_codes);
+}
+
+extern "C" int fv_hash_targets(fv_hasher *h, const int32_t *ids, uint64_t n, uint32_t k, int8_t *out_codes) {
+  FV_TRY(fv_check_hash_args(h, 1, k));
+  FV_REQUIRE(h->N % 2 == 0, FV_ERR_INVALID, "the matrix has %llu columns; targets need 2V",
+             (unsigned long long)h->N);
+  FV_REQUIRE(out_codes || n == 0, FV_ERR_INVALID, "null output");
+  // target block = columns [V, 2V) (flyvec/core.py:179); ids outside [0, V) are reported
+  const uint64_t V = h->N / 2;
+  for (uint64_t i = 0; i < n; ++i)
+    FV_REQUIRE(ids && ids[i] >= 0 && (uint64_t)ids[i] < V, FV_ERR_DATA,
+               "token id %d at position %llu is outside [0, %llu)", ids ? ids[i] : 0,
+               (unsigned long long)i, (unsigned long long)V);
+  return fv_hash_host(h, ids, n, 1, k, (int32_t)V, nullptr, out_codes);
+}
+
+extern "C" int fv_hasher_time_windows(fv_hasher *h, const int32_t *idx_dev, uint64_t n, uint32_t w, uint32_t k,
+                                      uint64_t *out_bits_dev, int8_t *out_codes_dev, uint32_t reps,
+                                      float *out_mean_ms) {
+  FV_TRY(fv_check_hash_args(h, w, k));
+  FV_REQUIRE(out_mean_ms && reps >= 1, FV_ERR_INVALID, "bad timing arguments");
+  hipEvent_t e0, e1;
+  FV_HIP(hipEventCreate(&e0));
+  FV_HIP(hipEventCreate(&e1));
+  FV_HIP(hipStreamSynchronize(h->stream));
+  FV_HIP(hipEventRecord(e0, h->stream));
+  int rc = FV_OK;
+  for (uint32_t i = 0; i < reps && rc == FV_OK; ++i)
+    rc = fv_enqueue_hash(h, idx_dev, n, w, k, 0, out_bits_dev, out_codes_dev);
+  FV_HIP(hipEventRecord(e1, h->stream));
+  FV_HIP(hipStreamSynchronize(h->stream));
+  float ms = 0.0f;
+  FV_HIP(hipEventElapsedTime(&ms, e0, e1));
+  *out_mean_ms = ms / (float)reps;
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return rc;
+}
+
+// ---- normalisation (flyvec/core.py:23-36, p = 2) -----------------------------------------------
+// numpy sums each row of syn**2 with its pairwise scheme: blocks of at most 128 elements are
+// summed with 8 interleaved accumulators combined as ((r0+r1)+(r2+r3))+((r4+r5)+(r6+r7)) plus a
+// sequential tail; longer ranges split at n/2 rounded down to a multiple of 8. The leaves of that
+// recursion are independent (first kernel); their combination order is a fixed tree replayed by a
+// small stack program (second kernel).
+
+struct fv_leaf {
+  uint32_t start, len;
+};
+
+static void fv_pairwise_plan(uint32_t start, uint32_t n, std::vector<fv_leaf> &leaves,
+                             std::vector<int32_t> &prog) {
+  if (n <= 128) {
+    prog.push_back((int32_t)leaves.size());
+    leaves.push_back({start, n});
+    return;
+  }
+  uint32_t n2 = n / 2;
+  n2 -= n2 % 8;
+  fv_pairwise_plan(start, n2, leaves, prog);
+  fv_pairwise_plan(start + n2, n - n2, leaves, prog);
+  prog.push_back(-1);  // pop two, push their sum
+}
+
+__global__ __launch_bounds__(256) void fv_leaf_sumsq_kernel(const float *__restrict__ Wt, uint32_t K,
+                                                            uint32_t ldk, const fv_leaf *__restrict__ leaves,
+                                                            float *__restrict__ leaf_sums) {
+  const uint32_t h = blockIdx.y * 256 + threadIdx.x;
+  if (h >= K) return;
+  const fv_leaf lf = leaves[blockIdx.x];
+  const float *col = Wt + (uint64_t)lf.start * ldk + h;
+#define FV_SQ(i) __fmul_rn(col[(uint64_t)(i) * ldk], col[(uint64_t)(i) * ldk])
+  float res;
+  if (lf.len < 8) {
+    res = -0.0f;
+    for (uint32_t i = 0; i < lf.len; ++i) res = __fadd_rn(res, FV_SQ(i));
+  } else {
+    float r[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) r[k] = FV_SQ(k);
+    uint32_t i = 8;
+    for (; i < lf.len - (lf.len % 8); i += 8) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) r[k] = __fadd_rn(r[k], FV_SQ(i + k));
+    }
+    res = __fadd_rn(__fadd_rn(__fadd_rn(r[0], r[1]), __fadd_rn(r[2], r[3])),
+                    __fadd_rn(__fadd_rn(r[4], r[5]), __fadd_rn(r[6], r[7])));
+    for (; i < lf.len; ++i) res = __fadd_rn(res, FV_SQ(i));
+  }
+#undef FV_SQ
+  leaf_sums[(uint64_t)blockIdx.x * K + h] = res;
+}
+
+__global__ void fv_combine_leaves_kernel(const float *__restrict__ leaf_sums, uint32_t K,
+                                         const int32_t *__restrict__ prog, uint32_t prog_len,
+                                         float *__restrict__ out) {
+  const uint32_t h = blockIdx.x * blockDim.x + threadIdx.x;
+  if (h >= K) return;
+  float stack[40];
+  int sp = 0;
+  for (uint32_t i = 0; i < prog_len; ++i) {
+    const int32_t op = prog[i];
+    if (op >= 0) {
+      stack[sp++] = leaf_sums[(uint64_t)op * K + h];
+    } else {
+      const float b = stack[--sp];
+      const float a = stack[--sp];
+      stack[sp++] = __fadd_rn(a, b);
+    }
+  }
+  // the reduction starts from add's identity: 0 + pairwise sum
+  out[h] = __fadd_rn(0.0f, stack[0]);
+}
+
+__global__ __launch_bounds__(256) void fv_scale_rows_kernel(float *__restrict__ Wt, uint64_t N, uint32_t K,
+                                                            uint32_t ldk, const float *__restrict__ div) {
+  const uint64_t total = N * ldk;
+  for (uint64_t p = (uint64_t)blockIdx.x * 256 + threadIdx.x; p < total; p += (uint64_t)gridDim.x * 256) {
+    const uint32_t h = (uint32_t)(p % ldk);
+    if (h < K) Wt[p] = Wt[p] / div[h];
+  }
+}
+
+// out_sums[h] = numpy.sum(W[h]**2) in numpy's fp32 pairwise order
+extern "C" int fv_hasher_row_sumsq(fv_hasher *h, float *out_sums) {
+  FV_REQUIRE(h && out_sums, FV_ERR_INVALID, "null argument");
+  std::vector<fv_leaf> leaves;
+  std::vector<int32_t> prog;
+  fv_pairwise_plan(0, (uint32_t)h->N, leaves, prog);
+  fv_leaf *d_leaves = nullptr;
+  int32_t *d_prog = nullptr;
+  float *d_leaf = nullptr, *d_out = nullptr;
+  hipError_t e = hipMalloc((void **)&d_leaves, leaves.size() * sizeof(fv_leaf));
+  if (e == hipSuccess) e = hipMalloc((void **)&d_prog, prog.size() * sizeof(int32_t));
+  if (e == hipSuccess) e = hipMalloc((void **)&d_leaf, leaves.size() * (size_t)h->K * sizeof(float));
+  if (e == hipSuccess) e = hipMalloc((void **)&d_out, (size_t)h->K * sizeof(float));
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(d_leaves, leaves.data(), leaves.size() * sizeof(fv_leaf), hipMemcpyHostToDevice, h->stream);
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(d_prog, prog.data(), prog.size() * sizeof(int32_t), hipMemcpyHostToDevice, h->stream);
+  if (e == hipSuccess) {
+    hipLaunchKernelGGL(fv_leaf_sumsq_kernel, dim3((unsigned)leaves.size(), (h->K + 255) / 256), dim3(256), 0,
+                       h->stream, h->Wt, h->K, h->ldk, d_leaves, d_leaf);
+    hipLaunchKernelGGL(fv_combine_leaves_kernel, dim3((h->K + 63) / 64), dim3(64), 0, h->stream, d_leaf, h->K,
+                       d_prog, (uint32_t)prog.size(), d_out);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(out_sums, d_out, (size_t)h->K * sizeof(float), hipMemcpyDeviceToHost, h->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(h->stream);
+  (void)hipFree(d_leaves);
+  (void)hipFree(d_prog);
+  (void)hipFree(d_leaf);
+  (void)hipFree(d_out);
+  if (e != hipSuccess) return fv_fail(FV_ERR_HIP, "row sums failed: %s", hipGetErrorString(e));
+  return FV_OK;
+}
+
+// W[h][:] /= divisors[h] (fp32 division, correctly rounded)
+extern "C" int fv_hasher_scale_rows(fv_hasher *h, const float *divisors) {
+  FV_REQUIRE(h && divisors, FV_ERR_INVALID, "null argument");
+  float *d = nullptr;
+  FV_HIP(hipMalloc((void **)&d, (size_t)h->K * sizeof(float)));
+  hipError_t e = hipMemcpyAsync(d, divisors, (size_t)h->K * sizeof(float), hipMemcpyHostToDevice, h->stream);
+  if (e == hipSuccess) {
+    hipLaunchKernelGGL(fv_scale_rows_kernel, dim3(h->max_blocks), dim3(256), 0, h->stream, h->Wt, h->N, h->K,
+                       h->ldk, d);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(h->stream);
+  (void)hipFree(d);
+  if (e != hipSuccess) return fv_fail(FV_ERR_HIP, "row scaling failed: %s", hipGetErrorString(e));
+  return FV_OK;
+}
+
+extern "C" int fv_hasher_normalize(fv_hasher *h, float prec) {
+  FV_REQUIRE(h, FV_ERR_INVALID, "null hasher");
+  std::vector<float> sums(h->K);
+  FV_TRY(fv_hasher_row_sumsq(h, sums.data()));
+  // power(x, 1/2) taken as the correctly rounded square root
+  for (auto &v : sums) v = sqrtf(v) + prec;
+  return fv_hasher_scale_rows(h, sums.data());
+}

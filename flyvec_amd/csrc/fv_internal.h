@@ -1,0 +1,136 @@
+// Internal declarations shared by the translation units of libflyvec_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "flyvec_hip.h"
+
+#define FV_WAVE 64
+#define FV_MAX_HID 2048   // 32 values per lane in the wave-per-window kernels
+#define FV_MAX_WINDOW 64  // one lane per window position
+
+// ---- error plumbing -------------------------------------------------------------
+int fv_fail(int code, const char *fmt, ...);
+void fv_clear_error();
+
+#define FV_HIP(call)                                                                          \
+  do {                                                                                        \
+    hipError_t e__ = (call);                                                                  \
+    if (e__ != hipSuccess)                                                                    \
+      return fv_fail(FV_ERR_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e__),      \
+                     __FILE__, __LINE__);                                                     \
+  } while (0)
+
+#define FV_TRY(call)          \
+  do {                        \
+    int rc__ = (call);        \
+    if (rc__ != FV_OK) return rc__; \
+  } while (0)
+
+#define FV_REQUIRE(cond, code, ...)              \
+  do {                                           \
+    if (!(cond)) return fv_fail(code, __VA_ARGS__); \
+  } while (0)
+
+// ---- device layout of the synapse matrix -----------------------------------------
+// Token-major: column i of the K x N checkpoint matrix is the contiguous row
+// Wt[i * ldk .. i * ldk + K), ldk = K rounded up to a multiple of 4 floats so every
+// row starts 16-byte aligned; the pad is kept at zero.
+static inline uint32_t fv_ldk(uint32_t K) { return (K + 3u) & ~3u; }
+
+// K x N row-major (staging, device) <-> token-major N x ldk (device). Asynchronous.
+int fv_launch_to_token_major(const float *W_rowmajor_dev, float *Wt_dev, uint32_t K, uint64_t N,
+                             uint32_t ldk, hipStream_t stream);
+int fv_launch_to_row_major(const float *Wt_dev, float *W_rowmajor_dev, uint32_t K, uint64_t N,
+                           uint32_t ldk, hipStream_t stream);
+// Upload / download a K x N host matrix through a temporary device staging buffer.
+int fv_upload_weights(const float *W_host, float *Wt_dev, uint32_t K, uint64_t N, uint32_t ldk,
+                      hipStream_t stream);
+int fv_download_weights(const float *Wt_dev, float *W_host, uint32_t K, uint64_t N, uint32_t ldk,
+                        hipStream_t stream);
+
+// ---- corpus kernels (fv_corpus.hip) ----------------------------------------------
+// All pointers are device memory.
+int fv_dev_count_windows(const uint64_t *offsets_dev, uint64_t n_chunks, uint64_t w,
+                         uint64_t *out_count_host, hipStream_t stream);
+int fv_dev_build_window_starts(const uint64_t *offsets_dev, uint64_t n_chunks, uint64_t w,
+                               uint64_t *starts_dev, uint64_t n_windows, hipStream_t stream);
+int fv_dev_inverse_frequency(const int32_t *corpus_dev, uint64_t n_tokens, uint64_t vocab,
+                             float *invf_dev, int32_t *out_min_host, int32_t *out_max_host,
+                             hipStream_t stream);
+
+// ---- wave-level helpers used by the window kernels --------------------------------
+// Order-preserving map fp32 -> uint32 (a < b  <=>  key(a) < key(b) for non-NaN a, b).
+__device__ __forceinline__ uint32_t fv_ord_key(float f) {
+  uint32_t u = __float_as_uint(f);
+  return u ^ (uint32_t)(((int32_t)u >> 31) | 0x80000000);
+}
+__device__ __forceinline__ float fv_ord_unkey(uint32_t k) {
+  uint32_t u = (k & 0x80000000u) ? (k ^ 0x80000000u) : ~k;
+  return __uint_as_float(u);
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t fv_dpp(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, 0xf, 0xf, false);
+}
+
+// Lane patterns that, applied in sequence with an idempotent commutative operator, leave
+// the reduction over each 16-lane row in every lane of that row.
+#define FV_DPP_QUAD_XOR1 0xB1  // quad_perm [1,0,3,2]
+#define FV_DPP_QUAD_XOR2 0x4E  // quad_perm [2,3,0,1]
+#define FV_DPP_ROW_ROR4 0x124
+#define FV_DPP_ROW_ROR8 0x128
+
+__device__ __forceinline__ uint32_t fv_readlane(uint32_t v, int lane) {
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, lane);
+}
+
+// Wave-uniform maximum of a 64-bit key over all 64 lanes (all lanes must be active).
+__device__ __forceinline__ uint64_t fv_wave_max_u64(uint64_t v) {
+#define FV_STEP64(CTRL)                                                 \
+  {                                                                     \
+    uint32_t lo = fv_dpp<CTRL>((uint32_t)v), hi = fv_dpp<CTRL>((uint32_t)(v >> 32)); \
+    uint64_t o = ((uint64_t)hi << 32) | lo;                             \
+    v = o > v ? o : v;                                                  \
+  }
+  FV_STEP64(FV_DPP_QUAD_XOR1)
+  FV_STEP64(FV_DPP_QUAD_XOR2)
+  FV_STEP64(FV_DPP_ROW_ROR4)
+  FV_STEP64(FV_DPP_ROW_ROR8)
+#undef FV_STEP64
+  uint64_t r = 0;
+#pragma unroll
+  for (int row = 0; row < 4; ++row) {
+    uint64_t x = ((uint64_t)fv_readlane((uint32_t)(v >> 32), row * 16) << 32) |
+                 fv_readlane((uint32_t)v, row * 16);
+    r = x > r ? x : r;
+  }
+  return r;
+}
+
+__device__ __forceinline__ uint32_t fv_wave_max_u32(uint32_t v) {
+#define FV_STEP32(CTRL)              \
+  {                                  \
+    uint32_t o = fv_dpp<CTRL>(v);    \
+    v = o > v ? o : v;               \
+  }
+  FV_STEP32(FV_DPP_QUAD_XOR1)
+  FV_STEP32(FV_DPP_QUAD_XOR2)
+  FV_STEP32(FV_DPP_ROW_ROR4)
+  FV_STEP32(FV_DPP_ROW_ROR8)
+#undef FV_STEP32
+  uint32_t r = 0;
+#pragma unroll
+  for (int row = 0; row < 4; ++row) {
+    uint32_t x = fv_readlane(v, row * 16);
+    r = x > r ? x : r;
+  }
+  return r;
+}
+
+__device__ __forceinline__ uint32_t fv_wave_min_u32(uint32_t v) { return ~fv_wave_max_u32(~v); }
+

@@ -1,0 +1,237 @@
+"""Python handles over the C ABI: ``Trainer`` (the minibatch step) and ``Hasher`` (top-k codes).
+
+These are thin: every operation is one call into libflyvec_hip.so; numpy is used only for the
+host buffers that cross the boundary.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import check, ptr
+
+
+def count_windows(offsets, w):
+    """flyvec/src/prune_input.cpp:64 getnum_samples."""
+    offsets = np.ascontiguousarray(offsets, dtype=np.uint64)
+    out = C.c_uint64(0)
+    check(_lib.load().fv_count_windows(ptr(offsets), max(len(offsets) - 1, 0), w, C.byref(out)))
+    return out.value
+
+
+def window_starts(offsets, w):
+    """flyvec/src/prune_input.cpp:88 compute_offset_phrases."""
+    offsets = np.ascontiguousarray(offsets, dtype=np.uint64)
+    n = count_windows(offsets, w)
+    out = np.empty(n, dtype=np.uint64)
+    check(_lib.load().fv_build_window_starts(ptr(offsets), max(len(offsets) - 1, 0), w, ptr(out), n))
+    return out
+
+
+def inverse_frequency(corpus, vocab):
+    """flyvec/src/model_arrays.cu:396 compute_inverse_word_frequency."""
+    corpus = np.ascontiguousarray(corpus, dtype=np.int32)
+    out = np.empty(int(vocab), dtype=np.float32)
+    check(_lib.load().fv_inverse_frequency(ptr(corpus), len(corpus), int(vocab), ptr(out)))
+    return out
+
+
+class Trainer:
+    """Owns the synapse matrix, the corpus and the window table in HBM."""
+
+    def __init__(self, vocab, hid=400, window=11, batch=10000, initial_learning_rate=0.002,
+                 delta=0.0, prec=1.0e-30, tie_rule=0):
+        self.lib = _lib.load()
+        self.vocab, self.hid, self.window, self.batch = int(vocab), int(hid), int(window), int(batch)
+        cfg = _lib.TrainConfig(vocab=self.vocab, hid=self.hid, window=self.window, batch=self.batch,
+                               tie_rule=int(tie_rule), initial_learning_rate=initial_learning_rate,
+                               delta=delta, prec=prec, reserved=0)
+        h = C.c_void_p()
+        check(self.lib.fv_trainer_create(C.byref(cfg), C.byref(h)))
+        self.handle = h
+
+    def close(self):
+        if getattr(self, "handle", None) is not None and self.handle.value:
+            self.lib.fv_trainer_destroy(self.handle)
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    # -- set-up ---------------------------------------------------------------------------
+    def set_corpus(self, tokens, offsets):
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        offsets = np.ascontiguousarray(offsets, dtype=np.uint64)
+        check(self.lib.fv_trainer_set_corpus(self.handle, ptr(tokens), len(tokens), ptr(offsets), len(offsets)))
+
+    @property
+    def num_windows(self):
+        out = C.c_uint64(0)
+        check(self.lib.fv_trainer_num_windows(self.handle, C.byref(out)))
+        return out.value
+
+    def window_starts(self):
+        out = np.empty(self.num_windows, dtype=np.uint64)
+        check(self.lib.fv_trainer_get_window_starts(self.handle, ptr(out), len(out)))
+        return out
+
+    def inverse_frequency(self):
+        out = np.empty(self.vocab, dtype=np.float32)
+        check(self.lib.fv_trainer_get_inverse_frequency(self.handle, ptr(out)))
+        return out
+
+    def set_weights(self, W):
+        W = np.ascontiguousarray(W, dtype=np.float32)
+        if W.shape != (self.hid, 2 * self.vocab):
+            raise ValueError(f"weights must be ({self.hid}, {2 * self.vocab}), got {W.shape}")
+        check(self.lib.fv_trainer_set_weights(self.handle, ptr(W)))
+
+    def get_weights(self):
+        out = np.empty((self.hid, 2 * self.vocab), dtype=np.float32)
+        check(self.lib.fv_trainer_get_weights(self.handle, ptr(out)))
+        return out
+
+    def shuffle(self, seed=0):
+        check(self.lib.fv_trainer_shuffle(self.handle, int(seed)))
+
+    def set_permutation(self, perm):
+        perm = np.ascontiguousarray(perm, dtype=np.uint64)
+        check(self.lib.fv_trainer_set_permutation(self.handle, ptr(perm), len(perm)))
+
+    def get_permutation(self):
+        out = np.empty(self.num_windows, dtype=np.uint64)
+        check(self.lib.fv_trainer_get_permutation(self.handle, ptr(out), len(out)))
+        return out
+
+    # -- the hot path ------------------------------------------------------------------------
+    def step(self, first_window, n_windows, eps):
+        check(self.lib.fv_trainer_step(self.handle, int(first_window), int(n_windows), float(eps)))
+
+    def run_epoch(self, epoch_id, n_epochs):
+        check(self.lib.fv_trainer_run_epoch(self.handle, int(epoch_id), int(n_epochs)))
+
+    def epoch_eps(self, epoch_id, n_epochs):
+        out = C.c_float(0)
+        check(self.lib.fv_trainer_epoch_eps(self.handle, int(epoch_id), int(n_epochs), C.byref(out)))
+        return out.value
+
+    def sync(self):
+        check(self.lib.fv_trainer_sync(self.handle))
+
+    def winners(self, n):
+        out = np.empty(int(n), dtype=np.int32)
+        check(self.lib.fv_trainer_get_winners(self.handle, ptr(out), len(out)))
+        return out
+
+    def step_stats(self):
+        xx = np.empty(self.hid, dtype=np.float32)
+        nc = C.c_float(0)
+        check(self.lib.fv_trainer_get_step_stats(self.handle, ptr(xx), C.byref(nc)))
+        return xx, nc.value
+
+    def row_norms(self, n_rows=10):
+        n_rows = min(int(n_rows), self.hid)
+        out = np.empty(n_rows, dtype=np.float64)
+        check(self.lib.fv_trainer_row_norms(self.handle, n_rows, ptr(out)))
+        return out
+
+    def time_steps(self, first_window, n_steps, eps, per_kernel=True):
+        total = C.c_float(0)
+        kern = (C.c_float * _lib.FV_TRAIN_KERNELS)()
+        check(self.lib.fv_trainer_time_steps(self.handle, int(first_window), int(n_steps), float(eps),
+                                             C.byref(total), kern if per_kernel else None))
+        return total.value, dict(zip(_lib.TRAIN_KERNEL_NAMES, list(kern))) if per_kernel else None
+
+
+class Hasher:
+    """A checkpoint matrix resident in HBM plus the batched top-k threshold code."""
+
+    def __init__(self, W):
+        self.lib = _lib.load()
+        W = np.ascontiguousarray(W, dtype=np.float32)
+        if W.ndim != 2:
+            raise ValueError("synapse matrix must be 2-D (K, N)")
+        self.hid, self.n_columns = W.shape
+        self.words = (self.hid + 63) // 64
+        h = C.c_void_p()
+        check(self.lib.fv_hasher_create(ptr(W), self.hid, self.n_columns, C.byref(h)))
+        self.handle = h
+
+    def close(self):
+        if getattr(self, "handle", None) is not None and self.handle.value:
+            self.lib.fv_hasher_destroy(self.handle)
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def normalize(self, prec=1.0e-32, p=2):
+        """flyvec/core.py:23-36 on the resident matrix: the two passes over the matrix run on the
+        device; the p-th root of the K row sums is numpy's, as in the reference."""
+        if p != 2:
+            raise NotImplementedError("only p = 2 (the reference's default) is built")
+        sums = np.empty(self.hid, dtype=np.float32)
+        check(self.lib.fv_hasher_row_sumsq(self.handle, ptr(sums)))
+        nc = np.power(sums, 1 / p).reshape(self.hid, 1)
+        div = np.ascontiguousarray((nc + prec).reshape(-1), dtype=np.float32)
+        check(self.lib.fv_hasher_scale_rows(self.handle, ptr(div)))
+
+    def weights(self):
+        out = np.empty((self.hid, self.n_columns), dtype=np.float32)
+        check(self.lib.fv_hasher_get_weights(self.handle, ptr(out)))
+        return out
+
+    def _check_k(self, k):
+        if not 0 < k < self.hid:
+            # the reference reads act_sort[k] (flyvec/core.py:157)
+            raise IndexError(f"hash length {k} is out of bounds for {self.hid} neurons")
+
+    def hash_targets(self, ids, k=50):
+        self._check_k(k)
+        ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
+        out = np.empty((len(ids), self.hid), dtype=np.int8)
+        check(self.lib.fv_hash_targets(self.handle, ptr(ids), len(ids), k, ptr(out)))
+        return out
+
+    def hash_windows(self, idx, k=50, packed=True, codes=False):
+        """idx (n, w) int32 column indices (-1 = masked). Returns packed uint64 words, int8 codes,
+        or both as a tuple."""
+        self._check_k(k)
+        idx = np.ascontiguousarray(idx, dtype=np.int32)
+        if idx.ndim != 2:
+            raise ValueError("idx must be (n, w)")
+        n, w = idx.shape
+        bits = np.empty((n, self.words), dtype=np.uint64) if packed else None
+        cds = np.empty((n, self.hid), dtype=np.int8) if codes else None
+        check(self.lib.fv_hash_windows(self.handle, ptr(idx), n, w, k, ptr(bits), ptr(cds)))
+        if packed and codes:
+            return bits, cds
+        return bits if packed else cds
+
+    def hash_windows_dev(self, idx_buf, n, w, k, bits_buf=None, codes_buf=None):
+        self._check_k(k)
+        check(self.lib.fv_hash_windows_dev(self.handle, idx_buf.ptr, n, w, k,
+                                           bits_buf.ptr if bits_buf else None,
+                                           codes_buf.ptr if codes_buf else None))
+
+    def sync(self):
+        check(self.lib.fv_hasher_sync(self.handle))
+
+    def time_windows(self, idx_buf, n, w, k, bits_buf=None, codes_buf=None, reps=10):
+        ms = C.c_float(0)
+        check(self.lib.fv_hasher_time_windows(self.handle, idx_buf.ptr, n, w, k,
+                                              bits_buf.ptr if bits_buf else None,
+                                              codes_buf.ptr if codes_buf else None, reps, C.byref(ms)))
+        return ms.value

@@ -1,0 +1,199 @@
+/*
+ * flyvec_hip.h -- C ABI of libflyvec_hip.so: the FlyVec training minibatch step and
+ * the top-k hashing path on one AMD MI355X (gfx950).
+ *
+ * One shared library replaces the five CUDA shared objects the reference's Python
+ * driver loads with ctypes (flyvec/train_flyvec.py:62-66) and adds the batched form
+ * of FlyVec.get_sparse_embedding (flyvec/core.py:139-163).  Every entry point cites
+ * the reference interface it stands in for.  Unlike the reference (void returns,
+ * exit() on error, flyvec/src/cuda_funcs.cu:36-54) every function returns a status
+ * and leaves a message for fv_last_error(); nothing here terminates the process.
+ *
+ * Conventions: plain pointers and sizes only.  Unless a name ends in _dev, pointer
+ * arguments are HOST memory owned by the caller.  The synapse matrix crosses this
+ * boundary exactly as the reference's checkpoint stores it: fp32, K x 2V, row-major
+ * (flyvec/train_flyvec.py:245-263; context block = columns [0,V), target block =
+ * [V,2V), flyvec/src/cuda_funcs.cu:929-932).  Handles are thread-compatible, not
+ * thread-safe.  The library uses device 0 unless fv_set_device() is called first.
+ */
+#ifndef FLYVEC_HIP_H
+#define FLYVEC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FV_OK 0
+#define FV_ERR_INVALID 1 /* bad argument or shape */
+#define FV_ERR_HIP 2     /* a HIP runtime call failed */
+#define FV_ERR_STATE 3   /* call order: corpus / weights / permutation not set */
+#define FV_ERR_DATA 4    /* input data violates the contract (token id out of range, ...) */
+
+/* ---- runtime ------------------------------------------------------------------ */
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *fv_last_error(void);
+
+/* flyvec/src/cuda_helpers.cu:31 get_cuda_num_devices */
+int fv_device_count(int *out_count);
+int fv_set_device(int device);
+/* Name, compute units and HBM bytes of the current device (for logs and the bench). */
+int fv_device_info(char *name, size_t name_cap, int *out_compute_units, uint64_t *out_hbm_bytes);
+
+/* flyvec/src/cuda_helpers.cu:22 do_gpu_cudaHostAlloc (pinned host staging memory) */
+int fv_host_alloc_pinned(size_t bytes, void **out_ptr);
+int fv_host_free_pinned(void *ptr);
+
+/* flyvec/src/cuda_helpers.cu:8 do_gpu_cudaMallocManaged -- the reference keeps every
+ * buffer in managed memory; here device buffers are explicit.  Used by callers that
+ * keep hash inputs / outputs resident in HBM (the *_dev entry points). */
+int fv_dev_alloc(size_t bytes, void **out_dev_ptr);
+int fv_dev_free(void *dev_ptr);
+int fv_dev_upload(void *dst_dev, const void *src_host, size_t bytes);
+int fv_dev_download(void *dst_host, const void *src_dev, size_t bytes);
+
+/* ---- window sampler, host half ------------------------------------------------ */
+
+/* flyvec/src/prune_input.cpp:64 getnum_samples: number of length-w windows that do not
+ * cross a chunk boundary, over chunks with w <= length < 214. offsets has n_chunks+1
+ * entries. */
+int fv_count_windows(const uint64_t *offsets, uint64_t n_chunks, uint64_t w, uint64_t *out_count);
+
+/* flyvec/src/prune_input.cpp:88 compute_offset_phrases: corpus position of every window,
+ * in chunk order; a start is the sum of all previous chunk LENGTHS plus the position in
+ * the chunk (offsets[0] is assumed 0, as the reference does). out_starts must hold
+ * `capacity` >= fv_count_windows entries. */
+int fv_build_window_starts(const uint64_t *offsets, uint64_t n_chunks, uint64_t w,
+                           uint64_t *out_starts, uint64_t capacity);
+
+/* flyvec/src/model_arrays.cu:396 compute_inverse_word_frequency: out[t] = 1/count(t) over
+ * the whole corpus, 0 for absent ids, negative ids ignored; counts saturate at 2^24 as the
+ * reference's fp32 counter does. */
+int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, uint64_t vocab, float *out_invf);
+
+/* ---- trainer ------------------------------------------------------------------ */
+
+typedef struct fv_trainer fv_trainer;
+
+/* The hyper-parameters flyvec/train_flyvec.py:191-213 pushes through set_model_param_int /
+ * set_model_param_float (flyvec/src/model_descriptor.cu:51-87). */
+typedef struct fv_train_config {
+  uint64_t vocab;              /* V ("vocabulary_size"); W is hid x 2V */
+  uint32_t hid;                /* K ("hid"), 1..2048 */
+  uint32_t window;             /* w ("W"), 1..64 */
+  uint32_t batch;              /* B ("Num"), windows per minibatch */
+  uint32_t tie_rule;           /* argmax ties: 0 lowest index, 1 the reference's lane-tree order
+                                  (flyvec/src/cuda_funcs.cu:488-561) */
+  float initial_learning_rate; /* "initial_learning_rate" */
+  float delta;                 /* "delta": must be 0 (anti-Hebbian term not built) */
+  float prec;                  /* "prec" */
+  uint32_t reserved;           /* 0 */
+} fv_train_config;
+
+/* flyvec/src/model_descriptor.cu:18 model_create_descriptor + flyvec/src/model_arrays.cu:15,22
+ * model_create_arrays / model_arrays_allocate_memory */
+int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_trainer);
+int fv_trainer_destroy(fv_trainer *t);
+
+/* flyvec/src/model_arrays.cu:358 set_up_INPUT_pointer + :396 compute_inverse_word_frequency
+ * + flyvec/src/prune_input.cpp:88: uploads the corpus (int32 ids in [0,V) or -1) and builds
+ * the window-start table, 1/frequency and the identity permutation in HBM. offsets has
+ * n_offsets entries (n_offsets-1 chunks). Fails with FV_ERR_DATA on ids outside [-1, V). */
+int fv_trainer_set_corpus(fv_trainer *t, const int32_t *tokens, uint64_t n_tokens,
+                          const uint64_t *offsets, uint64_t n_offsets);
+int fv_trainer_num_windows(fv_trainer *t, uint64_t *out_count);
+/* Read-back of what set_corpus built (parity hooks). */
+int fv_trainer_get_window_starts(fv_trainer *t, uint64_t *out_starts, uint64_t capacity);
+int fv_trainer_get_inverse_frequency(fv_trainer *t, float *out_invf);
+
+/* flyvec/src/model_arrays.cu:305 get_data_pointer("synapses"): the reference hands Python a
+ * pointer into managed memory; here the matrix is copied in / out (K x 2V fp32 row-major). */
+int fv_trainer_set_weights(fv_trainer *t, const float *W);
+int fv_trainer_get_weights(fv_trainer *t, float *out_W);
+
+/* flyvec/src/model_arrays.cu:442 do_reshuffle_indices: for i in order swap(perm[i],
+ * perm[r_i mod Nwin]), cumulative across calls.  The reference draws r from cuRAND's
+ * scrambled Sobol64; here r is a splitmix64 stream seeded by `seed`. */
+int fv_trainer_shuffle(fv_trainer *t, uint64_t seed);
+/* Test hook replacing the random stream: install / read the window permutation. */
+int fv_trainer_set_permutation(fv_trainer *t, const uint64_t *perm, uint64_t n);
+int fv_trainer_get_permutation(fv_trainer *t, uint64_t *out_perm, uint64_t capacity);
+
+/* One pass of the minibatch loop body, flyvec/src/cuda_funcs.cu:1662-1803, on windows
+ * perm[first_window .. first_window + n_windows) with n_windows <= batch. Asynchronous. */
+int fv_trainer_step(fv_trainer *t, uint64_t first_window, uint32_t n_windows, float eps);
+
+/* flyvec/src/cuda_funcs.cu:1220 launch_epoch_INPUT_AS_INT: eps = lr0 * (1 - epoch/n_epochs),
+ * then every minibatch of the current permutation (the last one takes the remainder only).
+ * Returns after the device has finished. */
+int fv_trainer_run_epoch(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs);
+/* eps of flyvec/src/cuda_funcs.cu:1229 for this trainer's learning rate. */
+int fv_trainer_epoch_eps(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs, float *out_eps);
+
+int fv_trainer_sync(fv_trainer *t);
+
+/* Parity hooks on the last step: winner per window (max_IDs[r][0], flyvec/src/cuda_funcs.cu:
+ * 1719), per-neuron totals xx (:1721) and max|ds| (flyvec/src/cu_special_reduction.cu:241). */
+int fv_trainer_get_winners(fv_trainer *t, int32_t *out_winners, uint32_t capacity);
+int fv_trainer_get_step_stats(fv_trainer *t, float *out_xx /* hid */, float *out_max_abs_ds);
+
+/* flyvec/src/cuda_funcs.cu:1234-1242: L2 norm of the first n_rows rows of W (the reference
+ * prints them for 10 rows before every epoch). */
+int fv_trainer_row_norms(fv_trainer *t, uint32_t n_rows, double *out_norms);
+
+/* Measurement: n_steps consecutive full minibatches starting at first_window, timed with HIP
+ * events on the trainer's stream. out_total_ms covers all steps; out_kernel_ms[FV_TRAIN_KERNELS]
+ * (nullable) receives the mean duration of each kernel of the step, measured in a second,
+ * separately instrumented run of the same steps. */
+#define FV_TRAIN_KERNELS 4 /* gather+winner, xx totals, max|ds|, update */
+int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint32_t n_steps, float eps,
+                          float *out_total_ms, float *out_kernel_ms);
+
+/* ---- hashing ------------------------------------------------------------------ */
+
+typedef struct fv_hasher fv_hasher;
+
+/* flyvec/core.py:82-88 (FlyVec.synapses): takes the checkpoint matrix (K x N fp32 row-major,
+ * N = 2V) and keeps it resident in HBM. */
+int fv_hasher_create(const float *W, uint32_t hid, uint64_t n_columns, fv_hasher **out_hasher);
+int fv_hasher_destroy(fv_hasher *h);
+
+/* flyvec/core.py:23-36 normalize_synapses, p = 2: each row divided by (sqrt(sum of squares)
+ * + prec), sum taken in numpy's pairwise fp32 order. In place on the resident matrix. */
+int fv_hasher_normalize(fv_hasher *h, float prec);
+/* The two device passes of that normalisation, for callers that take the p-th root themselves
+ * (numpy's power(x, 1/p) is what the reference calls): out_sums[r] = sum_i W[r][i]^2 in numpy's
+ * pairwise fp32 order; then W[r][:] /= divisors[r]. */
+int fv_hasher_row_sumsq(fv_hasher *h, float *out_sums /* hid */);
+int fv_hasher_scale_rows(fv_hasher *h, const float *divisors /* hid */);
+/* Current resident matrix, K x N row-major. */
+int fv_hasher_get_weights(fv_hasher *h, float *out_W);
+
+/* flyvec/core.py:153-158 get_sparse_embedding for n token ids at once: activation = column
+ * V + id; thr = fl32(a[k-1] + a[k]) / 2 over the descending order statistics; code = act > thr.
+ * out_codes is n x hid int8. Requires 0 < k < hid (the reference raises IndexError otherwise). */
+int fv_hash_targets(fv_hasher *h, const int32_t *ids, uint64_t n, uint32_t k, int8_t *out_codes);
+
+/* Windowed form: activation = fp32 sum, in window order, of the columns idx[r][0..w) (-1
+ * skipped), then the same threshold rule. Either output may be NULL: out_bits is
+ * n x ceil(hid/64) uint64 (neuron h -> word h>>6, bit h&63), out_codes is n x hid int8. */
+int fv_hash_windows(fv_hasher *h, const int32_t *idx, uint64_t n, uint32_t w, uint32_t k,
+                    uint64_t *out_bits, int8_t *out_codes);
+
+/* Same with idx and outputs already in HBM (fv_dev_alloc); asynchronous on the hasher's stream. */
+int fv_hash_windows_dev(fv_hasher *h, const int32_t *idx_dev, uint64_t n, uint32_t w, uint32_t k,
+                        uint64_t *out_bits_dev, int8_t *out_codes_dev);
+/* Waits for the stream; FV_ERR_DATA if any launched batch met a column index outside [-1, N). */
+int fv_hasher_sync(fv_hasher *h);
+/* Measurement: `reps` launches of fv_hash_windows_dev, mean kernel duration by HIP events. */
+int fv_hasher_time_windows(fv_hasher *h, const int32_t *idx_dev, uint64_t n, uint32_t w, uint32_t k,
+                           uint64_t *out_bits_dev, int8_t *out_codes_dev, uint32_t reps,
+                           float *out_mean_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLYVEC_HIP_H */

@@ -1,0 +1,313 @@
+/*
+ * CPU restatement of the FlyVec training minibatch step and its host set-up.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker the HIP library is
+ * compared against; nothing in the shipped package may link or call it.
+ * It follows the reference sources statement by statement (citations are
+ * path:line inside the reference tree) and keeps the reference's data layout
+ * (W is K x N row-major, N = 2V) and arithmetic (fp32 products, double
+ * accumulation of the window sums, one rounding to fp32; fp32 everywhere
+ * else).  Build with -ffp-contract=off so no multiply-add is fused.
+ *
+ * Pinned by (see tests/test_oracle_*.py):
+ *   fvo_count_windows / fvo_window_starts : the reference's own prune_input.cpp
+ *       compiled into oracle/_ref (bit-exact on random and edge-case offsets).
+ *   fvo_inverse_frequency, fvo_inflate, fvo_activations, fvo_argmax_*,
+ *   fvo_train_step : closed forms (one-window batch, W = 0 fixed point,
+ *       invariance to a global rescale of 1/frequency by a power of two,
+ *       max|dW| == eps), a from-scratch brute force in Python floats on tiny
+ *       shapes, and numpy restatements of each stage.
+ *
+ * Order-dependent fp32 sums (the reference uses atomics whose order is not
+ * defined) are realised here in increasing window order, then increasing
+ * position inside the window.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define FVO_MAXLEN 214 /* flyvec/src/prune_input.cpp:7 */
+
+int fvo_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* flyvec/src/prune_input.cpp:64-84 (getnum_samples) */
+uint64_t fvo_count_windows(const uint64_t *offsets, uint64_t n_chunks, uint64_t w) {
+  uint64_t total = 0;
+  for (uint64_t s = 0; s < n_chunks; ++s) {
+    uint64_t len = offsets[s + 1] - offsets[s];
+    if (len >= w && len < FVO_MAXLEN) total += len - w + 1;
+  }
+  return total;
+}
+
+/* flyvec/src/prune_input.cpp:88-122 (compute_offset_phrases): the start of a
+ * window is the running sum of ALL previous chunk lengths plus the position
+ * inside the chunk; offsets[s] itself is never used as a position. */
+void fvo_window_starts(const uint64_t *offsets, uint64_t n_chunks, uint64_t w, uint64_t *starts) {
+  uint64_t running = 0, cnt = 0;
+  for (uint64_t s = 0; s < n_chunks; ++s) {
+    uint64_t len = offsets[s + 1] - offsets[s];
+    if (len >= w && len < FVO_MAXLEN)
+      for (uint64_t i = 0; i < len - w + 1; ++i) starts[cnt++] = running + i;
+    running += len;
+  }
+}
+
+/* flyvec/src/model_arrays.cu:396-424: counts are accumulated IN FP32 (they stop
+ * growing at 2^24), negative ids are ignored, 1/count is formed in double and
+ * rounded once, absent ids get 0. */
+void fvo_inverse_frequency(const int32_t *corpus, uint64_t n_tok, uint64_t V, float *invf) {
+  for (uint64_t i = 0; i < V; ++i) invf[i] = 0.0f;
+  for (uint64_t i = 0; i < n_tok; ++i)
+    if (corpus[i] >= 0) invf[corpus[i]] = (float)((double)invf[corpus[i]] + 1.0);
+  for (uint64_t i = 0; i < V; ++i)
+    invf[i] = (invf[i] != 0) ? (float)(1.0 / (double)invf[i]) : 0.0f;
+}
+
+/* flyvec/src/cuda_funcs.cu:915-936 (inflate_from_M_kernel_4): window r of the
+ * minibatch is the corpus slice at starts[perm[first + r]]; the centre column
+ * (c == w/2) is shifted into the target block, masked ids (-1) stay -1. */
+void fvo_inflate(const int32_t *corpus, const uint64_t *starts, const uint64_t *perm,
+                 uint64_t first, uint64_t n, int w, uint64_t V, int32_t *idx) {
+  const int mid = w / 2;
+  for (uint64_t r = 0; r < n; ++r) {
+    const int32_t *src = corpus + starts[perm[first + r]];
+    for (int c = 0; c < w; ++c) {
+      int32_t val = src[c];
+      idx[r * (uint64_t)w + c] = (val == -1) ? -1 : (c == mid ? (int32_t)(val + (int64_t)V) : val);
+    }
+  }
+}
+
+/* flyvec/src/cuda_funcs.cu:248-263 (raw) and :289-305 (scaled by 1/frequency):
+ * per window and neuron a double accumulator over the window positions in
+ * order, skipping -1; the scaled product is formed in fp32 first. */
+void fvo_activations(const float *W, int K, uint64_t N, const int32_t *idx, uint64_t n, int w,
+                     const float *invf, uint64_t V, float *raw, float *scaled) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < (int64_t)n; ++r) {
+    const int32_t *ix = idx + (uint64_t)r * w;
+    for (int h = 0; h < K; ++h) {
+      const float *row = W + (uint64_t)h * N;
+      double sr = 0.0, ss = 0.0;
+      for (int c = 0; c < w; ++c) {
+        int32_t i = ix[c];
+        if (i != -1) {
+          float f = invf[(uint64_t)i % V];
+          float prod = row[i] * f; /* fp32 product, cuda_funcs.cu:298-299 */
+          ss += (double)prod;
+          sr += (double)row[i];
+        }
+      }
+      if (raw) raw[(uint64_t)r * K + h] = (float)sr;
+      if (scaled) scaled[(uint64_t)r * K + h] = (float)ss;
+    }
+  }
+}
+
+/* flyvec/src/cuda_funcs.cu:488-561 (get_max_and_m_max_kernel_2, first pass):
+ * a literal simulation of the 64 threads: each scans its stride-64 class
+ * keeping strictly greater values, seeded with (data[0], 0); a shuffle-down
+ * tree inside each 32-lane warp keeps the lower lane on ties; warp 1 replaces
+ * warp 0 only when strictly greater. */
+int fvo_argmax_reference(const float *data, int K) {
+  float val[64];
+  int ind[64];
+  for (int t = 0; t < 64; ++t) {
+    float best = data[0];
+    int bi = 0;
+    for (int i = t; i < K; i += 64)
+      if (data[i] > best) { best = data[i]; bi = i; }
+    val[t] = best;
+    ind[t] = bi;
+  }
+  for (int wp = 0; wp < 2; ++wp) {
+    float *v = val + 32 * wp;
+    int *x = ind + 32 * wp;
+    for (int d = 16; d >= 1; d /= 2) {
+      float nv[32];
+      int nx[32];
+      for (int l = 0; l < 32; ++l) {
+        /* __shfl_down_sync returns the caller's own value past the warp end */
+        float ov = (l + d < 32) ? v[l + d] : v[l];
+        int ox = (l + d < 32) ? x[l + d] : x[l];
+        if (ov > v[l]) { nv[l] = ov; nx[l] = ox; } else { nv[l] = v[l]; nx[l] = x[l]; }
+      }
+      memcpy(v, nv, sizeof nv);
+      memcpy(x, nx, sizeof nx);
+    }
+  }
+  float best = val[0];
+  int bi = ind[0];
+  if (val[32] > best) { best = val[32]; bi = ind[32]; }
+  return bi;
+}
+
+/* Plain argmax, lowest index on ties. */
+int fvo_argmax_lowest(const float *data, int K) {
+  int bi = 0;
+  for (int i = 1; i < K; ++i)
+    if (data[i] > data[bi]) bi = i;
+  return bi;
+}
+
+/* flyvec/src/cuda_funcs.cu:1229 */
+float fvo_epoch_eps(float lr0, uint64_t epoch, uint64_t n_epochs) {
+  return (float)(lr0 * (1.0 - ((float)epoch) / ((float)n_epochs)));
+}
+
+/*
+ * One minibatch step on already inflated indices (idx is n x w).
+ * Order follows flyvec/src/cuda_funcs.cu:1662-1803 for sparse_input = 1,
+ * frequency_scaling = 1, Lmid = Lbase = 1, delta = 0, p = 2:
+ *   :1688        ds <- W                      (cuda_func1_odd, p-1 = 1: a copy)
+ *   :1700-1701   scaled and raw activations   (from that copy, i.e. from W)
+ *   :1715        xx <- 0
+ *   :1719        winner = argmax of RAW
+ *   :1721        xx[winner] += SCALED[r][winner]              (:722-744)
+ *   :1722        ds[h][:] = xx[h] != 0 ? -xx[h]*W[h][:] : 0   (:394-406)
+ *   :1732        ds[winner][idx] += invf[idx % V]             (:657-672)
+ *   :1792        rows with xx == 0 zero-filled; nc = max|ds|  (cu_special_reduction.cu:26-99)
+ *   :1797-1799   s = eps / max(prec, nc)
+ *   :1803        rows with xx != 0: v = s*ds; |v| > 1e-10 ? W += v   (cu_special_reduction.cu:316-354)
+ * tie_rule: 0 = lowest index, 1 = the reference's lane-tree order.
+ * Outputs (any may be NULL): winners[n], sc_at_winner[n], xx[K], *nc_out.
+ * ds_scratch must hold K*N floats.
+ */
+void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx, uint64_t n, int w,
+                    const float *invf, float eps, float prec, int tie_rule, float *ds_scratch,
+                    int32_t *winners, float *sc_at_winner, float *xx_out, float *nc_out) {
+  int32_t *win = (int32_t *)malloc(sizeof(int32_t) * (n ? n : 1));
+  float *scw = (float *)malloc(sizeof(float) * (n ? n : 1));
+  float *xx = (float *)calloc((size_t)K, sizeof(float));
+  float *ds = ds_scratch;
+
+#pragma omp parallel
+  {
+    float *raw = (float *)malloc(sizeof(float) * (size_t)K);
+#pragma omp for schedule(static)
+    for (int64_t r = 0; r < (int64_t)n; ++r) {
+      const int32_t *ix = idx + (uint64_t)r * w;
+      for (int h = 0; h < K; ++h) {
+        const float *row = W + (uint64_t)h * N;
+        double sr = 0.0;
+        for (int c = 0; c < w; ++c)
+          if (ix[c] != -1) sr += (double)row[ix[c]];
+        raw[h] = (float)sr;
+      }
+      int best = tie_rule ? fvo_argmax_reference(raw, K) : fvo_argmax_lowest(raw, K);
+      const float *row = W + (uint64_t)best * N;
+      double ss = 0.0;
+      for (int c = 0; c < w; ++c)
+        if (ix[c] != -1) {
+          float prod = row[ix[c]] * invf[(uint64_t)ix[c] % V];
+          ss += (double)prod;
+        }
+      win[r] = best;
+      scw[r] = (float)ss;
+    }
+    free(raw);
+  }
+
+  /* xx: fp32 adds in increasing window order */
+  for (uint64_t r = 0; r < n; ++r) xx[win[r]] = xx[win[r]] + scw[r];
+
+  /* ds = -xx*W or 0 */
+#pragma omp parallel for schedule(static)
+  for (int h = 0; h < K; ++h) {
+    float *d = ds + (uint64_t)h * N;
+    const float *row = W + (uint64_t)h * N;
+    if (xx[h] != 0) {
+      float nx = -xx[h];
+      for (uint64_t c = 0; c < N; ++c) d[c] = nx * row[c];
+    } else {
+      for (uint64_t c = 0; c < N; ++c) d[c] = 0.0f;
+    }
+  }
+
+  /* sparse Hebbian term, increasing (window, position) order */
+  for (uint64_t r = 0; r < n; ++r) {
+    float *d = ds + (uint64_t)win[r] * N;
+    const int32_t *ix = idx + r * (uint64_t)w;
+    for (int c = 0; c < w; ++c)
+      if (ix[c] != -1) d[ix[c]] = d[ix[c]] + invf[(uint64_t)ix[c] % V];
+  }
+
+  /* rows with xx == 0 are zero-filled (drops their sparse term); nc = max|ds| */
+  float nc = 0.0f;
+#pragma omp parallel for schedule(static) reduction(max : nc)
+  for (int h = 0; h < K; ++h) {
+    float *d = ds + (uint64_t)h * N;
+    if (xx[h] != 0) {
+      float m = 0.0f;
+      for (uint64_t c = 0; c < N; ++c) {
+        float a = fabsf(d[c]);
+        m = a > m ? a : m;
+      }
+      nc = m > nc ? m : nc;
+    } else {
+      for (uint64_t c = 0; c < N; ++c) d[c] = 0.0f;
+    }
+  }
+
+  float s = (prec > nc) ? eps / prec : eps / nc;
+
+#pragma omp parallel for schedule(static)
+  for (int h = 0; h < K; ++h) {
+    if (xx[h] == 0) continue;
+    float *row = W + (uint64_t)h * N;
+    const float *d = ds + (uint64_t)h * N;
+    for (uint64_t c = 0; c < N; ++c) {
+      float v = s * d[c];
+      if (fabs((double)v) > 1.e-10) row[c] = row[c] + v;
+    }
+  }
+
+  if (winners) memcpy(winners, win, sizeof(int32_t) * n);
+  if (sc_at_winner) memcpy(sc_at_winner, scw, sizeof(float) * n);
+  if (xx_out) memcpy(xx_out, xx, sizeof(float) * (size_t)K);
+  if (nc_out) *nc_out = nc;
+  free(win);
+  free(scw);
+  free(xx);
+}
+
+/*
+ * n_steps consecutive minibatches of one epoch, as the loop at
+ * flyvec/src/cuda_funcs.cu:1662 walks them: step j takes windows
+ * perm[first + j*B .. first + (j+1)*B), the last one only its remainder
+ * (the reference re-uses stale rows there; this restatement processes the
+ * remainder only).  winners (if given) receives the winners of every step
+ * back to back.  Returns the number of windows processed.
+ */
+uint64_t fvo_train_steps(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
+                         const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
+                         uint64_t n_steps, int w, const float *invf, float eps, float prec,
+                         int tie_rule, int32_t *winners) {
+  const uint64_t N = 2 * V;
+  float *ds = (float *)malloc(sizeof(float) * (size_t)K * N);
+  int32_t *idx = (int32_t *)malloc(sizeof(int32_t) * B * (uint64_t)w);
+  uint64_t done = 0;
+  for (uint64_t j = 0; j < n_steps; ++j) {
+    uint64_t k0 = first + j * B;
+    if (k0 >= n_windows) break;
+    uint64_t n = (k0 + B <= n_windows) ? B : n_windows - k0;
+    fvo_inflate(corpus, starts, perm, k0, n, w, V, idx);
+    fvo_train_step(W, K, N, V, idx, n, w, invf, eps, prec, tie_rule, ds,
+                   winners ? winners + done : NULL, NULL, NULL, NULL);
+    done += n;
+  }
+  free(ds);
+  free(idx);
+  return done;
+}
