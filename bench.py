@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Benchmark of the FlyVec hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one training minibatch (sampler -> gather-sum -> winner -> xx -> max|ds| -> update)
+at the headline configuration: K = 400 neurons, V = 20000, w = 11, B = 10000 windows, on a
+synthetic 10 M-token Zipf(1.07) corpus with geometric chunk lengths, fp32, everything resident in
+HBM before the timed region.  One JSON line is printed:
+
+  value              training windows / s over the K timed steps
+  roofline           the dominant kernel of the step against the 8 TB/s HBM peak: achieved =
+                     algorithmic bytes of that kernel per launch / its mean duration, measured with
+                     HIP events on the trainer's stream
+  step_roofline_frac (algorithmic bytes of the whole step / 8 TB/s) / measured time per step
+  cpu_baseline       the CPU restatement of the same step (oracle/, C + OpenMP) timed on this host
+  hash               the batched top-k hash (1,048,576 windows, k = 32, bit-packed) the same way,
+                     with the reference's numpy per-word path as its CPU baseline
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # B/s, MI355X
+
+TRAIN = dict(K=400, V=20000, w=11, B=10000, n_tokens=10_000_000, lr0=2e-4, n_epochs=15, prec=1e-30)
+HASH = dict(K=400, V=20000, w=11, k=32, n=1 << 20)
+
+
+def train_bytes(K, N, w, B):
+    """Algorithmic HBM bytes per step and per kernel: every window gathers w rows of K floats once;
+    W is read once for max|ds| and read + written once by the update; ds is never stored; token
+    ids, 1/f lookups and the sparse count updates are 16 bytes per window position."""
+    per = {
+        "gather_winner": 4 * B * w * K,
+        "neuron_owners": 8 * B + 8 * B * w,
+        "absmax_ds": 4 * K * N,
+        "update": 8 * K * N,
+        "slot_update": 8 * B * w,
+    }
+    return 4 * B * w * K + 12 * K * N + 16 * B * w, per
+
+
+def hash_bytes_per_window(K, w):
+    return 4 * w * K + 4 * w + 8 * ((K + 63) // 64)
+
+
+def bench_train(steps, warmup, cpu_seconds):
+    from flyvec_amd import Trainer, synthetic
+    c = TRAIN
+    tokens, offsets = synthetic.corpus(c["n_tokens"], c["V"])
+    W0 = synthetic.synapses(c["K"], c["V"], seed=5)
+    t = Trainer(c["V"], c["K"], c["w"], c["B"], initial_learning_rate=c["lr0"], prec=c["prec"])
+    t.set_corpus(tokens, offsets)
+    nwin = t.num_windows
+    perm = np.random.default_rng(6).permutation(nwin).astype(np.uint64)
+    t.set_permutation(perm)
+    t.set_weights(W0)
+    eps = t.epoch_eps(0, c["n_epochs"])
+    need = (warmup + 2 * steps) * c["B"]
+    if need > nwin:
+        raise SystemExit(f"{warmup}+2x{steps} steps need {need} windows, the corpus has {nwin}")
+
+    for s in range(warmup):
+        t.step(s * c["B"], c["B"], eps)
+    t.sync()
+    # timed region: exactly `steps` steps, device idle before and after
+    t0 = time.perf_counter()
+    for s in range(steps):
+        t.step((warmup + s) * c["B"], c["B"], eps)
+    t.sync()
+    wall = time.perf_counter() - t0
+    # per-kernel durations (HIP events between the kernels) on the following `steps` steps
+    total_ms, kern_ms = t.time_steps((warmup + steps) * c["B"], steps, eps)
+    ev_ms_per_step = total_ms / steps
+    t.close()
+
+    N = 2 * c["V"]
+    step_bytes, per_kernel = train_bytes(c["K"], N, c["w"], c["B"])
+    dom = max(kern_ms, key=kern_ms.get)
+    achieved = per_kernel[dom] / (kern_ms[dom] * 1e-3)
+    ms_per_step = wall / steps * 1e3
+    out = {
+        "value": steps * c["B"] / wall,
+        "ms_per_step": ms_per_step,
+        "event_ms_per_step": ev_ms_per_step,
+        "kernel_ms": kern_ms,
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": None,
+                     "algorithmic_bytes": per_kernel[dom]},
+        "step_roofline_frac": (step_bytes / HBM_PEAK) / (ms_per_step * 1e-3),
+        "step_algorithmic_bytes": step_bytes,
+        "n_windows": nwin,
+    }
+
+    if cpu_seconds > 0:
+        from oracle import train_oracle as to
+        starts = to.window_starts(offsets, c["w"])
+        invf = to.inverse_frequency(tokens, c["V"])
+        Wc = W0.copy()
+        to.train_steps(Wc, tokens, starts, perm, 0, c["B"], 2, c["w"], invf, eps, c["prec"])  # warm caches
+        done, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < cpu_seconds and (done + 8) * c["B"] <= nwin:
+            to.train_steps(Wc, tokens, starts, perm, done * c["B"], c["B"], 8, c["w"], invf, eps, c["prec"])
+            done += 8
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": done * c["B"] / dt, "unit": "windows/s", "cores": to.num_threads(),
+                               "kind": "port",
+                               "sample": f"{done} steps of the same workload (B={c['B']}) by the C/OpenMP "
+                                         f"restatement of the reference step, {dt:.1f} s"}
+    return out
+
+
+def bench_hash(reps, cpu_seconds):
+    from flyvec_amd import Hasher, synthetic
+    from flyvec_amd._lib import DeviceBuffer
+    c = HASH
+    W = synthetic.synapses(c["K"], c["V"], seed=1)
+    idx = synthetic.window_indices(c["n"], c["w"], c["V"], seed=7)
+    h = Hasher(W)
+    d_idx = DeviceBuffer.from_numpy(idx)
+    d_bits = DeviceBuffer(c["n"] * h.words * 8)
+    h.time_windows(d_idx, c["n"], c["w"], c["k"], bits_buf=d_bits, reps=2)  # warm-up
+    ms = h.time_windows(d_idx, c["n"], c["w"], c["k"], bits_buf=d_bits, reps=reps)
+    h.sync()
+    bpw = hash_bytes_per_window(c["K"], c["w"])
+    achieved = bpw * c["n"] / (ms * 1e-3)
+    out = {"metric": "hash codes/s", "value": c["n"] / (ms * 1e-3), "unit": "codes/s", "ms_per_batch": ms,
+           "config": {"workload": f"batched contextual hash: K={c['K']} V={c['V']} w={c['w']} k={c['k']} "
+                                  f"n={c['n']} windows, 7 uint64 words out"},
+           "dtype": "f32",
+           "roofline": {"bound": "hbm", "kernel": "hash", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
+                        "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": None,
+                        "algorithmic_bytes": bpw * c["n"]}}
+    if cpu_seconds > 0:
+        from oracle import hash_oracle as ho
+        ids = synthetic.zipf_ids(4096, c["V"], seed=2)
+        n_done, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < cpu_seconds:
+            ho.hash_targets_loop(W, ids, 50)
+            n_done += len(ids)
+        dt = time.perf_counter() - t0
+        sample = idx[:32768]
+        t1 = time.perf_counter()
+        ho.hash_windows(W, sample, c["k"])
+        dtw = time.perf_counter() - t1
+        out["cpu_baseline"] = {"value": n_done / dt, "unit": "codes/s", "cores": 1, "kind": "port",
+                               "sample": f"numpy per-word path (argsort, k=50) on 4096 Zipf target ids, "
+                                         f"repeated for {dt:.1f} s",
+                               "windows_vectorised_numpy": {"value": len(sample) / dtw, "unit": "codes/s",
+                                                            "sample": f"{len(sample)} windows of the same batch"}}
+    h.close()
+    d_idx.free()
+    d_bits.free()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample length (0 = skip)")
+    ap.add_argument("--no-hash", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    from flyvec_amd import _lib
+    info = _lib.device_info()
+    tr = bench_train(args.steps, args.warmup, args.cpu_seconds)
+    c = TRAIN
+    line = {
+        "metric": "train windows/s at K=400,Nvoc=20k",
+        "value": tr["value"], "unit": "windows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": tr["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"single training minibatch step: K={c['K']} Nvoc={c['V']} w={c['w']} B={c['B']}, "
+                               f"{c['n_tokens']} Zipf(1.07) tokens, geometric chunks (mean 25), "
+                               f"{tr['n_windows']} windows, lr 2e-4, fp32"},
+        "device": info["name"].strip(),
+        "roofline": tr["roofline"],
+        "step_roofline_frac": tr["step_roofline_frac"],
+        "step_algorithmic_bytes": tr["step_algorithmic_bytes"],
+        "event_ms_per_step": tr["event_ms_per_step"],
+        "kernel_ms": tr["kernel_ms"],
+    }
+    if "cpu_baseline" in tr:
+        line["cpu_baseline"] = tr["cpu_baseline"]
+    if not args.no_hash:
+        line["hash"] = bench_hash(reps=10, cpu_seconds=min(args.cpu_seconds, 5.0))
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

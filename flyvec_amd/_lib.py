@@ -8,11 +8,14 @@ from pathlib import Path
 
 import numpy as np
 
-LIB_PATH = Path(__file__).resolve().parent / "lib" / "libflyvec_hip.so"
+import os
+
+# FLYVEC_HIP_LIB points at another build of the same library (e.g. one compiled with extra flags).
+LIB_PATH = Path(os.environ.get("FLYVEC_HIP_LIB") or Path(__file__).resolve().parent / "lib" / "libflyvec_hip.so")
 
 FV_OK, FV_ERR_INVALID, FV_ERR_HIP, FV_ERR_STATE, FV_ERR_DATA = range(5)
-FV_TRAIN_KERNELS = 4
-TRAIN_KERNEL_NAMES = ("gather_winner", "xx_totals", "absmax_ds", "update")
+FV_TRAIN_KERNELS = 5
+TRAIN_KERNEL_NAMES = ("gather_winner", "neuron_owners", "absmax_ds", "update", "slot_update")
 
 
 class FlyvecError(RuntimeError):

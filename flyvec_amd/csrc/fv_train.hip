@@ -2,34 +2,48 @@
 //
 // Replaces the kernel chain of flyvec/src/cuda_funcs.cu:1662-1803 (sparse input, frequency
 // scaling, Lmid = Lbase = 1, delta = 0, p = 2).  The reference materialises ds (K x N) and
-// walks it five times per step; here ds is never stored:
+// walks it five times per step; here ds is never stored and nothing uses global atomics:
 //
 //   1. gather+winner   one wavefront per window: sampler (cuda_funcs.cu:915-936), raw
 //                      activation = sum of ~w token rows of the token-major matrix with the K
 //                      neurons spread over lanes (:248-263, double accumulators, one rounding),
-//                      argmax by a wave reduction (:488-561), the winner's frequency-scaled
-//                      activation (:289-305, needed only at the winner, :731), and the sparse
-//                      Hebbian term recorded as integer counts per (winner, token) plus one
-//                      flag bit per 4 matrix elements (:657-672).
-//   2. xx totals       xx[h] = sum of the scaled activations of the windows h won, added in
-//                      window order (:722-744; the reference's atomic order is undefined, this
-//                      one is fixed so a step is reproducible bit for bit).
-//   3. max|ds|         ds = -xx[h] * W + count * (1/f) re-derived on the fly from W, xx and the
-//                      flagged counts; grid-wide maximum of |ds| (:394-406,
-//                      cu_special_reduction.cu:26-99, 153-189).
+//                      argmax by a wave reduction (:488-561) and the winner's frequency-scaled
+//                      activation (:289-305; it is only ever read at the winner, :731).
+//   2. neuron owners   one block per neuron h: the ordered list of windows h won; xx[h] = sum of
+//                      their scaled activations in window order (:722-744 -- the reference's
+//                      atomic order is undefined, this one is fixed, so a step is reproducible
+//                      bit for bit); then the sparse Hebbian term of row h (:657-672): the block
+//                      alone owns elements (h, token), so it counts repeated tokens in LDS, and
+//                      for each distinct token saves the true weight and the count in a slot
+//                      record, evaluates ds there, and plants a sentinel in W.
+//   3. max|ds|         dense pass: ds = -xx[h] * W (:394-406), sentinel elements skipped; block
+//                      maxima (cu_special_reduction.cu:26-99, 153-189).
 //   4. update          W += s * ds where |s * ds| > 1e-10, s = eps / max(prec, max|ds|), rows
 //                      with xx == 0 untouched (cuda_funcs.cu:1797-1799,
-//                      cu_special_reduction.cu:316-354); clears the counts and flags it consumed.
+//                      cu_special_reduction.cu:316-354); dense blocks leave sentinels alone,
+//                      slot blocks of the same launch write the final value over each sentinel.
 //
-// Because every one of the n additions of 1/f onto ds[h][i] adds the same value, the
-// reference's result for that element depends only on n; replaying n sequential fp32 adds
-// reproduces it exactly whatever order its atomics ran in.
+// Every one of the n additions of 1/f onto ds[h][i] adds the same value, so the reference's
+// result for that element depends only on n; replaying n sequential fp32 adds reproduces it
+// exactly whatever order its atomics ran in.
 #include <math.h>
 #include <string.h>
 
 #include <vector>
 
 #include "fv_internal.h"
+#include "fv_repeat_add.h"
+
+// Written over W[p] while the true weight of a sparse element waits in its slot record. A quiet
+// NaN with a payload no arithmetic produces.
+#define FV_SENTINEL 0x7fc5ca1eu
+#define FV_SLOT_INVALID 0xffffffffu
+
+struct fv_slot {
+  uint32_t p;  // element index i * ldk + h, or FV_SLOT_INVALID
+  uint32_t n;  // pending additions of 1/f
+  float wv;    // the weight the sentinel replaced
+};
 
 struct fv_trainer {
   fv_train_config cfg;
@@ -38,17 +52,21 @@ struct fv_trainer {
   uint32_t total4;  // N * ldk / 4 (float4 elements of the matrix)
   hipStream_t stream;
   float *Wt;
-  uint32_t *cnt;    // per matrix element: additions of 1/f pending for the current step
-  uint32_t *flags;  // bit g set <=> some cnt in float4 group g is non-zero
   int32_t *corpus;
   uint64_t n_tokens;
   uint64_t *starts, *perm;
   uint64_t n_windows;
   float *invf;
-  int32_t *win;
-  float *sc;
-  float *xx;
-  uint32_t *scalars;  // [0] bits of max|ds| of the current step
+  int32_t *idx;     // B x w column indices of the current minibatch
+  int32_t *win;     // B winners
+  float *sc;        // B scaled activations at the winner
+  uint32_t *order;  // B window ids grouped by winner, ascending inside a group
+  uint32_t nb_chunk;  // column counters per LDS pass of the neuron kernel
+  fv_slot *slots;   // B x w slot records
+  float *xx;        // ldk
+  float *emax;      // K: max|ds| over the sparse elements of each neuron
+  float *bmax;      // dense_blocks: max|ds| of each dense block
+  float *scalars;   // [0] max|ds| of the last step
   uint32_t last_n;
   uint64_t shuffle_calls;
   bool have_corpus, have_weights;
@@ -56,7 +74,7 @@ struct fv_trainer {
   float update_cut;  // largest fp32 <= 1e-10
 };
 
-// ---- kernel 1: sampler + gather-sum + winner + sparse counts ---------------------------------
+// ---- kernel 1: sampler + gather-sum + winner ----------------------------------------------------
 
 struct fv_gather_args {
   const float *Wt;
@@ -64,11 +82,9 @@ struct fv_gather_args {
   const uint64_t *starts;
   const uint64_t *perm;
   const float *invf;
-  uint32_t *cnt;
-  uint32_t *flags;
+  int32_t *idx;
   int32_t *win;
   float *sc;
-  uint32_t *scalars;
   uint64_t first;
   uint32_t n, K, ldk, w, V, tie_rule;
 };
@@ -109,7 +125,6 @@ template <int NV>
 __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a) {
   const int lane = threadIdx.x & 63;
   const uint32_t r = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (blockIdx.x == 0 && threadIdx.x == 0) a.scalars[0] = 0;  // max|ds| of this step starts at 0
   if (r >= a.n) return;
 
   // sampler: lane c holds column index c of the window (flyvec/src/cuda_funcs.cu:915-936)
@@ -118,6 +133,7 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
     const uint64_t s = a.starts[a.perm[a.first + r]];
     const int32_t tok = a.corpus[s + lane];
     idx = tok < 0 ? -1 : (lane == (int)(a.w / 2) ? tok + (int32_t)a.V : tok);
+    a.idx[(uint64_t)r * a.w + lane] = idx;
   }
 
   double acc[NV];
@@ -151,12 +167,9 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
   }
 
   // frequency-scaled activation of the winner: fp32 products, double sum in window order
-  const bool ok = (uint32_t)idx < 2 * a.V;
   double pd = 0.0;
-  uint64_t p = 0;
-  if (ok) {
-    p = (uint64_t)idx * a.ldk + hstar;
-    const float wv = a.Wt[p];
+  if ((uint32_t)idx < 2 * a.V) {
+    const float wv = a.Wt[(uint64_t)idx * a.ldk + hstar];
     const float f = a.invf[(uint32_t)idx >= a.V ? (uint32_t)idx - a.V : (uint32_t)idx];
     pd = (double)__fmul_rn(wv, f);
   }
@@ -171,75 +184,31 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
     a.win[r] = (int32_t)hstar;
     a.sc[r] = (float)s;
   }
-
-  // sparse Hebbian term: one more pending addition of 1/f at (winner, token)
-  if (ok) {
-    atomicAdd(&a.cnt[p], 1u);
-    atomicOr(&a.flags[p >> 7], 1u << ((p >> 2) & 31));
-  }
 }
 
-// ---- kernel 2: xx[h] = sum over the windows h won, in window order ------------------------------
+// ---- kernel 2: one block per neuron -- its windows, xx, and its sparse elements --------------------
 
-__global__ __launch_bounds__(256) void fv_xx_totals_kernel(const int32_t *__restrict__ win,
-                                                           const float *__restrict__ sc, uint32_t n,
-                                                           uint32_t K, uint32_t ldk,
-                                                           float *__restrict__ xx) {
-  const int lane = threadIdx.x & 63;
-  const uint32_t h = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (h >= ldk) return;
-  float acc = 0.0f;
-  if (h < K) {
-    for (uint32_t base = 0; base < n; base += 64) {
-      const uint32_t r = base + lane;
-      const int32_t wv = r < n ? win[r] : -1;
-      uint64_t m = __ballot(wv == (int32_t)h);
-      if (m) {
-        const float sv = r < n ? sc[r] : 0.0f;
-        while (m) {
-          const int l = __ffsll((long long)m) - 1;
-          acc = __fadd_rn(acc, __uint_as_float(fv_readlane(__float_as_uint(sv), l)));
-          m &= m - 1;
-        }
-      }
-    }
-  }
-  if (lane == 0) xx[h] = acc;
-}
+#define FV_NB_THREADS 1024
+#define FV_NB_WAVES (FV_NB_THREADS / 64)
+#define FV_NB_MAX_CHUNK 32768  // column counters per LDS pass (128 KB of the CU's 160 KB)
+#define FV_NB_SC_CACHE 2048
 
-// ---- kernels 3 and 4: dense passes over the matrix ------------------------------------------------
-
-struct fv_dense_args {
-  float4 *Wt4;
-  uint4 *cnt4;
-  uint64_t *flags64;
-  const float *xx;
+struct fv_neuron_args {
+  const int32_t *win;
+  const float *sc;
+  const int32_t *idx;
   const float *invf;
-  uint32_t *scalars;
-  uint32_t total4, ldk4, V;
-  float eps, prec, update_cut;
+  float *Wt;
+  float *xx;
+  float *emax;
+  uint32_t *order;
+  fv_slot *slots;
+  uint32_t n, K, ldk, w, V, chunk;
 };
 
-// ds for the 4 consecutive neurons of one token held by this lane.
-__device__ __forceinline__ float4 fv_ds_value(const float4 w, const float4 x, bool flagged,
-                                              const uint4 *__restrict__ cnt4, uint32_t p4,
-                                              uint32_t ldk4, const float *__restrict__ invf,
-                                              uint32_t V) {
-  float4 v;
-  v.x = x.x != 0.0f ? __fmul_rn(-x.x, w.x) : 0.0f;
-  v.y = x.y != 0.0f ? __fmul_rn(-x.y, w.y) : 0.0f;
-  v.z = x.z != 0.0f ? __fmul_rn(-x.z, w.z) : 0.0f;
-  v.w = x.w != 0.0f ? __fmul_rn(-x.w, w.w) : 0.0f;
-  if (flagged) {
-    const uint4 n = cnt4[p4];
-    const uint32_t i = p4 / ldk4;  // token row; the target block repeats the frequencies
-    const float f = invf[i >= V ? i - V : i];
-    if (x.x != 0.0f) for (uint32_t t = 0; t < n.x; ++t) v.x = __fadd_rn(v.x, f);
-    if (x.y != 0.0f) for (uint32_t t = 0; t < n.y; ++t) v.y = __fadd_rn(v.y, f);
-    if (x.z != 0.0f) for (uint32_t t = 0; t < n.z; ++t) v.z = __fadd_rn(v.z, f);
-    if (x.w != 0.0f) for (uint32_t t = 0; t < n.w; ++t) v.w = __fadd_rn(v.w, f);
-  }
-  return v;
+// ds of one sparse element: the dense term, then n sequential additions of 1/f.
+__device__ __forceinline__ float fv_sparse_ds(float xx, float wv, float f, uint32_t n) {
+  return fv_add_repeat(__fmul_rn(-xx, wv), f, n);
 }
 
 __device__ __forceinline__ float fv_absmax_keep(float m, float v) {
@@ -247,66 +216,274 @@ __device__ __forceinline__ float fv_absmax_keep(float m, float v) {
   return a > m ? a : m;  // a NaN never replaces m, as in the reference's comparison
 }
 
-template <bool UPDATE>
-__global__ __launch_bounds__(256) void fv_dense_kernel(fv_dense_args a) {
+// Exclusive prefix sum of one value per thread over the block, and the block total.
+__device__ __forceinline__ uint32_t fv_block_exclusive_scan(uint32_t v, uint32_t *wave_tot /*FV_NB_WAVES+1*/,
+                                                            uint32_t *total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t incl = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t o = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += o;
+  }
+  __syncthreads();
+  if (lane == 63) wave_tot[wave] = incl;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t run = 0;
+    for (int i = 0; i < FV_NB_WAVES; ++i) {
+      const uint32_t t = wave_tot[i];
+      wave_tot[i] = run;
+      run += t;
+    }
+    wave_tot[FV_NB_WAVES] = run;
+  }
+  __syncthreads();
+  *total = wave_tot[FV_NB_WAVES];
+  return wave_tot[wave] + incl - v;
+}
+
+__global__ __launch_bounds__(FV_NB_THREADS) void fv_neuron_kernel(fv_neuron_args a) {
+  extern __shared__ uint32_t cnt[];  // a.chunk counters, one per column index of the current pass
+  __shared__ float scbuf[FV_NB_SC_CACHE];
+  __shared__ uint32_t wave_tot[FV_NB_WAVES + 1];
+  __shared__ uint32_t sh_lt, sh_pos;
+  __shared__ float sh_xx, sh_wmax[FV_NB_WAVES];
+
+  const uint32_t h = blockIdx.x;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t n = a.n;
+  const int32_t *__restrict__ win = a.win;
+  const int32_t *__restrict__ idx = a.idx;
+
+  if (tid == 0) {
+    sh_lt = 0;
+    sh_pos = 0;
+  }
+  for (uint32_t i = tid; i < a.chunk / 4; i += FV_NB_THREADS) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+
+  // (1) windows won by lower neurons / by this one. Each thread takes a contiguous segment, so the
+  // per-thread match counts scan into window order; matches of the first 64 windows of a segment
+  // are remembered as a bit mask so the second walk needs no reload.
+  const uint32_t seg = (n + FV_NB_THREADS - 1) / FV_NB_THREADS;
+  const uint32_t r0 = min(tid * seg, n), r1 = min(r0 + seg, n);
+  uint32_t lt = 0, eq = 0;
+  uint64_t mask = 0;
+#pragma unroll 8
+  for (uint32_t r = r0; r < r1; ++r) {
+    const uint32_t wv = (uint32_t)win[r];
+    lt += wv < h;
+    const bool hit = wv == h;
+    eq += hit;
+    if (hit && r - r0 < 64) mask |= 1ull << (r - r0);
+  }
+  __syncthreads();
+  {
+    uint32_t wl = lt;  // wave-reduce before touching the shared counter
+    for (int d = 32; d >= 1; d >>= 1) wl += __shfl_down(wl, d, 64);
+    if ((tid & 63) == 0 && wl) atomicAdd(&sh_lt, wl);
+  }
+  uint32_t c_h;
+  const uint32_t my_off = fv_block_exclusive_scan(eq, wave_tot, &c_h);
+  const uint32_t base = sh_lt;  // start of this neuron's group in order[]
+  {
+    uint32_t pos = base + my_off;
+    while (mask) {
+      a.order[pos++] = r0 + (uint32_t)__ffsll((long long)mask) - 1;
+      mask &= mask - 1;
+    }
+    for (uint32_t r = r0 + 64; r < r1; ++r)
+      if ((uint32_t)win[r] == h) a.order[pos++] = r;
+  }
+  __syncthreads();  // order[base .. base + c_h) is now readable by the whole block
+  const uint32_t *__restrict__ order = a.order + base;
+
+  // (2) xx[h]: fp32 adds in window order
+  float xx = 0.0f;
+  for (uint32_t j0 = 0; j0 < c_h; j0 += FV_NB_SC_CACHE) {
+    const uint32_t m = min(c_h - j0, (uint32_t)FV_NB_SC_CACHE);
+    for (uint32_t j = tid; j < m; j += FV_NB_THREADS) scbuf[j] = a.sc[order[j0 + j]];
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll 8
+      for (uint32_t j = 0; j < m; ++j) xx = __fadd_rn(xx, scbuf[j]);
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    sh_xx = xx;
+    a.xx[h] = xx;
+  }
+  __syncthreads();
+  xx = sh_xx;
+
+  // (3) sparse elements of row h. The neuron's windows own the slot records [base*w, (base+c_h)*w).
+  const uint32_t m_ent = c_h * a.w;
+  fv_slot *slots = a.slots + (uint64_t)base * a.w;
+  float m = 0.0f;
+  uint32_t n_emitted = 0;
+  if (xx != 0.0f) {  // (the reference zero-fills ds of a row with xx == 0: no sparse term, no update)
+    const uint32_t n_cols = 2 * a.V;
+    for (uint32_t lo = 0; lo < n_cols; lo += a.chunk) {
+      // count the occurrences of every column index of this pass: one window per thread at a time
+      for (uint32_t j = tid; j < c_h; j += FV_NB_THREADS) {
+        const int32_t *row = idx + (uint64_t)order[j] * a.w;
+        for (uint32_t c = 0; c < a.w; ++c) {
+          const int32_t i = row[c];
+          const uint32_t k = (uint32_t)i - lo;
+          if ((uint32_t)i < n_cols && k < a.chunk) atomicAdd(&cnt[k], 1u);
+        }
+      }
+      __syncthreads();
+      // every non-zero counter is one distinct element (h, column): save its weight and count in
+      // a slot record, evaluate ds, plant the sentinel; reset the counter for the next pass
+      for (uint32_t k4 = tid; k4 < a.chunk / 4; k4 += FV_NB_THREADS) {
+        const uint4 c4 = ((const uint4 *)cnt)[k4];
+        if ((c4.x | c4.y | c4.z | c4.w) == 0) continue;
+        ((uint4 *)cnt)[k4] = make_uint4(0, 0, 0, 0);
+        const uint32_t cc[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (cc[q] == 0) continue;
+          const uint32_t i = lo + k4 * 4 + q;
+          fv_slot sl;
+          sl.p = i * a.ldk + h;
+          sl.n = cc[q];
+          sl.wv = a.Wt[sl.p];
+          const float f = a.invf[i >= a.V ? i - a.V : i];
+          m = fv_absmax_keep(m, fv_sparse_ds(xx, sl.wv, f, sl.n));
+          a.Wt[sl.p] = __uint_as_float(FV_SENTINEL);
+          slots[atomicAdd(&sh_pos, 1u)] = sl;
+        }
+      }
+      __syncthreads();
+    }
+    n_emitted = sh_pos;
+  }
+  for (uint32_t e = n_emitted + tid; e < m_ent; e += FV_NB_THREADS) slots[e].p = FV_SLOT_INVALID;
+  const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));  // m >= 0: bit order == value order
+  if ((tid & 63) == 0) sh_wmax[tid >> 6] = __uint_as_float(wm);
+  __syncthreads();
+  if (tid == 0) {
+    float bm = 0.0f;
+    for (int i = 0; i < FV_NB_WAVES; ++i) bm = fmaxf(bm, sh_wmax[i]);
+    a.emax[h] = bm;
+  }
+}
+
+// ---- kernels 3 and 4: dense passes over the matrix ------------------------------------------------
+
+struct fv_dense_args {
+  float4 *Wt4;
+  const float *xx;
+  const float *invf;
+  const fv_slot *slots;
+  const float *emax;
+  float *bmax;
+  float *scalars;
+  uint32_t total4, ldk4, ldk, V, K, n_slots, slot_blocks, n_bmax;
+  float eps, prec, update_cut;
+};
+
+__device__ __forceinline__ bool fv_is_sentinel(float w) { return __float_as_uint(w) == FV_SENTINEL; }
+
+__device__ __forceinline__ float fv_dense_ds(float x, float w) {
+  return (x != 0.0f && !fv_is_sentinel(w)) ? __fmul_rn(-x, w) : 0.0f;
+}
+
+// Block-wide maximum of non-negative floats; result valid in thread 0.
+__device__ __forceinline__ float fv_block_max_nonneg(float m, float *smem4) {
+  const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) smem4[threadIdx.x >> 6] = __uint_as_float(wm);
+  __syncthreads();
+  return fmaxf(fmaxf(smem4[0], smem4[1]), fmaxf(smem4[2], smem4[3]));
+}
+
+__global__ __launch_bounds__(256) void fv_absmax_kernel(fv_dense_args a) {
   extern __shared__ float4 xs4[];  // xx, ldk4 float4
+  __shared__ float smem4[4];
   for (uint32_t q = threadIdx.x; q < a.ldk4; q += 256) xs4[q] = ((const float4 *)a.xx)[q];
   __syncthreads();
-
-  float s = 0.0f;
-  if (UPDATE) {
-    const float nc = __uint_as_float(a.scalars[0]);
-    s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
-  }
-
-  const int lane = threadIdx.x & 63;
   const uint32_t stride = gridDim.x * 256;
   const uint32_t dq = stride % a.ldk4;
-  uint32_t p4 = blockIdx.x * 256 + threadIdx.x;
-  uint32_t q = p4 % a.ldk4;
+  uint32_t q = (blockIdx.x * 256 + threadIdx.x) % a.ldk4;
   float m = 0.0f;
-  // The loop bound is taken on the wave's first element so the whole wave iterates together.
-  for (uint32_t base = p4 - lane; base < a.total4; base += stride, p4 += stride) {
-    const uint64_t fw = a.flags64[__builtin_amdgcn_readfirstlane(base >> 6)];
-    if (p4 < a.total4) {
-      float4 w = a.Wt4[p4];
-      const float4 x = xs4[q];
-      const bool flagged = (fw >> lane) & 1;
-      const float4 v = fv_ds_value(w, x, flagged, a.cnt4, p4, a.ldk4, a.invf, a.V);
-      if (!UPDATE) {
-        m = fv_absmax_keep(m, v.x);
-        m = fv_absmax_keep(m, v.y);
-        m = fv_absmax_keep(m, v.z);
-        m = fv_absmax_keep(m, v.w);
-      } else {
-        bool changed = false;
-        float d;
-        d = __fmul_rn(s, v.x); if (fabsf(d) > a.update_cut) { w.x = __fadd_rn(w.x, d); changed = true; }
-        d = __fmul_rn(s, v.y); if (fabsf(d) > a.update_cut) { w.y = __fadd_rn(w.y, d); changed = true; }
-        d = __fmul_rn(s, v.z); if (fabsf(d) > a.update_cut) { w.z = __fadd_rn(w.z, d); changed = true; }
-        d = __fmul_rn(s, v.w); if (fabsf(d) > a.update_cut) { w.w = __fadd_rn(w.w, d); changed = true; }
-        if (changed) a.Wt4[p4] = w;
-        if (flagged) a.cnt4[p4] = make_uint4(0, 0, 0, 0);
-      }
-    }
-    if (UPDATE && fw != 0 && lane == 0) a.flags64[base >> 6] = 0;
+  for (uint32_t p4 = blockIdx.x * 256 + threadIdx.x; p4 < a.total4; p4 += stride) {
+    const float4 w = a.Wt4[p4];
+    const float4 x = xs4[q];
+    m = fv_absmax_keep(m, fv_dense_ds(x.x, w.x));
+    m = fv_absmax_keep(m, fv_dense_ds(x.y, w.y));
+    m = fv_absmax_keep(m, fv_dense_ds(x.z, w.z));
+    m = fv_absmax_keep(m, fv_dense_ds(x.w, w.w));
     q += dq;
     if (q >= a.ldk4) q -= a.ldk4;
   }
+  const float bm = fv_block_max_nonneg(m, smem4);
+  if (threadIdx.x == 0) a.bmax[blockIdx.x] = bm;
+}
 
-  if (!UPDATE) {
-    __shared__ uint32_t wave_max[4];
-    const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));  // m >= 0: bit order == value order
-    if (lane == 0) wave_max[threadIdx.x >> 6] = wm;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      uint32_t b = wave_max[0];
-      b = wave_max[1] > b ? wave_max[1] : b;
-      b = wave_max[2] > b ? wave_max[2] : b;
-      b = wave_max[3] > b ? wave_max[3] : b;
-      if (b) atomicMax(&a.scalars[0], b);
-    }
+__global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
+  extern __shared__ float4 xs4[];
+  __shared__ float smem4[4];
+  __shared__ float sh_s;
+  for (uint32_t q = threadIdx.x; q < a.ldk4; q += 256) xs4[q] = ((const float4 *)a.xx)[q];
+  // max|ds| = max over the dense block maxima and the per-neuron sparse maxima
+  float nc = 0.0f;
+  for (uint32_t i = threadIdx.x; i < a.n_bmax; i += 256) nc = fmaxf(nc, a.bmax[i]);
+  for (uint32_t i = threadIdx.x; i < a.K; i += 256) nc = fmaxf(nc, a.emax[i]);
+  nc = fv_block_max_nonneg(nc, smem4);
+  if (threadIdx.x == 0) {
+    sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
+    if (blockIdx.x == 0) a.scalars[0] = nc;
   }
+  __syncthreads();
+  const float s = sh_s;
+
+  const uint32_t bid = blockIdx.x;
+  const uint32_t stride = gridDim.x * 256;
+  const uint32_t dq = stride % a.ldk4;
+  uint32_t q = (bid * 256 + threadIdx.x) % a.ldk4;
+  for (uint32_t p4 = bid * 256 + threadIdx.x; p4 < a.total4; p4 += stride) {
+    float4 w = a.Wt4[p4];
+    const float4 x = xs4[q];
+    const bool s0 = fv_is_sentinel(w.x), s1 = fv_is_sentinel(w.y), s2 = fv_is_sentinel(w.z),
+               s3 = fv_is_sentinel(w.w);
+    bool c0 = false, c1 = false, c2 = false, c3 = false;
+    float d;
+    d = __fmul_rn(s, fv_dense_ds(x.x, w.x)); if (fabsf(d) > a.update_cut) { w.x = __fadd_rn(w.x, d); c0 = true; }
+    d = __fmul_rn(s, fv_dense_ds(x.y, w.y)); if (fabsf(d) > a.update_cut) { w.y = __fadd_rn(w.y, d); c1 = true; }
+    d = __fmul_rn(s, fv_dense_ds(x.z, w.z)); if (fabsf(d) > a.update_cut) { w.z = __fadd_rn(w.z, d); c2 = true; }
+    d = __fmul_rn(s, fv_dense_ds(x.w, w.w)); if (fabsf(d) > a.update_cut) { w.w = __fadd_rn(w.w, d); c3 = true; }
+    if (s0 | s1 | s2 | s3) {
+      // the slot kernel writes the sentinel positions; store the other components one by one
+      float *wp = (float *)&a.Wt4[p4];
+      if (c0) wp[0] = w.x;
+      if (c1) wp[1] = w.y;
+      if (c2) wp[2] = w.z;
+      if (c3) wp[3] = w.w;
+    } else if (c0 | c1 | c2 | c3) {
+      a.Wt4[p4] = w;
+    }
+    q += dq;
+    if (q >= a.ldk4) q -= a.ldk4;
+  }
+}
+
+// Kernel 5: the final value of every sparse element goes over its sentinel. Runs after the dense
+// update so no dense thread can mistake a finished element for an ordinary weight.
+__global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
+  const uint32_t e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= a.n_slots) return;
+  const fv_slot sl = a.slots[e];
+  if (sl.p == FV_SLOT_INVALID) return;
+  const float nc = a.scalars[0];
+  const float s = a.prec > nc ? a.eps / a.prec : a.eps / nc;
+  const uint32_t i = sl.p / a.ldk, h = sl.p - i * a.ldk;
+  const float f = a.invf[i >= a.V ? i - a.V : i];
+  const float v = fv_sparse_ds(a.xx[h], sl.wv, f, sl.n);
+  const float d = __fmul_rn(s, v);
+  ((float *)a.Wt4)[sl.p] = fabsf(d) > a.update_cut ? __fadd_rn(sl.wv, d) : sl.wv;
 }
 
 // ---- row norms (log line of flyvec/src/cuda_funcs.cu:1234-1242) -------------------------------
@@ -345,8 +522,11 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   if (t->stream) (void)hipStreamSynchronize(t->stream);
   fv_trainer_free_corpus(t);
   (void)hipFree(t->Wt);
-  (void)hipFree(t->cnt);
-  (void)hipFree(t->flags);
+  (void)hipFree(t->idx);
+  (void)hipFree(t->order);
+  (void)hipFree(t->slots);
+  (void)hipFree(t->emax);
+  (void)hipFree(t->bmax);
   (void)hipFree(t->win);
   (void)hipFree(t->sc);
   (void)hipFree(t->xx);
@@ -358,21 +538,27 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
 
 static int fv_trainer_alloc(fv_trainer *t) {
   const size_t elems = (size_t)t->N * t->ldk;
-  const size_t flag_words64 = ((size_t)t->total4 + 63) / 64;
   FV_HIP(hipStreamCreate(&t->stream));
   FV_HIP(hipMalloc((void **)&t->Wt, elems * sizeof(float)));
-  FV_HIP(hipMalloc((void **)&t->cnt, elems * sizeof(uint32_t)));
-  FV_HIP(hipMalloc((void **)&t->flags, flag_words64 * sizeof(uint64_t)));
+  FV_HIP(hipMalloc((void **)&t->idx, (size_t)t->B * t->w * sizeof(int32_t)));
   FV_HIP(hipMalloc((void **)&t->win, (size_t)t->B * sizeof(int32_t)));
   FV_HIP(hipMalloc((void **)&t->sc, (size_t)t->B * sizeof(float)));
+  FV_HIP(hipMalloc((void **)&t->order, (size_t)t->B * sizeof(uint32_t)));
+  FV_HIP(hipMalloc((void **)&t->slots, (size_t)t->B * t->w * sizeof(fv_slot)));
   FV_HIP(hipMalloc((void **)&t->xx, (size_t)t->ldk * sizeof(float)));
-  FV_HIP(hipMalloc((void **)&t->scalars, 16 * sizeof(uint32_t)));
+  FV_HIP(hipMalloc((void **)&t->emax, (size_t)t->K * sizeof(float)));
+  FV_HIP(hipMalloc((void **)&t->bmax, (size_t)t->dense_blocks * sizeof(float)));
+  FV_HIP(hipMalloc((void **)&t->scalars, 16 * sizeof(float)));
   FV_HIP(hipMemsetAsync(t->Wt, 0, elems * sizeof(float), t->stream));
-  FV_HIP(hipMemsetAsync(t->cnt, 0, elems * sizeof(uint32_t), t->stream));
-  FV_HIP(hipMemsetAsync(t->flags, 0, flag_words64 * sizeof(uint64_t), t->stream));
   FV_HIP(hipMemsetAsync(t->xx, 0, (size_t)t->ldk * sizeof(float), t->stream));
-  FV_HIP(hipMemsetAsync(t->scalars, 0, 16 * sizeof(uint32_t), t->stream));
+  FV_HIP(hipMemsetAsync(t->scalars, 0, 16 * sizeof(float), t->stream));
   FV_HIP(hipStreamSynchronize(t->stream));
+  // the neuron kernel counts column indices in LDS: as much of the column range per pass as fits
+  uint32_t chunk = (uint32_t)((t->N + 255) / 256 * 256);
+  if (chunk > FV_NB_MAX_CHUNK) chunk = FV_NB_MAX_CHUNK;
+  t->nb_chunk = chunk;
+  FV_HIP(hipFuncSetAttribute((const void *)fv_neuron_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                             (int)(chunk * sizeof(uint32_t))));
   return FV_OK;
 }
 
@@ -392,8 +578,10 @@ extern "C" int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_tr
              "delta != 0 (anti-Hebbian term on the m-th winner) is not implemented");
   const uint32_t ldk = fv_ldk(cfg->hid);
   const uint64_t N = 2 * cfg->vocab;
-  FV_REQUIRE(N * ldk / 4 < (1ull << 31), FV_ERR_INVALID,
-             "synapse matrix of %llu x %u floats exceeds 2^33 elements", (unsigned long long)N, ldk);
+  FV_REQUIRE(N * ldk < 0xffffffffull - (1u << 24), FV_ERR_INVALID,
+             "synapse matrix of %llu x %u floats exceeds 2^32 elements", (unsigned long long)N, ldk);
+  FV_REQUIRE((uint64_t)cfg->batch * cfg->window < (1ull << 31), FV_ERR_INVALID,
+             "batch x window = %llu is out of range", (unsigned long long)cfg->batch * cfg->window);
   fv_trainer *t = new fv_trainer();
   memset(t, 0, sizeof *t);
   t->cfg = *cfg;
@@ -592,11 +780,9 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.starts = t->starts;
   g.perm = t->perm;
   g.invf = t->invf;
-  g.cnt = t->cnt;
-  g.flags = t->flags;
+  g.idx = t->idx;
   g.win = t->win;
   g.sc = t->sc;
-  g.scalars = t->scalars;
   g.first = first;
   g.n = n;
   g.K = t->K;
@@ -616,27 +802,51 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
       return fv_fail(FV_ERR_INVALID, "hid = %u not supported", t->K);
   }
   if (ev) FV_HIP(hipEventRecord(ev[1], t->stream));
-  hipLaunchKernelGGL(fv_xx_totals_kernel, dim3((t->ldk + 3) / 4), dim3(256), 0, t->stream, t->win,
-                     t->sc, n, t->K, t->ldk, t->xx);
+  fv_neuron_args nb;
+  nb.win = t->win;
+  nb.sc = t->sc;
+  nb.idx = t->idx;
+  nb.invf = t->invf;
+  nb.Wt = t->Wt;
+  nb.xx = t->xx;
+  nb.emax = t->emax;
+  nb.order = t->order;
+  nb.slots = t->slots;
+  nb.chunk = t->nb_chunk;
+  nb.n = n;
+  nb.K = t->K;
+  nb.ldk = t->ldk;
+  nb.w = t->w;
+  nb.V = (uint32_t)t->V;
+  hipLaunchKernelGGL(fv_neuron_kernel, dim3(t->K), dim3(FV_NB_THREADS), t->nb_chunk * sizeof(uint32_t),
+                     t->stream, nb);
   if (ev) FV_HIP(hipEventRecord(ev[2], t->stream));
   fv_dense_args d;
   d.Wt4 = (float4 *)t->Wt;
-  d.cnt4 = (uint4 *)t->cnt;
-  d.flags64 = (uint64_t *)t->flags;
   d.xx = t->xx;
   d.invf = t->invf;
+  d.slots = t->slots;
+  d.emax = t->emax;
+  d.bmax = t->bmax;
   d.scalars = t->scalars;
   d.total4 = t->total4;
   d.ldk4 = t->ldk / 4;
+  d.ldk = t->ldk;
   d.V = (uint32_t)t->V;
+  d.K = t->K;
+  d.n_slots = n * t->w;
+  d.slot_blocks = (d.n_slots + 255) / 256;
+  d.n_bmax = t->dense_blocks;
   d.eps = eps;
   d.prec = t->cfg.prec;
   d.update_cut = t->update_cut;
   const size_t smem = (size_t)t->ldk * sizeof(float);
-  hipLaunchKernelGGL(fv_dense_kernel<false>, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
+  hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[3], t->stream));
-  hipLaunchKernelGGL(fv_dense_kernel<true>, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
+  hipLaunchKernelGGL(fv_update_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
+  hipLaunchKernelGGL(fv_slot_update_kernel, dim3(d.slot_blocks), dim3(256), 0, t->stream, d);
+  if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
   FV_HIP(hipGetLastError());
   t->last_n = n;
   return FV_OK;
@@ -702,9 +912,7 @@ extern "C" int fv_trainer_get_step_stats(fv_trainer *t, float *out_xx, float *ou
   FV_HIP(hipStreamSynchronize(t->stream));
   if (out_xx) FV_HIP(hipMemcpy(out_xx, t->xx, (size_t)t->K * sizeof(float), hipMemcpyDeviceToHost));
   if (out_max_abs_ds) {
-    uint32_t bits = 0;
-    FV_HIP(hipMemcpy(&bits, t->scalars, sizeof bits, hipMemcpyDeviceToHost));
-    memcpy(out_max_abs_ds, &bits, sizeof bits);
+    FV_HIP(hipMemcpy(out_max_abs_ds, t->scalars, sizeof(float), hipMemcpyDeviceToHost));
   }
   return FV_OK;
 }
