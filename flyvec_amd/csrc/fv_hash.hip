@@ -318,11 +318,13 @@ extern "C" int fv_hasher_time_windows(fv_hasher *h, const int32_t *idx_dev, uint
 }
 
 // ---- normalisation (flyvec/core.py:23-36, p = 2) -----------------------------------------------
-// numpy sums each row of syn**2 with its pairwise scheme: blocks of at most 128 elements are
-// summed with 8 interleaved accumulators combined as ((r0+r1)+(r2+r3))+((r4+r5)+(r6+r7)) plus a
-// sequential tail; longer ranges split at n/2 rounded down to a multiple of 8. The leaves of that
-// recursion are independent (first kernel); their combination order is a fixed tree replayed by a
-// small stack program (second kernel).
+// numpy sums each row of syn**2 in runs of 8192 elements (its buffer size), added in order onto 0;
+// each run is summed with its pairwise scheme: blocks of at most 128 elements with 8 interleaved
+// accumulators combined as ((r0+r1)+(r2+r3))+((r4+r5)+(r6+r7)) plus a sequential tail; longer
+// ranges split at n/2 rounded down to a multiple of 8. The leaves of that recursion are
+// independent (first kernel); their combination order is a fixed tree replayed by a small stack
+// program (second kernel).
+#define FV_NUMPY_BUFSIZE 8192u
 
 struct fv_leaf {
   uint32_t start, len;
@@ -382,14 +384,15 @@ __global__ void fv_combine_leaves_kernel(const float *__restrict__ leaf_sums, ui
     const int32_t op = prog[i];
     if (op >= 0) {
       stack[sp++] = leaf_sums[(uint64_t)op * K + h];
+    } else if (op == -2) {
+      stack[sp++] = 0.0f;
     } else {
       const float b = stack[--sp];
       const float a = stack[--sp];
       stack[sp++] = __fadd_rn(a, b);
     }
   }
-  // the reduction starts from add's identity: 0 + pairwise sum
-  out[h] = __fadd_rn(0.0f, stack[0]);
+  out[h] = stack[0];
 }
 
 __global__ __launch_bounds__(256) void fv_scale_rows_kernel(float *__restrict__ Wt, uint64_t N, uint32_t K,
@@ -406,7 +409,12 @@ extern "C" int fv_hasher_row_sumsq(fv_hasher *h, float *out_sums) {
   FV_REQUIRE(h && out_sums, FV_ERR_INVALID, "null argument");
   std::vector<fv_leaf> leaves;
   std::vector<int32_t> prog;
-  fv_pairwise_plan(0, (uint32_t)h->N, leaves, prog);
+  prog.push_back(-2);  // push 0: the reduction starts from add's identity
+  for (uint32_t s0 = 0; s0 < (uint32_t)h->N; s0 += FV_NUMPY_BUFSIZE) {
+    const uint32_t len = (uint32_t)h->N - s0 < FV_NUMPY_BUFSIZE ? (uint32_t)h->N - s0 : FV_NUMPY_BUFSIZE;
+    fv_pairwise_plan(s0, len, leaves, prog);
+    prog.push_back(-1);
+  }
   fv_leaf *d_leaves = nullptr;
   int32_t *d_prog = nullptr;
   float *d_leaf = nullptr, *d_out = nullptr;

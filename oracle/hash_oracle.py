@@ -105,3 +105,45 @@ def normalize_synapses(syn: np.ndarray, prec=1.0e-32, p=2) -> np.ndarray:
     K, N = syn.shape
     nc = np.power(np.sum(syn ** p, axis=1), 1 / p).reshape(K, 1)
     return syn / np.tile(nc + prec, (1, N))
+
+
+def pairwise_sum_f32(a: np.ndarray) -> np.float32:
+    """numpy's float32 pairwise summation of one contiguous run, restated: blocks of at most 128
+    elements are summed with 8 interleaved accumulators combined as ((r0+r1)+(r2+r3))+((r4+r5)+
+    (r6+r7)) plus a sequential tail; longer ranges split at n/2 rounded down to a multiple of 8."""
+    a = np.asarray(a, dtype=np.float32)
+    n = len(a)
+    if n < 8:
+        res = np.float32(-0.0)
+        for x in a:
+            res = np.float32(res + x)
+        return res
+    if n <= 128:
+        r = [np.float32(a[k]) for k in range(8)]
+        i = 8
+        while i < n - (n % 8):
+            for k in range(8):
+                r[k] = np.float32(r[k] + a[i + k])
+            i += 8
+        res = np.float32(np.float32(np.float32(r[0] + r[1]) + np.float32(r[2] + r[3])) +
+                         np.float32(np.float32(r[4] + r[5]) + np.float32(r[6] + r[7])))
+        while i < n:
+            res = np.float32(res + a[i])
+            i += 1
+        return res
+    n2 = n // 2
+    n2 -= n2 % 8
+    return np.float32(pairwise_sum_f32(a[:n2]) + pairwise_sum_f32(a[n2:]))
+
+
+NUMPY_BUFSIZE = 8192  # numpy.getbufsize() default: add.reduce hands the inner loop runs of this many elements
+
+
+def numpy_row_sum_f32(a: np.ndarray) -> np.float32:
+    """numpy.sum of one contiguous float32 row, restated: starting from 0, the pairwise sum of each
+    run of 8192 elements is added in order.  The device kernels of fv_hasher_row_sumsq follow this
+    plan; the test-suite checks it against numpy.sum itself."""
+    out = np.float32(0)
+    for s in range(0, len(a), NUMPY_BUFSIZE):
+        out = np.float32(out + pairwise_sum_f32(a[s:s + NUMPY_BUFSIZE]))
+    return out

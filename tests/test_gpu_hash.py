@@ -1,0 +1,156 @@
+"""Parity of the HIP hashing path against the numpy restatement of flyvec/core.py:153-158,
+through the C ABI.  Codes are compared bit for bit."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+f32 = np.float32
+
+
+def test_config1_target_ids(gpu):
+    """K = 400, V = 20000, 4096 Zipf target ids, k = 50, int8 codes (the reference's per-word path)."""
+    from flyvec_amd import Hasher, synthetic
+    from oracle import hash_oracle as ho
+    W = synthetic.synapses(400, 20000, seed=1)
+    ids = synthetic.zipf_ids(4096, 20000, seed=2)
+    h = Hasher(W)
+    got = h.hash_targets(ids, 50)
+    assert got.dtype == np.int8 and got.shape == (4096, 400)
+    assert np.array_equal(got, ho.hash_targets_loop(W, ids, 50))
+    assert (got.sum(axis=1) == 50).all()
+    h.close()
+
+
+def test_config3_window_batch(gpu):
+    """K = 400, V = 20000, 1,048,576 windows of w = 11, k = 32, 7 packed words per window.  The first
+    262,144 windows are compared with the numpy oracle bit for bit (CPU time bounds the sample); the
+    whole batch is checked through popcount, packed-vs-int8 agreement and repeatability."""
+    from flyvec_amd import Hasher, synthetic
+    from oracle import hash_oracle as ho
+    K, V, w, k, n = 400, 20000, 11, 32, 1 << 20
+    W = synthetic.synapses(K, V, seed=1)
+    idx = synthetic.window_indices(n, w, V, seed=7)
+    h = Hasher(W)
+    bits = h.hash_windows(idx, k, packed=True)
+    assert bits.shape == (n, 7) and bits.dtype == np.uint64
+    m = 1 << 18
+    want = ho.hash_windows(W, idx[:m], k)
+    assert np.array_equal(bits[:m], ho.pack_codes(want))
+    pop = np.unpackbits(bits.view(np.uint8), axis=1).sum(axis=1)
+    assert pop.max() <= k and (pop == k).mean() > 0.999          # exactly k bits unless fp32 ties
+    assert not (bits[:, 6] >> np.uint64(16)).any()                  # no bit beyond neuron 399
+    sub = slice(n - 50000, n)
+    b2, c2 = h.hash_windows(idx[sub], k, packed=True, codes=True)
+    assert np.array_equal(b2, bits[sub]) and np.array_equal(ho.pack_codes(c2), b2)
+    h.close()
+
+
+@pytest.mark.parametrize("K,V,w,k", [(2, 10, 1, 1), (5, 20, 3, 2), (63, 50, 11, 10), (64, 50, 11, 63), (65, 50, 5, 1),
+                                     (130, 40, 64, 50), (400, 300, 15, 399), (1000, 200, 15, 32), (2048, 30, 7, 100)])
+def test_shapes(gpu, K, V, w, k):
+    from flyvec_amd import Hasher
+    from oracle import hash_oracle as ho
+    rng = np.random.default_rng(K + w)
+    W = rng.standard_normal((K, 2 * V)).astype(f32)
+    idx = rng.integers(0, 2 * V, size=(700, w)).astype(np.int32)
+    idx[rng.random(idx.shape) < 0.1] = -1
+    idx[3] = -1                                                     # a fully masked window: all activations 0
+    h = Hasher(W)
+    bits, codes = h.hash_windows(idx, k, packed=True, codes=True)
+    want = ho.hash_windows(W, idx, k)
+    assert np.array_equal(codes, want)
+    assert np.array_equal(bits, ho.pack_codes(want))
+    assert codes[3].sum() == 0
+    h.close()
+
+
+def test_ties_adjacent_floats_and_equal_activations(gpu):
+    from flyvec_amd import Hasher
+    from oracle import hash_oracle as ho
+    rng = np.random.default_rng(3)
+    K, V = 100, 40
+    W = rng.integers(-2, 3, size=(K, 2 * V)).astype(f32)           # coarse grid: ties at the k / k+1 boundary
+    W[:, 5] = 1.0
+    W[: K // 2, 5] = np.nextafter(f32(1.0), f32(2.0))               # two adjacent floats only
+    W[:, 6] = 0.25                                                  # all equal
+    idx = rng.integers(0, 2 * V, size=(2000, 3)).astype(np.int32)
+    idx[0] = [5, -1, -1]
+    idx[1] = [6, -1, -1]
+    h = Hasher(W)
+    for k in (1, 7, 50, 99):
+        codes = h.hash_windows(idx, k, packed=False, codes=True)
+        want = ho.hash_windows(W, idx, k)
+        assert np.array_equal(codes, want)
+        assert (codes.sum(axis=1) <= k).all() and (codes.sum(axis=1) < k).any()
+        assert codes[1].sum() == 0
+    h.close()
+
+
+def test_argument_and_data_errors(gpu):
+    from flyvec_amd import Hasher, _lib
+    rng = np.random.default_rng(4)
+    K, V = 16, 10
+    h = Hasher(rng.standard_normal((K, 2 * V)).astype(f32))
+    with pytest.raises(IndexError):
+        h.hash_targets([1, 2], K)                                   # the reference reads act_sort[k]
+    with pytest.raises(IndexError):
+        h.hash_targets([1, 2], 0)
+    with pytest.raises(_lib.FlyvecError) as e:
+        h.hash_targets([1, V], 4)
+    assert e.value.code == _lib.FV_ERR_DATA
+    with pytest.raises(_lib.FlyvecError) as e:
+        h.hash_windows(np.array([[0, 2 * V, 1]], dtype=np.int32), 4)
+    assert e.value.code == _lib.FV_ERR_DATA
+    assert h.hash_windows(np.array([[0, 1, 2]], dtype=np.int32), 4).shape == (1, 1)   # still usable
+    assert h.hash_targets(np.array([], dtype=np.int32), 4).shape == (0, K)            # empty batch
+    assert np.array_equal(h.weights(), h.weights())
+    h.close()
+
+
+def test_normalize_matches_numpy(gpu):
+    from flyvec_amd import Hasher
+    from oracle import hash_oracle as ho
+    rng = np.random.default_rng(5)
+    for K, N in ((400, 40000), (37, 2 * 4097), (8, 6), (64, 2 * 8192)):
+        W = (rng.standard_normal((K, N)) * 10.0 ** rng.integers(-2, 2, size=(K, 1))).astype(f32)
+        h = Hasher(W)
+        assert np.array_equal(h.weights(), W)
+        h.normalize()
+        assert np.array_equal(h.weights(), ho.normalize_synapses(W)), (K, N)
+        h.close()
+
+
+def test_flyvec_wrapper_semantics(gpu, tmp_path):
+    """The behaviours the reference's notebook asserts (nbs/00_core.ipynb:333-350) on a synthetic model."""
+    from flyvec_amd import FlyVec
+    from oracle import hash_oracle as ho
+    rng = np.random.default_rng(6)
+    vocab = ["<UNK>", "hello", "world", "market", "fly"] + [f"tok{i}" for i in range(95)]
+    K, V = 400, len(vocab)
+    W = rng.standard_normal((K, 2 * V)).astype(f32)
+    path = tmp_path / "model.npy"
+    np.save(path, W)
+    (tmp_path / "config.yaml").write_text("synapses: model.npy\nnormalize_synapses: true\ntokenizer: tok.pkl\n")
+    model = FlyVec.from_config(tmp_path / "config.yaml", tokenizer=vocab)
+    Wn = ho.normalize_synapses(W)
+    emb = model.get_sparse_embedding("market")
+    assert emb["token"] == "market" and emb["id"] == 3
+    assert emb["embedding"].dtype == np.int8 and emb["embedding"].shape == (400,) and emb["embedding"].sum() == 50
+    assert np.array_equal(emb["embedding"], ho.sparse_code(Wn[:, V + 3], 50))
+    assert np.array_equal(model.get_sparse_embedding("hello world")["embedding"],
+                          model.get_sparse_embedding("hello")["embedding"])              # first token only
+    assert np.array_equal(model.get_sparse_embedding("HeLLo")["embedding"],
+                          model.get_sparse_embedding("hello")["embedding"])              # case-insensitive
+    assert model.get_sparse_embedding("market", 4)["embedding"].sum() == 4
+    unk = model.get_sparse_embedding("DefNotAWord")
+    assert unk["id"] == 0 and unk["token"] == "<UNK>" and not unk["embedding"].any()
+    assert unk["embedding"].dtype == np.uint8
+    with pytest.raises(ValueError, match="empty string"):
+        model.get_sparse_embedding("")
+    assert np.array_equal(model.get_dense_embedding("fly")["embedding"], Wn[:, V + 4])
+    vecs = model.simple_word_vectors(k=20)
+    assert set(vecs) == set(vocab) and all(v.shape == (400,) for v in vecs.values())
+    assert np.array_equal(vecs["world"], ho.sparse_code(Wn[:, V + 2], 20)) and not vecs["<UNK>"].any()
+    win = np.array([[1, 2, V + 3, 4, -1]], dtype=np.int32)
+    assert np.array_equal(model.get_context_embeddings(win, 30), ho.hash_windows(Wn, win, 30))

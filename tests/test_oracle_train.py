@@ -1,0 +1,303 @@
+"""Pins the training-step restatement (oracle/flyvec_oracle.c) without any import of the reference.
+
+Nothing in the reference tests the trainer, so the C restatement is checked against
+  * a from-scratch brute force of the same rule in Python scalars on tiny shapes,
+  * numpy restatements of the sampler and the activations,
+  * closed forms: one-window batch, W = 0 fixed point, invariance to rescaling 1/frequency by a
+    power of two, max|dW| == eps, rows changed == distinct winners with a non-zero total, masked
+    ids contribute nothing,
+  * for the reference's argmax reduction order, a second derivation (closed-form priority key)
+    of what the literal 64-thread simulation in C computes.
+"""
+import numpy as np
+import pytest
+
+from oracle import train_oracle as to
+
+f32 = np.float32
+
+
+# ---- brute force ---------------------------------------------------------------------------------
+
+def brute_argmax_lowest(raw):
+    best = 0
+    for i in range(1, len(raw)):
+        if raw[i] > raw[best]:
+            best = i
+    return best
+
+
+def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest):
+    """flyvec/src/cuda_funcs.cu:1662-1803 (sparse, frequency scaling, delta = 0) in Python scalars."""
+    W = W.copy()
+    K, N = W.shape
+    V = N // 2
+    n, w = idx.shape
+    win, sc = [], []
+    for r in range(n):
+        raw = []
+        for h in range(K):
+            s = 0.0  # double accumulator
+            for c in range(w):
+                i = idx[r, c]
+                if i != -1:
+                    s += float(W[h, i])
+            raw.append(f32(s))
+        b = argmax(raw)
+        ss = 0.0
+        for c in range(w):
+            i = idx[r, c]
+            if i != -1:
+                ss += float(f32(W[b, i] * invf[i % V]))  # fp32 product, double sum
+        win.append(b)
+        sc.append(f32(ss))
+    xx = [f32(0)] * K
+    for r in range(n):
+        xx[win[r]] = f32(xx[win[r]] + sc[r])
+    ds = np.zeros((K, N), dtype=f32)
+    for h in range(K):
+        if xx[h] != 0:
+            for c in range(N):
+                ds[h, c] = f32(-xx[h]) * W[h, c]
+    for r in range(n):
+        for c in range(w):
+            i = idx[r, c]
+            if i != -1:
+                ds[win[r], i] = f32(ds[win[r], i] + invf[i % V])
+    nc = f32(0)
+    for h in range(K):
+        if xx[h] != 0:
+            nc = max(nc, f32(np.max(np.abs(ds[h]))))
+        else:
+            ds[h] = 0
+    s = f32(eps) / f32(prec) if f32(prec) > nc else f32(eps) / nc
+    for h in range(K):
+        if xx[h] != 0:
+            for c in range(N):
+                v = f32(s * ds[h, c])
+                if abs(float(v)) > 1.0e-10:
+                    W[h, c] = f32(W[h, c] + v)
+    return W, np.array(win, dtype=np.int32), np.array(xx, dtype=f32), float(nc)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_step_against_brute_force(seed):
+    rng = np.random.default_rng(seed)
+    K, V, w, n = int(rng.integers(2, 5)), int(rng.integers(3, 7)), 3, int(rng.integers(1, 9))
+    W = rng.standard_normal((K, 2 * V)).astype(f32)
+    idx = rng.integers(0, V, size=(n, w)).astype(np.int32)
+    idx[:, w // 2] += V
+    idx[rng.random((n, w)) < 0.15] = -1
+    invf = (1.0 / rng.integers(1, 50, size=V)).astype(f32)
+    eps, prec = 2e-2, 1e-30
+    want_W, want_win, want_xx, want_nc = brute_step(W, idx, invf, eps, prec)
+    got_W = W.copy()
+    res = to.train_step(got_W, idx, invf, eps, prec, tie_rule=0)
+    assert np.array_equal(res["winners"], want_win)
+    assert np.array_equal(res["xx"], want_xx)
+    assert res["nc"] == want_nc
+    assert np.array_equal(got_W, want_W)
+
+
+# ---- stages against numpy ----------------------------------------------------------------------------
+
+def test_inflate_against_numpy():
+    rng = np.random.default_rng(1)
+    V, w = 50, 5
+    corpus = rng.integers(0, V, size=2000).astype(np.int32)
+    corpus[rng.integers(0, 2000, 50)] = -1
+    starts = np.sort(rng.integers(0, 2000 - w, size=300)).astype(np.uint64)
+    perm = rng.permutation(300).astype(np.uint64)
+    got = to.inflate(corpus, starts, perm, 20, 100, w, V)
+    want = np.stack([corpus[int(starts[p]):int(starts[p]) + w] for p in perm[20:120]]).copy()
+    mid = want[:, w // 2]
+    want[:, w // 2] = np.where(mid == -1, -1, mid + V)  # centre column goes to the target block
+    assert np.array_equal(got, want)
+
+
+def test_activations_against_numpy():
+    rng = np.random.default_rng(2)
+    K, V, w, n = 37, 40, 7, 64
+    W = rng.standard_normal((K, 2 * V)).astype(f32)
+    idx = rng.integers(0, 2 * V, size=(n, w)).astype(np.int32)
+    idx[rng.random((n, w)) < 0.1] = -1
+    invf = rng.random(V).astype(f32)
+    raw, sc = to.activations(W, idx, invf)
+    ok = idx >= 0
+    cols = np.where(ok, idx, 0)
+    g = W[:, cols]                                  # (K, n, w) fp32
+    want_raw = np.zeros((K, n))
+    want_sc = np.zeros((K, n))
+    for c in range(w):                               # double accumulation in window order
+        want_raw += np.where(ok[:, c], g[:, :, c].astype(np.float64), 0.0)
+        prod = (g[:, :, c] * invf[cols[:, c] % V]).astype(f32)   # fp32 product
+        want_sc += np.where(ok[:, c], prod.astype(np.float64), 0.0)
+    assert np.array_equal(raw, want_raw.T.astype(f32))
+    assert np.array_equal(sc, want_sc.T.astype(f32))
+
+
+def test_eps_schedule():
+    # flyvec/src/cuda_funcs.cu:1229: fp32 ratio, double product, one rounding
+    for lr0, ep, nep in [(2e-4, 0, 15), (2e-4, 7, 15), (0.002, 14, 15), (0.002, 3, 7)]:
+        want = f32(float(f32(lr0)) * (1.0 - float(f32(f32(ep) / f32(nep)))))
+        assert to.epoch_eps(lr0, ep, nep) == want
+
+
+# ---- argmax tie rules ------------------------------------------------------------------------------------
+
+def reference_priority(h):
+    """Closed form of the reduction order of flyvec/src/cuda_funcs.cu:488-561: thread t = h % 64
+    scans h = t, t+64, ...; warp 0 beats warp 1; inside a warp the shuffle-down tree with a strict
+    comparison prefers lanes in bit-reversed order; index 0 seeds every thread."""
+    if h == 0:
+        return (-1, 0, 0)
+    t, q = h % 64, h // 64
+    rev = int(f"{t % 32:05b}"[::-1], 2)
+    return (t // 32, rev, q)
+
+
+def argmax_by_priority(row):
+    m = max(row)
+    return min((h for h in range(len(row)) if row[h] == m), key=reference_priority)
+
+
+def test_reference_tie_rule_examples():
+    K = 400
+    row = np.zeros(K, dtype=f32)
+    assert to.argmax_reference(row) == 0          # all equal
+    row[:] = -1
+    row[1] = row[2] = 5                              # lane 2 (bit-reversed 8) beats lane 1 (16)
+    assert to.argmax_reference(row) == 2 and to.argmax_lowest(row) == 1
+    row[:] = -1
+    row[67] = row[5] = 5                             # lane 5 (reversed 20) beats lane 3 (24)
+    assert to.argmax_reference(row) == 5
+    row[:] = -1
+    row[40] = row[33] = 5                            # warp 1 lanes: 8 -> 2, 1 -> 16
+    assert to.argmax_reference(row) == 40
+    row[:] = -1
+    row[0] = row[17] = 5                             # the seed (data[0], 0) is never replaced by an equal
+    assert to.argmax_reference(row) == 0
+    row[:] = -1
+    row[64 + 9] = row[9] = 5                         # same thread: the lower index is met first
+    assert to.argmax_reference(row) == 9
+
+
+@pytest.mark.parametrize("K", [1, 5, 63, 64, 65, 130, 400, 1000])
+def test_reference_tie_rule_against_closed_form(K):
+    rng = np.random.default_rng(K)
+    for _ in range(200):
+        row = rng.integers(0, 4, size=K).astype(f32)  # few distinct values: ties everywhere
+        assert to.argmax_reference(row) == argmax_by_priority(list(row))
+        assert to.argmax_lowest(row) == int(np.argmax(row))
+    for _ in range(50):
+        row = rng.standard_normal(K).astype(f32)      # no ties: every rule is plain argmax
+        assert to.argmax_reference(row) == int(np.argmax(row)) == to.argmax_lowest(row)
+
+
+# ---- closed forms ---------------------------------------------------------------------------------------------
+
+def setup_small(seed, K=16, V=30, w=5, n=40):
+    rng = np.random.default_rng(seed)
+    W = (0.1 * rng.standard_normal((K, 2 * V))).astype(f32)
+    idx = rng.integers(0, V, size=(n, w)).astype(np.int32)
+    idx[:, w // 2] += V
+    invf = (1.0 / rng.integers(1, 200, size=V)).astype(f32)
+    return W, idx, invf
+
+
+def test_single_window_closed_form():
+    W, idx, invf = setup_small(0, n=1)
+    V = W.shape[1] // 2
+    W0 = W.copy()
+    res = to.train_step(W, idx, invf, 1e-3)
+    mu = int(res["winners"][0])
+    raw = W0[:, idx[0]].astype(np.float64).sum(axis=1).astype(f32)
+    assert mu == int(np.argmax(raw))
+    sc = f32((W0[mu, idx[0]] * invf[idx[0] % V]).astype(f32).astype(np.float64).sum())
+    assert res["xx"][mu] == sc and np.count_nonzero(res["xx"]) == 1
+    ds = f32(-sc) * W0[mu]
+    for i in idx[0]:
+        ds[i] = f32(ds[i] + invf[i % V])
+    assert np.array_equal(res["ds"][mu], ds)
+    changed = np.flatnonzero((W != W0).any(axis=1))
+    assert changed.tolist() == [mu]                  # every other row untouched
+
+
+def test_zero_matrix_is_a_fixed_point():
+    W, idx, invf = setup_small(1)
+    W[:] = 0
+    res = to.train_step(W, idx, invf, 1e-3)
+    assert not W.any() and res["nc"] == 0.0 and not res["xx"].any()
+    assert (res["winners"] == 0).all()               # all-equal activations: index 0 under both rules
+
+
+def test_rows_changed_are_the_winners_and_step_size_is_eps():
+    W, idx, invf = setup_small(2)
+    W0 = W.copy()
+    eps = 1e-3
+    res = to.train_step(W, idx, invf, eps)
+    won = np.unique(res["winners"])
+    won = won[res["xx"][won] != 0]
+    assert np.flatnonzero((W != W0).any(axis=1)).tolist() == won.tolist()
+    assert res["nc"] == np.abs(res["ds"]).max()
+    assert abs(np.abs(W - W0).max() - eps) <= 2e-7 * max(1.0, np.abs(W0).max())  # s * nc == eps up to rounding
+
+
+def test_invariant_to_power_of_two_rescale_of_inverse_frequency():
+    # xx and the sparse term are both linear in 1/f and max|ds| divides the scale out; a power of
+    # two makes every intermediate scale exactly
+    W, idx, invf = setup_small(3)
+    Wa, Wb = W.copy(), W.copy()
+    ra = to.train_step(Wa, idx, invf, 1e-3)
+    rb = to.train_step(Wb, idx, (invf * f32(8)).astype(f32), 1e-3)
+    assert np.array_equal(ra["winners"], rb["winners"])
+    assert np.array_equal(rb["xx"], ra["xx"] * f32(8)) and rb["nc"] == ra["nc"] * 8
+    assert np.array_equal(Wa, Wb)
+
+
+def test_masked_positions_contribute_nothing():
+    W, idx, invf = setup_small(4)
+    V = W.shape[1] // 2
+    # a column nobody else uses, then mask it: same result as if those windows were shorter
+    idx2 = idx.copy()
+    idx2[:, 0] = -1
+    Wa = W.copy()
+    ra = to.train_step(Wa, idx2, invf, 1e-3)
+    Wz = W.copy()
+    Wz[:, V - 1] = 0                                   # a zero column adds exactly 0 to every sum ...
+    idx3 = idx.copy()
+    idx3[:, 0] = V - 1
+    invf3 = invf.copy()
+    invf3[V - 1] = 0                                   # ... and a zero 1/f adds 0 to ds
+    idx3[idx3 == V - 1] = V - 1
+    keep = ~(idx[:, 1:] == V - 1).any(axis=1)          # windows that do not otherwise use that column
+    Wb = Wz.copy()
+    rb = to.train_step(Wb, idx3[keep], invf3, 1e-3)
+    Wc = Wz.copy()
+    rc = to.train_step(Wc, idx2[keep], invf3, 1e-3)
+    assert np.array_equal(rb["winners"], rc["winners"]) and np.array_equal(Wb, Wc)
+    assert ra["winners"].shape[0] == idx.shape[0]
+
+
+def test_multi_step_driver_matches_single_steps():
+    rng = np.random.default_rng(7)
+    V, K, w, B = 40, 12, 5, 16
+    corpus = rng.integers(0, V, size=3000).astype(np.int32)
+    off = np.concatenate([[0], np.cumsum(rng.geometric(1 / 20, size=200))]).astype(np.uint64)
+    off = off[off <= 3000]
+    starts = to.window_starts(off, w)
+    perm = rng.permutation(len(starts)).astype(np.uint64)
+    invf = to.inverse_frequency(corpus, V)
+    W = (0.1 * rng.standard_normal((K, 2 * V))).astype(f32)
+    Wa, Wb = W.copy(), W.copy()
+    wins = to.train_steps(Wa, corpus, starts, perm, 0, B, 3, w, invf, 1e-3)
+    got = []
+    for s in range(3):
+        idx = to.inflate(corpus, starts, perm, s * B, B, w, V)
+        got.append(to.train_step(Wb, idx, invf, 1e-3)["winners"])
+    assert np.array_equal(wins, np.concatenate(got)) and np.array_equal(Wa, Wb)
+    # last partial batch: only the remainder is processed
+    tail = len(perm) - (len(perm) // B) * B
+    if tail:
+        wt = to.train_steps(Wa, corpus, starts, perm, (len(perm) // B) * B, B, 1, w, invf, 1e-3)
+        assert len(wt) == tail
