@@ -40,7 +40,8 @@ def train_bytes(K, N, w, B):
     ids, 1/f lookups and the sparse count updates are 16 bytes per window position."""
     per = {
         "gather_winner": 4 * B * w * K,
-        "neuron_owners": 8 * B + 8 * B * w,
+        "group_xx": 8 * B,
+        "sparse_owners": 8 * B * w,
         "absmax_ds": 4 * K * N,
         "update": 8 * K * N,
         "slot_update": 8 * B * w,

@@ -14,8 +14,8 @@ import os
 LIB_PATH = Path(os.environ.get("FLYVEC_HIP_LIB") or Path(__file__).resolve().parent / "lib" / "libflyvec_hip.so")
 
 FV_OK, FV_ERR_INVALID, FV_ERR_HIP, FV_ERR_STATE, FV_ERR_DATA = range(5)
-FV_TRAIN_KERNELS = 5
-TRAIN_KERNEL_NAMES = ("gather_winner", "neuron_owners", "absmax_ds", "update", "slot_update")
+FV_TRAIN_KERNELS = 6
+TRAIN_KERNEL_NAMES = ("gather_winner", "group_xx", "sparse_owners", "absmax_ds", "update", "slot_update")
 
 
 class FlyvecError(RuntimeError):

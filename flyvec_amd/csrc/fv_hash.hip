@@ -39,33 +39,8 @@ struct fv_hash_args {
   uint32_t *err;
 };
 
-template <int NV, int RB>
-__device__ __forceinline__ void fv_hash_gather(const float *__restrict__ Wt, uint32_t ldk, uint32_t K,
-                                               int lane, int w, int32_t idx_lane, float (&acc)[NV]) {
-  for (int c0 = 0; c0 < w; c0 += RB) {
-    float v[RB][NV];
-#pragma unroll
-    for (int b = 0; b < RB; ++b) {
-      const int c = c0 + b;
-      const int32_t i = (int32_t)fv_readlane((uint32_t)idx_lane, c < 63 ? c : 63);
-      const bool ok = (c < w) && (i >= 0);
-      const float *row = Wt + (uint64_t)(ok ? i : 0) * ldk + lane;
-#pragma unroll
-      for (int j = 0; j < NV; ++j) {
-        const bool in = ok && (j < NV - 1 || (uint32_t)(lane + 64 * j) < K);
-        v[b][j] = in ? row[64 * j] : 0.0f;
-      }
-    }
-#pragma unroll
-    for (int b = 0; b < RB; ++b)
-#pragma unroll
-      for (int j = 0; j < NV; ++j) acc[j] = __fadd_rn(acc[j], v[b][j]);
-  }
-}
-
 template <int NV>
 __global__ __launch_bounds__(256) void fv_hash_kernel(fv_hash_args a) {
-  constexpr int RB = NV <= 2 ? 16 : NV <= 4 ? 8 : NV <= 8 ? 4 : NV <= 16 ? 2 : 1;
   const int lane = threadIdx.x & 63;
   const uint64_t n_waves = (uint64_t)gridDim.x * 4;
   for (uint64_t r = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6); r < a.n; r += n_waves) {
@@ -84,7 +59,7 @@ __global__ __launch_bounds__(256) void fv_hash_kernel(fv_hash_args a) {
     float acc[NV];
 #pragma unroll
     for (int j = 0; j < NV; ++j) acc[j] = 0.0f;
-    fv_hash_gather<NV, RB>(a.Wt, a.ldk, a.K, lane, (int)a.w, idx, acc);
+    fv_gather_accumulate<NV, fv_rows_per_batch<NV>::value, float>(a.Wt, a.ldk, a.K, a.n_cols, lane, (int)a.w, idx, acc);
 
     uint32_t key[NV];
 #pragma unroll

@@ -134,3 +134,53 @@ __device__ __forceinline__ uint32_t fv_wave_max_u32(uint32_t v) {
 
 __device__ __forceinline__ uint32_t fv_wave_min_u32(uint32_t v) { return ~fv_wave_max_u32(~v); }
 
+
+// ---- gather-sum of one window, shared by the training and the hashing kernel ----------------
+// Lane l holds neurons l, l + 64, ... of the window's activation. acc[j] += W[idx_c][l + 64 j]
+// for every window position c in order (idx_c is held by lane c of idx_lane; positions whose
+// index is outside [0, n_cols) add +0, which leaves a sum that started at +0 unchanged).
+// Every load is unconditional -- rows of skipped positions read row 0, lanes past K re-read
+// element K - 1, both replaced by 0 afterwards -- so a batch of RB rows is RB * NV independent
+// loads in flight per lane with no branch between them.
+template <int NV, int RB, typename Acc>
+__device__ __forceinline__ void fv_gather_batch(const float *__restrict__ Wt, uint32_t ldk, uint32_t n_cols,
+                                                const uint32_t (&off)[NV], bool last_valid, int c0,
+                                                int32_t idx_lane, Acc (&acc)[NV]) {
+  float v[RB][NV];
+  bool ok[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    const int32_t i = (int32_t)fv_readlane((uint32_t)idx_lane, c0 + b);
+    ok[b] = (uint32_t)i < n_cols;
+    const float *row = Wt + (uint64_t)(ok[b] ? (uint32_t)i : 0u) * ldk;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[b][j] = row[off[j]];
+  }
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const bool use = ok[b] && (j < NV - 1 || last_valid);
+      acc[j] = acc[j] + (Acc)(use ? v[b][j] : 0.0f);
+    }
+  }
+}
+
+template <int NV, int RB, typename Acc>
+__device__ __forceinline__ void fv_gather_accumulate(const float *__restrict__ Wt, uint32_t ldk, uint32_t K,
+                                                     uint32_t n_cols, int lane, int w, int32_t idx_lane,
+                                                     Acc (&acc)[NV]) {
+  uint32_t off[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) off[j] = (uint32_t)lane + 64u * j;
+  const bool last_valid = off[NV - 1] < K;
+  if (!last_valid) off[NV - 1] = K - 1;
+  int c0 = 0;
+  for (; c0 + RB <= w; c0 += RB) fv_gather_batch<NV, RB, Acc>(Wt, ldk, n_cols, off, last_valid, c0, idx_lane, acc);
+  for (; c0 < w; ++c0) fv_gather_batch<NV, 1, Acc>(Wt, ldk, n_cols, off, last_valid, c0, idx_lane, acc);
+}
+
+template <int NV>
+struct fv_rows_per_batch {
+  static constexpr int value = NV <= 2 ? 16 : NV <= 4 ? 8 : NV <= 8 ? 4 : NV <= 16 ? 2 : 1;
+};

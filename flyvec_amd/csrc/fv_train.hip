@@ -61,11 +61,10 @@ struct fv_trainer {
   int32_t *win;     // B winners
   float *sc;        // B scaled activations at the winner
   uint32_t *order;  // B window ids grouped by winner, ascending inside a group
-  uint32_t nb_chunk;  // column counters per LDS pass of the neuron kernel
-  fv_slot *slots;   // B x w slot records
+  uint32_t *group_base, *group_count;  // K each
+  fv_slot *slots;   // FV_NB_CLASSES regions of B x w slot records
   float *xx;        // ldk
-  float *emax;      // K: max|ds| over the sparse elements of each neuron
-  float *bmax;      // dense_blocks: max|ds| of each dense block
+  float *bmax;      // max|ds| of each dense block and each slot block of the absmax launch
   float *scalars;   // [0] max|ds| of the last step
   uint32_t last_n;
   uint64_t shuffle_calls;
@@ -87,38 +86,6 @@ struct fv_gather_args {
   float *sc;
   uint64_t first;
   uint32_t n, K, ldk, w, V, tie_rule;
-};
-
-// acc[j] += W[idx_c][lane + 64 j] for every window position c, in order; positions are taken
-// RB at a time so RB * NV independent loads are in flight per lane.
-template <int NV, int RB, typename Acc>
-__device__ __forceinline__ void fv_gather_accumulate(const float *__restrict__ Wt, uint32_t ldk,
-                                                     uint32_t K, uint32_t n_cols, int lane, int w,
-                                                     int32_t idx_lane, Acc (&acc)[NV]) {
-  for (int c0 = 0; c0 < w; c0 += RB) {
-    float v[RB][NV];
-#pragma unroll
-    for (int b = 0; b < RB; ++b) {
-      const int c = c0 + b;
-      const int32_t i = (int32_t)fv_readlane((uint32_t)idx_lane, c < 63 ? c : 63);
-      const bool ok = (c < w) && ((uint32_t)i < n_cols);
-      const float *row = Wt + (uint64_t)(ok ? i : 0) * ldk + lane;
-#pragma unroll
-      for (int j = 0; j < NV; ++j) {
-        const bool in = ok && (j < NV - 1 || (uint32_t)(lane + 64 * j) < K);
-        v[b][j] = in ? row[64 * j] : 0.0f;
-      }
-    }
-#pragma unroll
-    for (int b = 0; b < RB; ++b)
-#pragma unroll
-      for (int j = 0; j < NV; ++j) acc[j] = acc[j] + (Acc)v[b][j];
-  }
-}
-
-template <int NV>
-struct fv_rows_per_batch {
-  static constexpr int value = NV <= 2 ? 16 : NV <= 4 ? 8 : NV <= 8 ? 4 : NV <= 16 ? 2 : 1;
 };
 
 template <int NV>
@@ -186,24 +153,29 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
   }
 }
 
-// ---- kernel 2: one block per neuron -- its windows, xx, and its sparse elements --------------------
+// ---- kernel 2: group the windows by winner, xx ----------------------------------------------------
+//
+// One block per neuron h scans the winner array once (every thread a contiguous run, so per-thread
+// match counts are in window order) and writes the neuron's windows, ascending, to
+// order[group_base[h] .. +group_count[h]); it then adds their scaled activations in that order: xx[h].
 
-#define FV_NB_THREADS 1024
-#define FV_NB_WAVES (FV_NB_THREADS / 64)
-#define FV_NB_MAX_CHUNK 32768  // column counters per LDS pass (128 KB of the CU's 160 KB)
-#define FV_NB_SC_CACHE 2048
+#define FV_NB_MAX_THREADS 1024
+#ifndef FV_NB_CLASS_SHIFT
+#define FV_NB_CLASS_SHIFT 2
+#endif
+#define FV_NB_CLASSES (1 << FV_NB_CLASS_SHIFT)  // column classes per neuron (kernel 3)
+#define FV_NB_CNT_WORDS 5120    // LDS counter words per class block (20 KB)
+#define FV_NB_ROUND 2048        // scaled activations staged in LDS at a time
+#define FV_NB_LOADS 16          // independent loads issued together
 
-struct fv_neuron_args {
-  const int32_t *win;
+struct fv_group_args {
+  const int32_t *win;  // padded: readable up to n rounded up to 16
   const float *sc;
-  const int32_t *idx;
-  const float *invf;
-  float *Wt;
-  float *xx;
-  float *emax;
   uint32_t *order;
-  fv_slot *slots;
-  uint32_t n, K, ldk, w, V, chunk;
+  uint32_t *group_base;
+  uint32_t *group_count;
+  float *xx;
+  uint32_t n;
 };
 
 // ds of one sparse element: the dense term, then n sequential additions of 1/f.
@@ -216,9 +188,20 @@ __device__ __forceinline__ float fv_absmax_keep(float m, float v) {
   return a > m ? a : m;  // a NaN never replaces m, as in the reference's comparison
 }
 
-// Exclusive prefix sum of one value per thread over the block, and the block total.
-__device__ __forceinline__ uint32_t fv_block_exclusive_scan(uint32_t v, uint32_t *wave_tot /*FV_NB_WAVES+1*/,
-                                                            uint32_t *total) {
+// Sum over the block of one value per thread (result in every thread).
+__device__ __forceinline__ uint32_t fv_block_sum_u32(uint32_t v, uint32_t *smem /*17*/) {
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_down(v, d, 64);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+  __syncthreads();
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  uint32_t t = 0;
+  for (int i = 0; i < n_waves; ++i) t += smem[i];
+  return t;
+}
+
+// Exclusive prefix sum of one value per thread over the block.
+__device__ __forceinline__ uint32_t fv_block_exclusive_scan(uint32_t v, uint32_t *smem /*17*/) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   uint32_t incl = v;
 #pragma unroll
@@ -227,148 +210,211 @@ __device__ __forceinline__ uint32_t fv_block_exclusive_scan(uint32_t v, uint32_t
     if (lane >= d) incl += o;
   }
   __syncthreads();
-  if (lane == 63) wave_tot[wave] = incl;
+  if (lane == 63) smem[wave] = incl;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    uint32_t run = 0;
-    for (int i = 0; i < FV_NB_WAVES; ++i) {
-      const uint32_t t = wave_tot[i];
-      wave_tot[i] = run;
-      run += t;
-    }
-    wave_tot[FV_NB_WAVES] = run;
-  }
-  __syncthreads();
-  *total = wave_tot[FV_NB_WAVES];
-  return wave_tot[wave] + incl - v;
+  uint32_t before = 0;
+  for (int i = 0; i < wave; ++i) before += smem[i];
+  return before + incl - v;
 }
 
-__global__ __launch_bounds__(FV_NB_THREADS) void fv_neuron_kernel(fv_neuron_args a) {
-  extern __shared__ uint32_t cnt[];  // a.chunk counters, one per column index of the current pass
-  __shared__ float scbuf[FV_NB_SC_CACHE];
-  __shared__ uint32_t wave_tot[FV_NB_WAVES + 1];
-  __shared__ uint32_t sh_lt, sh_pos;
-  __shared__ float sh_xx, sh_wmax[FV_NB_WAVES];
+__global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_args a) {
+  __shared__ float scbuf[FV_NB_ROUND];
+  __shared__ uint32_t red[17];
 
   const uint32_t h = blockIdx.x;
-  const uint32_t tid = threadIdx.x;
+  const uint32_t tid = threadIdx.x, T = blockDim.x;
   const uint32_t n = a.n;
   const int32_t *__restrict__ win = a.win;
-  const int32_t *__restrict__ idx = a.idx;
 
-  if (tid == 0) {
-    sh_lt = 0;
-    sh_pos = 0;
-  }
-  for (uint32_t i = tid; i < a.chunk / 4; i += FV_NB_THREADS) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
-
-  // (1) windows won by lower neurons / by this one. Each thread takes a contiguous segment, so the
-  // per-thread match counts scan into window order; matches of the first 64 windows of a segment
-  // are remembered as a bit mask so the second walk needs no reload.
-  const uint32_t seg = (n + FV_NB_THREADS - 1) / FV_NB_THREADS;
+  // A thread's run is a multiple of 4 windows, read as 16-byte loads; matches among its first 64
+  // windows are kept as a bit mask.
+  const uint32_t seg = ((n + T - 1) / T + 3) & ~3u;
   const uint32_t r0 = min(tid * seg, n), r1 = min(r0 + seg, n);
+  const uint32_t n_pad = (n + 15) & ~15u;
   uint32_t lt = 0, eq = 0;
   uint64_t mask = 0;
-#pragma unroll 8
-  for (uint32_t r = r0; r < r1; ++r) {
-    const uint32_t wv = (uint32_t)win[r];
-    lt += wv < h;
-    const bool hit = wv == h;
-    eq += hit;
-    if (hit && r - r0 < 64) mask |= 1ull << (r - r0);
+  for (uint32_t rb = r0; rb < r1; rb += FV_NB_LOADS) {
+    int4 wv4[FV_NB_LOADS / 4];
+#pragma unroll
+    for (int q = 0; q < FV_NB_LOADS / 4; ++q) wv4[q] = *(const int4 *)(win + min(rb + 4 * q, n_pad - 4));
+#pragma unroll
+    for (int q = 0; q < FV_NB_LOADS; ++q) {
+      const int4 v4 = wv4[q >> 2];
+      const uint32_t wv = (uint32_t)((q & 3) == 0 ? v4.x : (q & 3) == 1 ? v4.y : (q & 3) == 2 ? v4.z : v4.w);
+      const bool in = rb + q < r1;
+      lt += in && wv < h;
+      const bool hit = in && wv == h;
+      eq += hit;
+      const uint32_t o = rb + q - r0;
+      mask |= o < 64 ? (uint64_t)hit << o : 0ull;
+    }
   }
-  __syncthreads();
-  {
-    uint32_t wl = lt;  // wave-reduce before touching the shared counter
-    for (int d = 32; d >= 1; d >>= 1) wl += __shfl_down(wl, d, 64);
-    if ((tid & 63) == 0 && wl) atomicAdd(&sh_lt, wl);
+  const uint32_t base = fv_block_sum_u32(lt, red);  // windows won by lower neurons
+  const uint32_t my_off = fv_block_exclusive_scan(eq, red);
+  const uint32_t c_h = fv_block_sum_u32(eq, red);
+  if (tid == 0) {
+    a.group_base[h] = base;
+    a.group_count[h] = c_h;
   }
-  uint32_t c_h;
-  const uint32_t my_off = fv_block_exclusive_scan(eq, wave_tot, &c_h);
-  const uint32_t base = sh_lt;  // start of this neuron's group in order[]
+  uint32_t *order = a.order + base;
   {
-    uint32_t pos = base + my_off;
-    while (mask) {
-      a.order[pos++] = r0 + (uint32_t)__ffsll((long long)mask) - 1;
-      mask &= mask - 1;
+    uint32_t rank = my_off;
+    uint64_t mm = mask;
+    while (mm) {
+      order[rank++] = r0 + (uint32_t)__ffsll((long long)mm) - 1;
+      mm &= mm - 1;
     }
     for (uint32_t r = r0 + 64; r < r1; ++r)
-      if ((uint32_t)win[r] == h) a.order[pos++] = r;
+      if ((uint32_t)win[r] == h) order[rank++] = r;
   }
-  __syncthreads();  // order[base .. base + c_h) is now readable by the whole block
-  const uint32_t *__restrict__ order = a.order + base;
+  __syncthreads();  // the neuron's part of order[] is now readable by the whole block
 
-  // (2) xx[h]: fp32 adds in window order
+  // xx[h] = fp32 sum of the scaled activations in window order
   float xx = 0.0f;
-  for (uint32_t j0 = 0; j0 < c_h; j0 += FV_NB_SC_CACHE) {
-    const uint32_t m = min(c_h - j0, (uint32_t)FV_NB_SC_CACHE);
-    for (uint32_t j = tid; j < m; j += FV_NB_THREADS) scbuf[j] = a.sc[order[j0 + j]];
+  for (uint32_t j0 = 0; j0 < c_h; j0 += FV_NB_ROUND) {
+    const uint32_t mr = min(c_h - j0, (uint32_t)FV_NB_ROUND);
+    for (uint32_t jb = tid; jb < mr; jb += 4 * T) {  // up to 4 independent loads per thread
+      uint32_t r[4];
+      float v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) r[q] = order[j0 + min(jb + q * T, mr - 1)];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = a.sc[r[q]];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (jb + q * T < mr) scbuf[jb + q * T] = v[q];
+    }
     __syncthreads();
     if (tid == 0) {
-#pragma unroll 8
-      for (uint32_t j = 0; j < m; ++j) xx = __fadd_rn(xx, scbuf[j]);
+      uint32_t j = 0;
+      for (; j + 16 <= mr; j += 16) {  // 16 values fetched together, then the dependent adds
+        float4 v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = *(const float4 *)&scbuf[j + 4 * q];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          xx = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(xx, v[q].x), v[q].y), v[q].z), v[q].w);
+      }
+      for (; j < mr; ++j) xx = __fadd_rn(xx, scbuf[j]);
     }
     __syncthreads();
   }
-  if (tid == 0) {
-    sh_xx = xx;
-    a.xx[h] = xx;
-  }
-  __syncthreads();
-  xx = sh_xx;
+  if (tid == 0) a.xx[h] = xx;
+}
 
-  // (3) sparse elements of row h. The neuron's windows own the slot records [base*w, (base+c_h)*w).
+// ---- kernel 3: sparse elements -----------------------------------------------------------------------
+//
+// FV_NB_CLASSES blocks per neuron h; block q owns the elements (h, column i) with
+// i mod FV_NB_CLASSES == q, so a neuron that won a large share of the minibatch is spread over
+// several blocks and no two blocks share an element.  A block counts the occurrences of each of
+// its columns over the neuron's windows in LDS, and for every distinct one saves
+// (element, count, weight) in a slot record and plants the sentinel in W.
+
+struct fv_sparse_args {
+  const uint32_t *order;
+  const uint32_t *group_base;
+  const uint32_t *group_count;
+  const int32_t *idx;
+  float *Wt;
+  fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records
+  uint64_t slot_stride;
+  uint32_t ldk, w, V;
+};
+
+__global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
+  __shared__ uint32_t cnt[FV_NB_CNT_WORDS];
+  __shared__ uint32_t sh_pos;
+  constexpr uint32_t T = 256;
+  const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT;
+  const uint32_t q = blockIdx.x & (FV_NB_CLASSES - 1);
+  const uint32_t tid = threadIdx.x;
+  const uint32_t c_h = a.group_count[h];
+  if (c_h == 0) return;
+  const uint32_t base = a.group_base[h];
+  const uint32_t *__restrict__ order = a.order + base;
+  const int32_t *__restrict__ idx = a.idx;
+  const uint32_t n_cols = 2 * a.V;
   const uint32_t m_ent = c_h * a.w;
-  fv_slot *slots = a.slots + (uint64_t)base * a.w;
-  float m = 0.0f;
-  uint32_t n_emitted = 0;
-  if (xx != 0.0f) {  // (the reference zero-fills ds of a row with xx == 0: no sparse term, no update)
-    const uint32_t n_cols = 2 * a.V;
-    for (uint32_t lo = 0; lo < n_cols; lo += a.chunk) {
-      // count the occurrences of every column index of this pass: one window per thread at a time
-      for (uint32_t j = tid; j < c_h; j += FV_NB_THREADS) {
-        const int32_t *row = idx + (uint64_t)order[j] * a.w;
-        for (uint32_t c = 0; c < a.w; ++c) {
-          const int32_t i = row[c];
-          const uint32_t k = (uint32_t)i - lo;
-          if ((uint32_t)i < n_cols && k < a.chunk) atomicAdd(&cnt[k], 1u);
-        }
-      }
-      __syncthreads();
-      // every non-zero counter is one distinct element (h, column): save its weight and count in
-      // a slot record, evaluate ds, plant the sentinel; reset the counter for the next pass
-      for (uint32_t k4 = tid; k4 < a.chunk / 4; k4 += FV_NB_THREADS) {
-        const uint4 c4 = ((const uint4 *)cnt)[k4];
-        if ((c4.x | c4.y | c4.z | c4.w) == 0) continue;
-        ((uint4 *)cnt)[k4] = make_uint4(0, 0, 0, 0);
-        const uint32_t cc[4] = {c4.x, c4.y, c4.z, c4.w};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          if (cc[q] == 0) continue;
-          const uint32_t i = lo + k4 * 4 + q;
-          fv_slot sl;
-          sl.p = i * a.ldk + h;
-          sl.n = cc[q];
-          sl.wv = a.Wt[sl.p];
-          const float f = a.invf[i >= a.V ? i - a.V : i];
-          m = fv_absmax_keep(m, fv_sparse_ds(xx, sl.wv, f, sl.n));
-          a.Wt[sl.p] = __uint_as_float(FV_SENTINEL);
-          slots[atomicAdd(&sh_pos, 1u)] = sl;
-        }
-      }
-      __syncthreads();
-    }
-    n_emitted = sh_pos;
-  }
-  for (uint32_t e = n_emitted + tid; e < m_ent; e += FV_NB_THREADS) slots[e].p = FV_SLOT_INVALID;
-  const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));  // m >= 0: bit order == value order
-  if ((tid & 63) == 0) sh_wmax[tid >> 6] = __uint_as_float(wm);
+  fv_slot *slots = a.slots + (uint64_t)q * a.slot_stride + (uint64_t)base * a.w;
+
+  if (tid == 0) sh_pos = 0;
+  for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
   __syncthreads();
-  if (tid == 0) {
-    float bm = 0.0f;
-    for (int i = 0; i < FV_NB_WAVES; ++i) bm = fmaxf(bm, sh_wmax[i]);
-    a.emax[h] = bm;
+
+  // No counter can exceed the neuron's number of window positions: below 2^16 of them, two 16-bit
+  // counters share a word and one pass covers twice as many columns.
+  const bool narrow = m_ent < 65536u;
+  const uint32_t span = narrow ? 2 * FV_NB_CNT_WORDS : FV_NB_CNT_WORDS;          // class columns per pass
+  const uint32_t class_cols = (n_cols + FV_NB_CLASSES - 1) >> FV_NB_CLASS_SHIFT;  // columns of a class
+  uint32_t emitted = 0;
+
+  for (uint32_t lo = 0; lo < class_cols; lo += span) {
+    // count: one window position per thread at a time, FV_NB_LOADS of them in flight
+    for (uint32_t eb = tid; eb < m_ent; eb += FV_NB_LOADS * T) {
+      uint32_t rr[FV_NB_LOADS], cc[FV_NB_LOADS];
+      int32_t iv[FV_NB_LOADS];
+#pragma unroll
+      for (int u = 0; u < FV_NB_LOADS; ++u) {
+        const uint32_t e = min(eb + u * T, m_ent - 1);
+        const uint32_t j = e / a.w;
+        cc[u] = e - j * a.w;
+        rr[u] = order[j];
+      }
+#pragma unroll
+      for (int u = 0; u < FV_NB_LOADS; ++u) iv[u] = idx[(uint64_t)rr[u] * a.w + cc[u]];
+#pragma unroll
+      for (int u = 0; u < FV_NB_LOADS; ++u) {
+        const uint32_t i = (uint32_t)iv[u];
+        const uint32_t k = (i >> FV_NB_CLASS_SHIFT) - lo;
+        if (eb + u * T < m_ent && i < n_cols && (i & (FV_NB_CLASSES - 1)) == q && k < span) {
+          if (narrow)
+            atomicAdd(&cnt[k >> 1], 1u << (16 * (k & 1)));
+          else
+            atomicAdd(&cnt[k], 1u);
+        }
+      }
+    }
+    __syncthreads();
+    // every non-zero counter is one distinct element: append (element, count) to the slot records
+    // and reset the counter for the next pass ...
+    for (uint32_t k4 = tid; k4 < FV_NB_CNT_WORDS / 4; k4 += T) {
+      const uint4 c4 = ((const uint4 *)cnt)[k4];
+      if ((c4.x | c4.y | c4.z | c4.w) == 0) continue;
+      ((uint4 *)cnt)[k4] = make_uint4(0, 0, 0, 0);
+      const uint32_t cw[4] = {c4.x, c4.y, c4.z, c4.w};
+      const uint32_t per = narrow ? 8 : 4;  // counters in this uint4
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (u >= (int)per) break;
+        const uint32_t c = narrow ? (cw[u >> 1] >> (16 * (u & 1))) & 0xffffu : cw[u];
+        if (c == 0) continue;
+        const uint32_t col = ((lo + k4 * per + u) << FV_NB_CLASS_SHIFT) | q;
+        const uint32_t e = atomicAdd(&sh_pos, 1u);
+        slots[e].p = col * a.ldk + h;
+        slots[e].n = c;
+      }
+    }
+    __syncthreads();
+    // ... then one element per thread: save its weight and plant the sentinel
+    const uint32_t end = sh_pos;
+    for (uint32_t eb = emitted + tid; eb < end; eb += 4 * T) {
+      uint32_t pe[4];
+      float wv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) pe[u] = slots[min(eb + u * T, end - 1)].p;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) wv[u] = a.Wt[pe[u]];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (eb + u * T < end) {
+          slots[eb + u * T].wv = wv[u];
+          a.Wt[pe[u]] = __uint_as_float(FV_SENTINEL);
+        }
+    }
+    emitted = end;
+    __syncthreads();
   }
+  for (uint32_t e = emitted + tid; e < m_ent; e += T) slots[e].p = FV_SLOT_INVALID;
 }
 
 // ---- kernels 3 and 4: dense passes over the matrix ------------------------------------------------
@@ -377,13 +423,19 @@ struct fv_dense_args {
   float4 *Wt4;
   const float *xx;
   const float *invf;
-  const fv_slot *slots;
-  const float *emax;
-  float *bmax;
+  const fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records, n_slots used in each
+  uint64_t slot_stride;
+  float *bmax;           // dense_blocks + slot_blocks block maxima of |ds|
   float *scalars;
-  uint32_t total4, ldk4, ldk, V, K, n_slots, slot_blocks, n_bmax;
+  uint32_t total4, ldk4, ldk, V, K, n_slots, slot_blocks, dense_blocks;
   float eps, prec, update_cut;
 };
+
+// Slot record of flat index e over the FV_NB_CLASSES regions (e < FV_NB_CLASSES * n_slots).
+__device__ __forceinline__ const fv_slot *fv_slot_at(const fv_dense_args &a, uint32_t e) {
+  const uint32_t region = e / a.n_slots;
+  return a.slots + (uint64_t)region * a.slot_stride + (e - region * a.n_slots);
+}
 
 __device__ __forceinline__ bool fv_is_sentinel(float w) { return __float_as_uint(w) == FV_SENTINEL; }
 
@@ -405,19 +457,32 @@ __global__ __launch_bounds__(256) void fv_absmax_kernel(fv_dense_args a) {
   __shared__ float smem4[4];
   for (uint32_t q = threadIdx.x; q < a.ldk4; q += 256) xs4[q] = ((const float4 *)a.xx)[q];
   __syncthreads();
-  const uint32_t stride = gridDim.x * 256;
-  const uint32_t dq = stride % a.ldk4;
-  uint32_t q = (blockIdx.x * 256 + threadIdx.x) % a.ldk4;
   float m = 0.0f;
-  for (uint32_t p4 = blockIdx.x * 256 + threadIdx.x; p4 < a.total4; p4 += stride) {
-    const float4 w = a.Wt4[p4];
-    const float4 x = xs4[q];
-    m = fv_absmax_keep(m, fv_dense_ds(x.x, w.x));
-    m = fv_absmax_keep(m, fv_dense_ds(x.y, w.y));
-    m = fv_absmax_keep(m, fv_dense_ds(x.z, w.z));
-    m = fv_absmax_keep(m, fv_dense_ds(x.w, w.w));
-    q += dq;
-    if (q >= a.ldk4) q -= a.ldk4;
+  if (blockIdx.x >= a.dense_blocks) {
+    // sparse elements: the dense term plus count additions of 1/f; a row with xx == 0 has ds == 0
+    const uint32_t e = (blockIdx.x - a.dense_blocks) * 256 + threadIdx.x;
+    if (e < FV_NB_CLASSES * a.n_slots) {
+      const fv_slot sl = *fv_slot_at(a, e);
+      if (sl.p != FV_SLOT_INVALID) {
+        const uint32_t i = sl.p / a.ldk, h = sl.p - i * a.ldk;
+        const float x = ((const float *)xs4)[h];
+        if (x != 0.0f) m = fv_absmax_keep(m, fv_sparse_ds(x, sl.wv, a.invf[i >= a.V ? i - a.V : i], sl.n));
+      }
+    }
+  } else {
+    const uint32_t stride = a.dense_blocks * 256;
+    const uint32_t dq = stride % a.ldk4;
+    uint32_t q = (blockIdx.x * 256 + threadIdx.x) % a.ldk4;
+    for (uint32_t p4 = blockIdx.x * 256 + threadIdx.x; p4 < a.total4; p4 += stride) {
+      const float4 w = a.Wt4[p4];
+      const float4 x = xs4[q];
+      m = fv_absmax_keep(m, fv_dense_ds(x.x, w.x));
+      m = fv_absmax_keep(m, fv_dense_ds(x.y, w.y));
+      m = fv_absmax_keep(m, fv_dense_ds(x.z, w.z));
+      m = fv_absmax_keep(m, fv_dense_ds(x.w, w.w));
+      q += dq;
+      if (q >= a.ldk4) q -= a.ldk4;
+    }
   }
   const float bm = fv_block_max_nonneg(m, smem4);
   if (threadIdx.x == 0) a.bmax[blockIdx.x] = bm;
@@ -428,10 +493,9 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
   __shared__ float smem4[4];
   __shared__ float sh_s;
   for (uint32_t q = threadIdx.x; q < a.ldk4; q += 256) xs4[q] = ((const float4 *)a.xx)[q];
-  // max|ds| = max over the dense block maxima and the per-neuron sparse maxima
+  // max|ds| = max over the block maxima of the dense and the sparse elements
   float nc = 0.0f;
-  for (uint32_t i = threadIdx.x; i < a.n_bmax; i += 256) nc = fmaxf(nc, a.bmax[i]);
-  for (uint32_t i = threadIdx.x; i < a.K; i += 256) nc = fmaxf(nc, a.emax[i]);
+  for (uint32_t i = threadIdx.x; i < a.dense_blocks + a.slot_blocks; i += 256) nc = fmaxf(nc, a.bmax[i]);
   nc = fv_block_max_nonneg(nc, smem4);
   if (threadIdx.x == 0) {
     sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
@@ -474,16 +538,19 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
 // update so no dense thread can mistake a finished element for an ordinary weight.
 __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
   const uint32_t e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= a.n_slots) return;
-  const fv_slot sl = a.slots[e];
+  if (e >= FV_NB_CLASSES * a.n_slots) return;
+  const fv_slot sl = *fv_slot_at(a, e);
   if (sl.p == FV_SLOT_INVALID) return;
-  const float nc = a.scalars[0];
-  const float s = a.prec > nc ? a.eps / a.prec : a.eps / nc;
   const uint32_t i = sl.p / a.ldk, h = sl.p - i * a.ldk;
-  const float f = a.invf[i >= a.V ? i - a.V : i];
-  const float v = fv_sparse_ds(a.xx[h], sl.wv, f, sl.n);
-  const float d = __fmul_rn(s, v);
-  ((float *)a.Wt4)[sl.p] = fabsf(d) > a.update_cut ? __fadd_rn(sl.wv, d) : sl.wv;
+  const float x = a.xx[h];
+  float out = sl.wv;  // a row with xx == 0 is not updated: the saved weight goes back
+  if (x != 0.0f) {
+    const float nc = a.scalars[0];
+    const float s = a.prec > nc ? a.eps / a.prec : a.eps / nc;
+    const float d = __fmul_rn(s, fv_sparse_ds(x, sl.wv, a.invf[i >= a.V ? i - a.V : i], sl.n));
+    if (fabsf(d) > a.update_cut) out = __fadd_rn(sl.wv, d);
+  }
+  ((float *)a.Wt4)[sl.p] = out;
 }
 
 // ---- row norms (log line of flyvec/src/cuda_funcs.cu:1234-1242) -------------------------------
@@ -523,9 +590,10 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   fv_trainer_free_corpus(t);
   (void)hipFree(t->Wt);
   (void)hipFree(t->idx);
-  (void)hipFree(t->order);
   (void)hipFree(t->slots);
-  (void)hipFree(t->emax);
+  (void)hipFree(t->order);
+  (void)hipFree(t->group_base);
+  (void)hipFree(t->group_count);
   (void)hipFree(t->bmax);
   (void)hipFree(t->win);
   (void)hipFree(t->sc);
@@ -541,24 +609,21 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipStreamCreate(&t->stream));
   FV_HIP(hipMalloc((void **)&t->Wt, elems * sizeof(float)));
   FV_HIP(hipMalloc((void **)&t->idx, (size_t)t->B * t->w * sizeof(int32_t)));
-  FV_HIP(hipMalloc((void **)&t->win, (size_t)t->B * sizeof(int32_t)));
+  FV_HIP(hipMalloc((void **)&t->win, ((size_t)t->B + 16) * sizeof(int32_t)));  // read in 16-byte pieces
   FV_HIP(hipMalloc((void **)&t->sc, (size_t)t->B * sizeof(float)));
   FV_HIP(hipMalloc((void **)&t->order, (size_t)t->B * sizeof(uint32_t)));
-  FV_HIP(hipMalloc((void **)&t->slots, (size_t)t->B * t->w * sizeof(fv_slot)));
+  FV_HIP(hipMalloc((void **)&t->group_base, (size_t)t->K * sizeof(uint32_t)));
+  FV_HIP(hipMalloc((void **)&t->group_count, (size_t)t->K * sizeof(uint32_t)));
+  FV_HIP(hipMalloc((void **)&t->slots, (size_t)FV_NB_CLASSES * t->B * t->w * sizeof(fv_slot)));
   FV_HIP(hipMalloc((void **)&t->xx, (size_t)t->ldk * sizeof(float)));
-  FV_HIP(hipMalloc((void **)&t->emax, (size_t)t->K * sizeof(float)));
-  FV_HIP(hipMalloc((void **)&t->bmax, (size_t)t->dense_blocks * sizeof(float)));
+  FV_HIP(hipMalloc((void **)&t->bmax,
+                   ((size_t)t->dense_blocks + ((size_t)FV_NB_CLASSES * t->B * t->w + 255) / 256) * sizeof(float)));
+  FV_HIP(hipMemsetAsync(t->win, 0, ((size_t)t->B + 16) * sizeof(int32_t), t->stream));
   FV_HIP(hipMalloc((void **)&t->scalars, 16 * sizeof(float)));
   FV_HIP(hipMemsetAsync(t->Wt, 0, elems * sizeof(float), t->stream));
   FV_HIP(hipMemsetAsync(t->xx, 0, (size_t)t->ldk * sizeof(float), t->stream));
   FV_HIP(hipMemsetAsync(t->scalars, 0, 16 * sizeof(float), t->stream));
   FV_HIP(hipStreamSynchronize(t->stream));
-  // the neuron kernel counts column indices in LDS: as much of the column range per pass as fits
-  uint32_t chunk = (uint32_t)((t->N + 255) / 256 * 256);
-  if (chunk > FV_NB_MAX_CHUNK) chunk = FV_NB_MAX_CHUNK;
-  t->nb_chunk = chunk;
-  FV_HIP(hipFuncSetAttribute((const void *)fv_neuron_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                             (int)(chunk * sizeof(uint32_t))));
   return FV_OK;
 }
 
@@ -766,6 +831,7 @@ extern "C" int fv_trainer_get_permutation(fv_trainer *t, uint64_t *out_perm, uin
   return FV_OK;
 }
 
+
 template <int NV>
 static void fv_launch_gather(const fv_gather_args &a, hipStream_t stream) {
   hipLaunchKernelGGL(fv_gather_winner_kernel<NV>, dim3((a.n + 3) / 4), dim3(256), 0, stream, a);
@@ -802,31 +868,37 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
       return fv_fail(FV_ERR_INVALID, "hid = %u not supported", t->K);
   }
   if (ev) FV_HIP(hipEventRecord(ev[1], t->stream));
-  fv_neuron_args nb;
-  nb.win = t->win;
-  nb.sc = t->sc;
-  nb.idx = t->idx;
-  nb.invf = t->invf;
-  nb.Wt = t->Wt;
-  nb.xx = t->xx;
-  nb.emax = t->emax;
-  nb.order = t->order;
-  nb.slots = t->slots;
-  nb.chunk = t->nb_chunk;
-  nb.n = n;
-  nb.K = t->K;
-  nb.ldk = t->ldk;
-  nb.w = t->w;
-  nb.V = (uint32_t)t->V;
-  hipLaunchKernelGGL(fv_neuron_kernel, dim3(t->K), dim3(FV_NB_THREADS), t->nb_chunk * sizeof(uint32_t),
-                     t->stream, nb);
+  fv_group_args gr;
+  gr.win = t->win;
+  gr.sc = t->sc;
+  gr.order = t->order;
+  gr.group_base = t->group_base;
+  gr.group_count = t->group_count;
+  gr.xx = t->xx;
+  gr.n = n;
+  // a thread's run of the winner array should fit its 64-bit match mask
+  const unsigned gr_threads = n <= 16384 ? 256 : FV_NB_MAX_THREADS;
+  hipLaunchKernelGGL(fv_group_kernel, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
   if (ev) FV_HIP(hipEventRecord(ev[2], t->stream));
+  fv_sparse_args sp;
+  sp.order = t->order;
+  sp.group_base = t->group_base;
+  sp.group_count = t->group_count;
+  sp.idx = t->idx;
+  sp.Wt = t->Wt;
+  sp.slots = t->slots;
+  sp.slot_stride = (uint64_t)t->B * t->w;
+  sp.ldk = t->ldk;
+  sp.w = t->w;
+  sp.V = (uint32_t)t->V;
+  hipLaunchKernelGGL(fv_sparse_kernel, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, sp);
+  if (ev) FV_HIP(hipEventRecord(ev[3], t->stream));
   fv_dense_args d;
   d.Wt4 = (float4 *)t->Wt;
   d.xx = t->xx;
   d.invf = t->invf;
   d.slots = t->slots;
-  d.emax = t->emax;
+  d.slot_stride = (uint64_t)t->B * t->w;
   d.bmax = t->bmax;
   d.scalars = t->scalars;
   d.total4 = t->total4;
@@ -835,18 +907,18 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.V = (uint32_t)t->V;
   d.K = t->K;
   d.n_slots = n * t->w;
-  d.slot_blocks = (d.n_slots + 255) / 256;
-  d.n_bmax = t->dense_blocks;
+  d.slot_blocks = (FV_NB_CLASSES * d.n_slots + 255) / 256;
+  d.dense_blocks = t->dense_blocks;
   d.eps = eps;
   d.prec = t->cfg.prec;
   d.update_cut = t->update_cut;
   const size_t smem = (size_t)t->ldk * sizeof(float);
-  hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
-  if (ev) FV_HIP(hipEventRecord(ev[3], t->stream));
-  hipLaunchKernelGGL(fv_update_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
+  hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks + d.slot_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
-  hipLaunchKernelGGL(fv_slot_update_kernel, dim3(d.slot_blocks), dim3(256), 0, t->stream, d);
+  hipLaunchKernelGGL(fv_update_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
+  hipLaunchKernelGGL(fv_slot_update_kernel, dim3(d.slot_blocks), dim3(256), 0, t->stream, d);
+  if (ev) FV_HIP(hipEventRecord(ev[6], t->stream));
   FV_HIP(hipGetLastError());
   t->last_n = n;
   return FV_OK;

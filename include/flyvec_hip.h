@@ -148,7 +148,7 @@ int fv_trainer_row_norms(fv_trainer *t, uint32_t n_rows, double *out_norms);
  * events on the trainer's stream. out_total_ms covers all steps; out_kernel_ms[FV_TRAIN_KERNELS]
  * (nullable) receives the mean duration of each kernel of the step, measured in a second,
  * separately instrumented run of the same steps. */
-#define FV_TRAIN_KERNELS 5 /* gather+winner, neuron owners (xx + sparse term), max|ds|, update, sparse update */
+#define FV_TRAIN_KERNELS 6 /* gather+winner, group by winner + xx, sparse owners, max|ds|, update, sparse update */
 int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint32_t n_steps, float eps,
                           float *out_total_ms, float *out_kernel_ms);
 
