@@ -34,6 +34,22 @@ TRAIN = dict(K=400, V=20000, w=11, B=10000, n_tokens=10_000_000, lr0=2e-4, n_epo
 HASH = dict(K=400, V=20000, w=11, k=32, n=1 << 20)
 
 
+# HBM-side bytes per launch at the headline configuration, from two rocprofv3 --pmc runs of this
+# script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter reads
+# for the plain copy kernel of --copy-calibration (FETCH_SIZE reads half the bytes copied: x2.0;
+# WRITE_SIZE reads them all: x1.0). Traffic below the algorithmic bytes means the rest was served
+# by the L2 caches.
+MEASURED_TRAFFIC = {
+    "update": (31328.5 * 2.0 + 62725.3) * 1024,
+    "absmax_ds": (34152.6 * 2.0 + 117.7) * 1024,
+    "gather_winner": (27205.2 * 2.0 + 625.1) * 1024,
+    "sparse_owners": (4603.9 * 2.0 + 6682.3) * 1024,
+    "group_xx": (398.1 * 2.0 + 87.1) * 1024,
+    "slot_update": (2891.1 * 2.0 + 1638.2) * 1024,
+    "hash": (2245614.6 * 2.0 + 78862.5) * 1024,
+}
+
+
 def train_bytes(K, N, w, B):
     """Algorithmic HBM bytes per step and per kernel: every window gathers w rows of K floats once;
     W is read once for max|ds| and read + written once by the update; ds is never stored; token
@@ -78,9 +94,13 @@ def bench_train(steps, warmup, cpu_seconds):
         t.step((warmup + s) * c["B"], c["B"], eps)
     t.sync()
     wall = time.perf_counter() - t0
-    # per-kernel durations (HIP events between the kernels) on the following `steps` steps
-    total_ms, kern_ms = t.time_steps((warmup + steps) * c["B"], steps, eps)
+    # the same number of steps again, timed by two HIP events on the trainer's stream
+    total_ms, _ = t.time_steps((warmup + steps) * c["B"], steps, eps, per_kernel=False)
     ev_ms_per_step = total_ms / steps
+    # per-kernel durations: each kernel of the last step launched back to back between two HIP
+    # events on that stream (bracketing every kernel inside a step would add ~3 us of event
+    # overhead to each); this destroys W, so it comes last
+    kern_ms = t.time_kernels(reps=50)
     t.close()
 
     N = 2 * c["V"]
@@ -94,7 +114,7 @@ def bench_train(steps, warmup, cpu_seconds):
         "event_ms_per_step": ev_ms_per_step,
         "kernel_ms": kern_ms,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": None,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": MEASURED_TRAFFIC.get(dom),
                      "algorithmic_bytes": per_kernel[dom]},
         "step_roofline_frac": (step_bytes / HBM_PEAK) / (ms_per_step * 1e-3),
         "step_algorithmic_bytes": step_bytes,
@@ -138,7 +158,7 @@ def bench_hash(reps, cpu_seconds):
                                   f"n={c['n']} windows, 7 uint64 words out"},
            "dtype": "f32",
            "roofline": {"bound": "hbm", "kernel": "hash", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
-                        "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": None,
+                        "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": MEASURED_TRAFFIC["hash"],
                         "algorithmic_bytes": bpw * c["n"]}}
     if cpu_seconds > 0:
         from oracle import hash_oracle as ho
@@ -170,6 +190,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample length (0 = skip)")
     ap.add_argument("--no-hash", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB copy kernel (yardstick for rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
@@ -197,6 +219,11 @@ def main():
         line["cpu_baseline"] = tr["cpu_baseline"]
     if not args.no_hash:
         line["hash"] = bench_hash(reps=10, cpu_seconds=min(args.cpu_seconds, 5.0))
+    if args.copy_calibration:
+        nbytes = 1 << 30
+        ms = _lib.calibration_copy(nbytes, reps=5)
+        line["copy_calibration"] = {"bytes_read": nbytes, "bytes_written": nbytes, "ms": ms,
+                                    "GB/s": 2 * nbytes / (ms * 1e-3) / 1e9}
     print(json.dumps(line))
 
 

@@ -53,6 +53,7 @@ SIGNATURES = {
     "fv_dev_free": [_vp],
     "fv_dev_upload": [_vp, _vp, C.c_size_t],
     "fv_dev_download": [_vp, _vp, C.c_size_t],
+    "fv_calibration_copy": [C.c_size_t, _u32, C.POINTER(_f32)],
     "fv_count_windows": [_vp, _u64, _u64, C.POINTER(_u64)],
     "fv_build_window_starts": [_vp, _u64, _u64, _vp, _u64],
     "fv_inverse_frequency": [_vp, _u64, _u64, _vp],
@@ -75,6 +76,7 @@ SIGNATURES = {
     "fv_trainer_get_step_stats": [_vp, _vp, C.POINTER(_f32)],
     "fv_trainer_row_norms": [_vp, _u32, _vp],
     "fv_trainer_time_steps": [_vp, _u64, _u32, _f32, C.POINTER(_f32), C.POINTER(_f32)],
+    "fv_trainer_time_kernel": [_vp, _u32, _u32, C.POINTER(_f32)],
     "fv_hasher_create": [_vp, _u32, _u64, _pp],
     "fv_hasher_destroy": [_vp],
     "fv_hasher_normalize": [_vp, _f32],
@@ -132,6 +134,13 @@ def device_info():
     mem = C.c_uint64(0)
     check(load().fv_device_info(name, 256, C.byref(cus), C.byref(mem)))
     return {"name": name.value.decode(), "compute_units": cus.value, "hbm_bytes": mem.value}
+
+
+def calibration_copy(nbytes, reps=5):
+    """Mean milliseconds of a plain copy kernel reading and writing nbytes each."""
+    ms = C.c_float(0)
+    check(load().fv_calibration_copy(int(nbytes), int(reps), C.byref(ms)))
+    return ms.value
 
 
 class DeviceBuffer:

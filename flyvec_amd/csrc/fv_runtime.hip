@@ -189,3 +189,43 @@ int fv_download_weights(const float *Wt_dev, float *W_host, uint32_t K, uint64_t
   (void)hipFree(stage);
   return rc;
 }
+
+// ---- calibration copy -------------------------------------------------------------------------------
+// A plain streaming copy of known size: the yardstick hardware byte counters are scaled by, and a
+// measured ceiling for this machine's copy bandwidth.
+
+__global__ __launch_bounds__(256) void fv_calibration_copy_kernel(const float4 *__restrict__ src,
+                                                                  float4 *__restrict__ dst, uint64_t n4) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (uint64_t)gridDim.x * 256)
+    dst[i] = src[i];
+}
+
+extern "C" int fv_calibration_copy(size_t bytes, uint32_t reps, float *out_mean_ms) {
+  FV_REQUIRE(bytes >= 16 && reps >= 1 && out_mean_ms, FV_ERR_INVALID, "fv_calibration_copy: bad arguments");
+  const uint64_t n4 = bytes / 16;
+  float4 *src = nullptr, *dst = nullptr;
+  FV_HIP(hipMalloc((void **)&src, n4 * 16));
+  hipError_t e = hipMalloc((void **)&dst, n4 * 16);
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (e == hipSuccess) e = hipMemset(src, 1, n4 * 16);
+  if (e == hipSuccess) e = hipEventCreate(&e0);
+  if (e == hipSuccess) e = hipEventCreate(&e1);
+  if (e == hipSuccess) {
+    const unsigned blocks = 256 * 8;
+    hipLaunchKernelGGL(fv_calibration_copy_kernel, dim3(blocks), dim3(256), 0, 0, src, dst, n4);  // warm-up
+    e = hipEventRecord(e0, 0);
+    for (uint32_t r = 0; r < reps; ++r)
+      hipLaunchKernelGGL(fv_calibration_copy_kernel, dim3(blocks), dim3(256), 0, 0, src, dst, n4);
+    if (e == hipSuccess) e = hipEventRecord(e1, 0);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    *out_mean_ms = ms / (float)reps;
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipFree(src);
+  (void)hipFree(dst);
+  if (e != hipSuccess) return fv_fail(FV_ERR_HIP, "calibration copy failed: %s", hipGetErrorString(e));
+  return FV_OK;
+}

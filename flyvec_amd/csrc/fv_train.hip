@@ -67,6 +67,8 @@ struct fv_trainer {
   float *bmax;      // max|ds| of each dense block and each slot block of the absmax launch
   float *scalars;   // [0] max|ds| of the last step
   uint32_t last_n;
+  uint64_t last_first;
+  float last_eps;
   uint64_t shuffle_calls;
   bool have_corpus, have_weights;
   unsigned dense_blocks;
@@ -837,9 +839,10 @@ static void fv_launch_gather(const fv_gather_args &a, hipStream_t stream) {
   hipLaunchKernelGGL(fv_gather_winner_kernel<NV>, dim3((a.n + 3) / 4), dim3(256), 0, stream, a);
 }
 
-// Enqueues the kernels of one step; ev (nullable) receives FV_TRAIN_KERNELS + 1 events recorded
-// around them.
-static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps, hipEvent_t *ev) {
+// Enqueues the kernels of one step (those whose bit is set in `which`); ev (nullable) receives
+// FV_TRAIN_KERNELS + 1 events recorded around them.
+static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps, hipEvent_t *ev,
+                           unsigned which = 0x3f) {
   fv_gather_args g;
   g.Wt = t->Wt;
   g.corpus = t->corpus;
@@ -857,7 +860,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.V = (uint32_t)t->V;
   g.tie_rule = t->cfg.tie_rule;
   if (ev) FV_HIP(hipEventRecord(ev[0], t->stream));
-  switch ((t->K + 63) / 64) {
+  if (which & 1u) switch ((t->K + 63) / 64) {
 #define FV_CASE(NV) case NV: fv_launch_gather<NV>(g, t->stream); break;
     FV_CASE(1) FV_CASE(2) FV_CASE(3) FV_CASE(4) FV_CASE(5) FV_CASE(6) FV_CASE(7) FV_CASE(8)
     FV_CASE(9) FV_CASE(10) FV_CASE(11) FV_CASE(12) FV_CASE(13) FV_CASE(14) FV_CASE(15) FV_CASE(16)
@@ -878,7 +881,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   gr.n = n;
   // a thread's run of the winner array should fit its 64-bit match mask
   const unsigned gr_threads = n <= 16384 ? 256 : FV_NB_MAX_THREADS;
-  hipLaunchKernelGGL(fv_group_kernel, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
+  if (which & 2u) hipLaunchKernelGGL(fv_group_kernel, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
   if (ev) FV_HIP(hipEventRecord(ev[2], t->stream));
   fv_sparse_args sp;
   sp.order = t->order;
@@ -891,7 +894,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.ldk = t->ldk;
   sp.w = t->w;
   sp.V = (uint32_t)t->V;
-  hipLaunchKernelGGL(fv_sparse_kernel, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, sp);
+  if (which & 4u) hipLaunchKernelGGL(fv_sparse_kernel, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, sp);
   if (ev) FV_HIP(hipEventRecord(ev[3], t->stream));
   fv_dense_args d;
   d.Wt4 = (float4 *)t->Wt;
@@ -913,14 +916,17 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.prec = t->cfg.prec;
   d.update_cut = t->update_cut;
   const size_t smem = (size_t)t->ldk * sizeof(float);
-  hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks + d.slot_blocks), dim3(256), smem, t->stream, d);
+  if (which & 8u)
+    hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks + d.slot_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
-  hipLaunchKernelGGL(fv_update_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
+  if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
-  hipLaunchKernelGGL(fv_slot_update_kernel, dim3(d.slot_blocks), dim3(256), 0, t->stream, d);
+  if (which & 32u) hipLaunchKernelGGL(fv_slot_update_kernel, dim3(d.slot_blocks), dim3(256), 0, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[6], t->stream));
   FV_HIP(hipGetLastError());
   t->last_n = n;
+  t->last_first = first;
+  t->last_eps = eps;
   return FV_OK;
 }
 
@@ -1044,5 +1050,27 @@ extern "C" int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint3
       }
   }
   for (auto &e : ev) (void)hipEventDestroy(e);
+  return rc;
+}
+
+extern "C" int fv_trainer_time_kernel(fv_trainer *t, uint32_t kernel_index, uint32_t reps, float *out_mean_ms) {
+  FV_REQUIRE(t && out_mean_ms, FV_ERR_INVALID, "null argument");
+  FV_REQUIRE(kernel_index < FV_TRAIN_KERNELS && reps >= 1, FV_ERR_INVALID, "bad kernel index or repetition count");
+  FV_REQUIRE(t->last_n > 0, FV_ERR_STATE, "no step has run yet");
+  hipEvent_t e0, e1;
+  FV_HIP(hipEventCreate(&e0));
+  FV_HIP(hipEventCreate(&e1));
+  FV_HIP(hipStreamSynchronize(t->stream));
+  int rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, nullptr, 1u << kernel_index);  // warm-up
+  FV_HIP(hipEventRecord(e0, t->stream));
+  for (uint32_t r = 0; r < reps && rc == FV_OK; ++r)
+    rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, nullptr, 1u << kernel_index);
+  FV_HIP(hipEventRecord(e1, t->stream));
+  FV_HIP(hipStreamSynchronize(t->stream));
+  float ms = 0.0f;
+  FV_HIP(hipEventElapsedTime(&ms, e0, e1));
+  *out_mean_ms = ms / (float)reps;
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
   return rc;
 }

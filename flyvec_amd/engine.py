@@ -152,6 +152,17 @@ class Trainer:
         return total.value, dict(zip(_lib.TRAIN_KERNEL_NAMES, list(kern))) if per_kernel else None
 
 
+    def _time_kernel(self, index, reps):
+        ms = C.c_float(0)
+        check(self.lib.fv_trainer_time_kernel(self.handle, index, reps, C.byref(ms)))
+        return ms.value
+
+    def time_kernels(self, reps=20):
+        """Mean duration (ms) of each kernel of the last step, launched back to back `reps` times.
+        Leaves W good for timing only."""
+        return {name: self._time_kernel(i, reps) for i, name in enumerate(_lib.TRAIN_KERNEL_NAMES)}
+
+
 class Hasher:
     """A checkpoint matrix resident in HBM plus the batched top-k threshold code."""
 

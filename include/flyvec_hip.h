@@ -55,6 +55,11 @@ int fv_dev_free(void *dev_ptr);
 int fv_dev_upload(void *dst_dev, const void *src_host, size_t bytes);
 int fv_dev_download(void *dst_host, const void *src_dev, size_t bytes);
 
+/* Measurement: `reps` launches of a plain device-to-device copy kernel moving `bytes` (read) +
+ * `bytes` (written); mean duration by HIP events. The yardstick for hardware byte counters. No
+ * counterpart in the reference. */
+int fv_calibration_copy(size_t bytes, uint32_t reps, float *out_mean_ms);
+
 /* ---- window sampler, host half ------------------------------------------------ */
 
 /* flyvec/src/prune_input.cpp:64 getnum_samples: number of length-w windows that do not
@@ -151,6 +156,12 @@ int fv_trainer_row_norms(fv_trainer *t, uint32_t n_rows, double *out_norms);
 #define FV_TRAIN_KERNELS 6 /* gather+winner, group by winner + xx, sparse owners, max|ds|, update, sparse update */
 int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint32_t n_steps, float eps,
                           float *out_total_ms, float *out_kernel_ms);
+
+/* Measurement: launches kernel `kernel_index` (0 .. FV_TRAIN_KERNELS-1) of the last step `reps`
+ * times back to back on its buffers and returns the mean duration between two HIP events on the
+ * trainer's stream. The kernels that write W are not idempotent: the matrix is left in a state
+ * that is only good for timing, so install weights again before training on. */
+int fv_trainer_time_kernel(fv_trainer *t, uint32_t kernel_index, uint32_t reps, float *out_mean_ms);
 
 /* ---- hashing ------------------------------------------------------------------ */
 
