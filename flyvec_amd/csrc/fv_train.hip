@@ -64,14 +64,15 @@ struct fv_trainer {
   uint32_t *group_base, *group_count;  // K each
   fv_slot *slots;   // FV_NB_CLASSES regions of B x w slot records
   float *xx;        // ldk
-  float *bmax;      // max|ds| of each dense block and each slot block of the absmax launch
+  float *bmax;      // max|ds| of each block of the absmax launch, then of each block of the sparse launch
   float *scalars;   // [0] max|ds| of the last step
   uint32_t last_n;
   uint64_t last_first;
   float last_eps;
   uint64_t shuffle_calls;
   bool have_corpus, have_weights;
-  unsigned dense_blocks;
+  unsigned dense_blocks;   // blocks of the absmax launch
+  unsigned update_blocks;  // blocks of the dense update launch
   float update_cut;  // largest fp32 <= 1e-10
 };
 
@@ -188,6 +189,15 @@ __device__ __forceinline__ float fv_sparse_ds(float xx, float wv, float f, uint3
 __device__ __forceinline__ float fv_absmax_keep(float m, float v) {
   const float a = fabsf(v);
   return a > m ? a : m;  // a NaN never replaces m, as in the reference's comparison
+}
+
+// Block-wide maximum of non-negative floats; result valid in thread 0.
+__device__ __forceinline__ float fv_block_max_nonneg(float m, float *smem4) {
+  const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) smem4[threadIdx.x >> 6] = __uint_as_float(wm);
+  __syncthreads();
+  return fmaxf(fmaxf(smem4[0], smem4[1]), fmaxf(smem4[2], smem4[3]));
 }
 
 // Sum over the block of one value per thread (result in every thread).
@@ -320,6 +330,9 @@ struct fv_sparse_args {
   float *Wt;
   fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records
   uint64_t slot_stride;
+  const float *xx;
+  const float *invf;
+  float *bmax_sparse;  // one maximum of |ds| per block
   uint32_t ldk, w, V;
 };
 
@@ -331,8 +344,13 @@ __global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
   const uint32_t q = blockIdx.x & (FV_NB_CLASSES - 1);
   const uint32_t tid = threadIdx.x;
   const uint32_t c_h = a.group_count[h];
-  if (c_h == 0) return;
+  if (c_h == 0) {
+    if (tid == 0) a.bmax_sparse[blockIdx.x] = 0.0f;
+    return;
+  }
   const uint32_t base = a.group_base[h];
+  const float x_h = a.xx[h];
+  float ds_max = 0.0f;
   const uint32_t *__restrict__ order = a.order + base;
   const int32_t *__restrict__ idx = a.idx;
   const uint32_t n_cols = 2 * a.V;
@@ -397,26 +415,38 @@ __global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
       }
     }
     __syncthreads();
-    // ... then one element per thread: save its weight and plant the sentinel
+    // ... then one element per thread: save its weight, plant the sentinel, and take |ds| of the
+    // element (the dense term plus count additions of 1/f; a row with xx == 0 has ds == 0)
     const uint32_t end = sh_pos;
     for (uint32_t eb = emitted + tid; eb < end; eb += 4 * T) {
-      uint32_t pe[4];
-      float wv[4];
+      uint32_t pe[4], ne[4];
+      float wv[4], fe[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) pe[u] = slots[min(eb + u * T, end - 1)].p;
+      for (int u = 0; u < 4; ++u) {
+        const fv_slot *sl = &slots[min(eb + u * T, end - 1)];
+        pe[u] = sl->p;
+        ne[u] = sl->n;
+      }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) wv[u] = a.Wt[pe[u]];
+      for (int u = 0; u < 4; ++u) {
+        wv[u] = a.Wt[pe[u]];
+        const uint32_t col = pe[u] / a.ldk;
+        fe[u] = a.invf[col >= a.V ? col - a.V : col];
+      }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
         if (eb + u * T < end) {
           slots[eb + u * T].wv = wv[u];
           a.Wt[pe[u]] = __uint_as_float(FV_SENTINEL);
+          if (x_h != 0.0f) ds_max = fv_absmax_keep(ds_max, fv_sparse_ds(x_h, wv[u], fe[u], ne[u]));
         }
     }
     emitted = end;
     __syncthreads();
   }
   for (uint32_t e = emitted + tid; e < m_ent; e += T) slots[e].p = FV_SLOT_INVALID;
+  const float bm = fv_block_max_nonneg(ds_max, (float *)cnt);
+  if (tid == 0) a.bmax_sparse[blockIdx.x] = bm;
 }
 
 // ---- kernels 3 and 4: dense passes over the matrix ------------------------------------------------
@@ -427,9 +457,9 @@ struct fv_dense_args {
   const float *invf;
   const fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records, n_slots used in each
   uint64_t slot_stride;
-  float *bmax;           // dense_blocks + slot_blocks block maxima of |ds|
+  float *bmax;           // n_bmax block maxima of |ds|: dense blocks, then the sparse kernel's blocks
   float *scalars;
-  uint32_t total4, ldk4, ldk, V, K, n_slots, slot_blocks, dense_blocks;
+  uint32_t total4, ldk4, ldk, V, K, n_slots, n_bmax, dense_blocks;
   float eps, prec, update_cut;
 };
 
@@ -445,59 +475,112 @@ __device__ __forceinline__ float fv_dense_ds(float x, float w) {
   return (x != 0.0f && !fv_is_sentinel(w)) ? __fmul_rn(-x, w) : 0.0f;
 }
 
-// Block-wide maximum of non-negative floats; result valid in thread 0.
-__device__ __forceinline__ float fv_block_max_nonneg(float m, float *smem4) {
-  const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) smem4[threadIdx.x >> 6] = __uint_as_float(wm);
-  __syncthreads();
-  return fmaxf(fmaxf(smem4[0], smem4[1]), fmaxf(smem4[2], smem4[3]));
+// W += s * ds on four consecutive dense elements (flyvec/src/cuda_funcs.cu:1800-1803): an element
+// changes only where |s * ds| exceeds the cut; sentinel positions belong to the slot kernel.
+__device__ __forceinline__ void fv_update_four(const fv_dense_args &a, uint32_t p4, float4 w, const float4 x,
+                                               const float s) {
+  const bool s0 = fv_is_sentinel(w.x), s1 = fv_is_sentinel(w.y), s2 = fv_is_sentinel(w.z),
+             s3 = fv_is_sentinel(w.w);
+  bool c0 = false, c1 = false, c2 = false, c3 = false;
+  float d;
+  d = __fmul_rn(s, fv_dense_ds(x.x, w.x)); if (fabsf(d) > a.update_cut) { w.x = __fadd_rn(w.x, d); c0 = true; }
+  d = __fmul_rn(s, fv_dense_ds(x.y, w.y)); if (fabsf(d) > a.update_cut) { w.y = __fadd_rn(w.y, d); c1 = true; }
+  d = __fmul_rn(s, fv_dense_ds(x.z, w.z)); if (fabsf(d) > a.update_cut) { w.z = __fadd_rn(w.z, d); c2 = true; }
+  d = __fmul_rn(s, fv_dense_ds(x.w, w.w)); if (fabsf(d) > a.update_cut) { w.w = __fadd_rn(w.w, d); c3 = true; }
+  if (s0 | s1 | s2 | s3) {
+    // store the other components one by one
+    float *wp = (float *)&a.Wt4[p4];
+    if (c0) wp[0] = w.x;
+    if (c1) wp[1] = w.y;
+    if (c2) wp[2] = w.z;
+    if (c3) wp[3] = w.w;
+  } else if (c0 | c1 | c2 | c3) {
+    a.Wt4[p4] = w;
+  }
 }
 
+// 16-byte loads a thread of a dense pass has in flight, and the blocks per compute unit of its launch
+#ifndef FV_ABSMAX_UNROLL
+#define FV_ABSMAX_UNROLL 2
+#endif
+#ifndef FV_UPDATE_UNROLL
+#define FV_UPDATE_UNROLL 8
+#endif
+#ifndef FV_ABSMAX_BLOCKS_PER_CU
+#define FV_ABSMAX_BLOCKS_PER_CU 8
+#endif
+#ifndef FV_UPDATE_BLOCKS_PER_CU
+#define FV_UPDATE_BLOCKS_PER_CU 8
+#endif
+
+// Batch u of a thread's elements: 16-byte group p4 + u * stride, clamped so that the load is
+// unconditional; a group past the end is loaded but not used.
+template <int U>
+__device__ __forceinline__ void fv_dense_load(const fv_dense_args &a, uint32_t p4, uint32_t stride, float4 (&w)[U]) {
+#pragma unroll
+  for (int u = 0; u < U; ++u) w[u] = a.Wt4[min(p4 + u * stride, a.total4 - 1)];
+}
+
+// Kernel 4: block maxima of |ds| over the dense elements. A thread's first loads of W
+// are issued before the block stages xx in LDS.
 __global__ __launch_bounds__(256) void fv_absmax_kernel(fv_dense_args a) {
   extern __shared__ float4 xs4[];  // xx, ldk4 float4
   __shared__ float smem4[4];
-  for (uint32_t q = threadIdx.x; q < a.ldk4; q += 256) xs4[q] = ((const float4 *)a.xx)[q];
+  const uint32_t stride = gridDim.x * 256;
+  const uint32_t dq = stride % a.ldk4;
+  uint32_t p4 = blockIdx.x * 256 + threadIdx.x;
+  uint32_t q = p4 % a.ldk4;
+  float4 w[FV_ABSMAX_UNROLL];
+  fv_dense_load(a, p4, stride, w);
+  for (uint32_t i = threadIdx.x; i < a.ldk4; i += 256) xs4[i] = ((const float4 *)a.xx)[i];
   __syncthreads();
   float m = 0.0f;
-  if (blockIdx.x >= a.dense_blocks) {
-    // sparse elements: the dense term plus count additions of 1/f; a row with xx == 0 has ds == 0
-    const uint32_t e = (blockIdx.x - a.dense_blocks) * 256 + threadIdx.x;
-    if (e < FV_NB_CLASSES * a.n_slots) {
-      const fv_slot sl = *fv_slot_at(a, e);
-      if (sl.p != FV_SLOT_INVALID) {
-        const uint32_t i = sl.p / a.ldk, h = sl.p - i * a.ldk;
-        const float x = ((const float *)xs4)[h];
-        if (x != 0.0f) m = fv_absmax_keep(m, fv_sparse_ds(x, sl.wv, a.invf[i >= a.V ? i - a.V : i], sl.n));
+  while (p4 < a.total4) {
+#pragma unroll
+    for (int u = 0; u < FV_ABSMAX_UNROLL; ++u) {
+      if (p4 + u * stride < a.total4) {
+        const float4 x = xs4[q];
+        m = fv_absmax_keep(m, fv_dense_ds(x.x, w[u].x));
+        m = fv_absmax_keep(m, fv_dense_ds(x.y, w[u].y));
+        m = fv_absmax_keep(m, fv_dense_ds(x.z, w[u].z));
+        m = fv_absmax_keep(m, fv_dense_ds(x.w, w[u].w));
       }
-    }
-  } else {
-    const uint32_t stride = a.dense_blocks * 256;
-    const uint32_t dq = stride % a.ldk4;
-    uint32_t q = (blockIdx.x * 256 + threadIdx.x) % a.ldk4;
-    for (uint32_t p4 = blockIdx.x * 256 + threadIdx.x; p4 < a.total4; p4 += stride) {
-      const float4 w = a.Wt4[p4];
-      const float4 x = xs4[q];
-      m = fv_absmax_keep(m, fv_dense_ds(x.x, w.x));
-      m = fv_absmax_keep(m, fv_dense_ds(x.y, w.y));
-      m = fv_absmax_keep(m, fv_dense_ds(x.z, w.z));
-      m = fv_absmax_keep(m, fv_dense_ds(x.w, w.w));
       q += dq;
       if (q >= a.ldk4) q -= a.ldk4;
     }
+    p4 += FV_ABSMAX_UNROLL * stride;
+    if (p4 < a.total4) fv_dense_load(a, p4, stride, w);
   }
   const float bm = fv_block_max_nonneg(m, smem4);
   if (threadIdx.x == 0) a.bmax[blockIdx.x] = bm;
 }
 
+// Kernel 5: max|ds| from the block maxima, then W += (eps / max|ds|) * ds over the dense elements.
+// The first loads of W are in flight while the block reduces the maxima.
 __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
   extern __shared__ float4 xs4[];
   __shared__ float smem4[4];
   __shared__ float sh_s;
-  for (uint32_t q = threadIdx.x; q < a.ldk4; q += 256) xs4[q] = ((const float4 *)a.xx)[q];
-  // max|ds| = max over the block maxima of the dense and the sparse elements
+  const uint32_t stride = gridDim.x * 256;
+  const uint32_t dq = stride % a.ldk4;
+  uint32_t p4 = blockIdx.x * 256 + threadIdx.x;
+  uint32_t q = p4 % a.ldk4;
+  float4 w[FV_UPDATE_UNROLL];
+  fv_dense_load(a, p4, stride, w);
+  for (uint32_t i = threadIdx.x; i < a.ldk4; i += 256) xs4[i] = ((const float4 *)a.xx)[i];
   float nc = 0.0f;
-  for (uint32_t i = threadIdx.x; i < a.dense_blocks + a.slot_blocks; i += 256) nc = fmaxf(nc, a.bmax[i]);
+  {
+    const uint32_t n4 = a.n_bmax / 4;
+    const float4 *b4 = (const float4 *)a.bmax;
+    for (uint32_t i = threadIdx.x; i < n4; i += 4 * 256) {  // four 16-byte loads together
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = b4[min(i + u * 256, n4 - 1)];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) nc = fmaxf(nc, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
+    }
+    for (uint32_t i = 4 * n4 + threadIdx.x; i < a.n_bmax; i += 256) nc = fmaxf(nc, a.bmax[i]);
+  }
   nc = fv_block_max_nonneg(nc, smem4);
   if (threadIdx.x == 0) {
     sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
@@ -505,38 +588,19 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
   }
   __syncthreads();
   const float s = sh_s;
-
-  const uint32_t bid = blockIdx.x;
-  const uint32_t stride = gridDim.x * 256;
-  const uint32_t dq = stride % a.ldk4;
-  uint32_t q = (bid * 256 + threadIdx.x) % a.ldk4;
-  for (uint32_t p4 = bid * 256 + threadIdx.x; p4 < a.total4; p4 += stride) {
-    float4 w = a.Wt4[p4];
-    const float4 x = xs4[q];
-    const bool s0 = fv_is_sentinel(w.x), s1 = fv_is_sentinel(w.y), s2 = fv_is_sentinel(w.z),
-               s3 = fv_is_sentinel(w.w);
-    bool c0 = false, c1 = false, c2 = false, c3 = false;
-    float d;
-    d = __fmul_rn(s, fv_dense_ds(x.x, w.x)); if (fabsf(d) > a.update_cut) { w.x = __fadd_rn(w.x, d); c0 = true; }
-    d = __fmul_rn(s, fv_dense_ds(x.y, w.y)); if (fabsf(d) > a.update_cut) { w.y = __fadd_rn(w.y, d); c1 = true; }
-    d = __fmul_rn(s, fv_dense_ds(x.z, w.z)); if (fabsf(d) > a.update_cut) { w.z = __fadd_rn(w.z, d); c2 = true; }
-    d = __fmul_rn(s, fv_dense_ds(x.w, w.w)); if (fabsf(d) > a.update_cut) { w.w = __fadd_rn(w.w, d); c3 = true; }
-    if (s0 | s1 | s2 | s3) {
-      // the slot kernel writes the sentinel positions; store the other components one by one
-      float *wp = (float *)&a.Wt4[p4];
-      if (c0) wp[0] = w.x;
-      if (c1) wp[1] = w.y;
-      if (c2) wp[2] = w.z;
-      if (c3) wp[3] = w.w;
-    } else if (c0 | c1 | c2 | c3) {
-      a.Wt4[p4] = w;
+  while (p4 < a.total4) {
+#pragma unroll
+    for (int u = 0; u < FV_UPDATE_UNROLL; ++u) {
+      if (p4 + u * stride < a.total4) fv_update_four(a, p4 + u * stride, w[u], xs4[q], s);
+      q += dq;
+      if (q >= a.ldk4) q -= a.ldk4;
     }
-    q += dq;
-    if (q >= a.ldk4) q -= a.ldk4;
+    p4 += FV_UPDATE_UNROLL * stride;
+    if (p4 < a.total4) fv_dense_load(a, p4, stride, w);
   }
 }
 
-// Kernel 5: the final value of every sparse element goes over its sentinel. Runs after the dense
+// Kernel 6: the final value of every sparse element goes over its sentinel. Runs after the dense
 // update so no dense thread can mistake a finished element for an ordinary weight.
 __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
   const uint32_t e = blockIdx.x * 256 + threadIdx.x;
@@ -618,8 +682,7 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMalloc((void **)&t->group_count, (size_t)t->K * sizeof(uint32_t)));
   FV_HIP(hipMalloc((void **)&t->slots, (size_t)FV_NB_CLASSES * t->B * t->w * sizeof(fv_slot)));
   FV_HIP(hipMalloc((void **)&t->xx, (size_t)t->ldk * sizeof(float)));
-  FV_HIP(hipMalloc((void **)&t->bmax,
-                   ((size_t)t->dense_blocks + ((size_t)FV_NB_CLASSES * t->B * t->w + 255) / 256) * sizeof(float)));
+  FV_HIP(hipMalloc((void **)&t->bmax, ((size_t)t->dense_blocks + (size_t)FV_NB_CLASSES * t->K) * sizeof(float)));
   FV_HIP(hipMemsetAsync(t->win, 0, ((size_t)t->B + 16) * sizeof(int32_t), t->stream));
   FV_HIP(hipMalloc((void **)&t->scalars, 16 * sizeof(float)));
   FV_HIP(hipMemsetAsync(t->Wt, 0, elems * sizeof(float), t->stream));
@@ -666,8 +729,10 @@ extern "C" int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_tr
   int rc = fv_device_info(nullptr, 0, &cus, nullptr);
   if (rc == FV_OK) {
     uint64_t want = ((uint64_t)t->total4 + 255) / 256;
-    uint64_t cap = (uint64_t)(cus > 0 ? cus : 256) * 8;
-    t->dense_blocks = (unsigned)(want < cap ? (want ? want : 1) : cap);
+    if (want == 0) want = 1;
+    const uint64_t cu = (uint64_t)(cus > 0 ? cus : 256);
+    t->dense_blocks = (unsigned)(want < cu * FV_ABSMAX_BLOCKS_PER_CU ? want : cu * FV_ABSMAX_BLOCKS_PER_CU);
+    t->update_blocks = (unsigned)(want < cu * FV_UPDATE_BLOCKS_PER_CU ? want : cu * FV_UPDATE_BLOCKS_PER_CU);
     rc = fv_trainer_alloc(t);
   }
   if (rc != FV_OK) {
@@ -891,6 +956,9 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.Wt = t->Wt;
   sp.slots = t->slots;
   sp.slot_stride = (uint64_t)t->B * t->w;
+  sp.xx = t->xx;
+  sp.invf = t->invf;
+  sp.bmax_sparse = t->bmax + t->dense_blocks;
   sp.ldk = t->ldk;
   sp.w = t->w;
   sp.V = (uint32_t)t->V;
@@ -910,18 +978,19 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.V = (uint32_t)t->V;
   d.K = t->K;
   d.n_slots = n * t->w;
-  d.slot_blocks = (FV_NB_CLASSES * d.n_slots + 255) / 256;
+  d.n_bmax = t->dense_blocks + t->K * FV_NB_CLASSES;
   d.dense_blocks = t->dense_blocks;
+  const unsigned slot_blocks = (FV_NB_CLASSES * d.n_slots + 255) / 256;
   d.eps = eps;
   d.prec = t->cfg.prec;
   d.update_cut = t->update_cut;
   const size_t smem = (size_t)t->ldk * sizeof(float);
   if (which & 8u)
-    hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks + d.slot_blocks), dim3(256), smem, t->stream, d);
+    hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
-  if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
+  if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
-  if (which & 32u) hipLaunchKernelGGL(fv_slot_update_kernel, dim3(d.slot_blocks), dim3(256), 0, t->stream, d);
+  if (which & 32u) hipLaunchKernelGGL(fv_slot_update_kernel, dim3(slot_blocks), dim3(256), 0, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[6], t->stream));
   FV_HIP(hipGetLastError());
   t->last_n = n;
