@@ -61,10 +61,10 @@ def test_small_config_bit_exact(gpu, oracle_lib, tie):
 
 @pytest.mark.parametrize("K,w,V,B", [(5, 3, 40, 64), (63, 1, 100, 128), (64, 5, 100, 100), (65, 15, 200, 256),
                                      (130, 64, 300, 64), (1000, 15, 300, 512), (2048, 7, 64, 128),
-                                     (30, 11, 20000, 700)])
+                                     (30, 11, 20000, 700), (30, 11, 30000, 700)])
 def test_shapes_bit_exact(gpu, oracle_lib, K, w, V, B):
     # K not a multiple of 64 / 4, every lane-count template, w from 1 to 64, and (last case) more
-    # columns than one LDS counting pass of the neuron kernel holds
+    # columns per class than one LDS counting pass of the sparse kernel holds (2V / 4 > 10240)
     n_tokens = 40000 if V < 20000 else 120000
     wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=V, K=K, w=w, B=B, steps=6, n_tokens=n_tokens, mean_chunk=40)
     assert np.array_equal(wg, wo)
@@ -103,6 +103,40 @@ def test_one_neuron_wins_everything(gpu, oracle_lib):
     wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=V, K=K, w=11, B=B, steps=3, W0=W0, n_tokens=100000)
     assert (wg == 3).all() and np.array_equal(wg, wo)
     assert np.array_equal(Wg, Wo)
+
+
+@pytest.mark.parametrize("V", [300, 12000])
+def test_heavy_neuron_uses_32_bit_counters(gpu, oracle_lib, V):
+    # one neuron wins 7000 windows of 11: 77000 window positions, past what 16-bit counters hold;
+    # with V = 12000 its column classes also need more than one counting pass (2V / 4 > 5120)
+    from flyvec_amd import synthetic
+    K, B = 6, 7000
+    W0 = synthetic.synapses(K, V, sigma=0.01)
+    W0[2] = np.abs(W0[2]) + 1.0
+    wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=V, K=K, w=11, B=B, steps=2, W0=W0, n_tokens=120000)
+    assert (wg == 2).all() and np.array_equal(wg, wo)
+    assert np.array_equal(Wg, Wo)
+
+
+def test_minibatch_larger_than_the_match_masks(gpu, oracle_lib):
+    # 70000 windows per step: the grouping kernel's threads take runs of more than 64 windows
+    wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=200, K=5, w=3, B=70000, steps=2, n_tokens=200000, mean_chunk=40)
+    assert np.array_equal(wg, wo)
+    assert np.array_equal(Wg, Wo)
+
+
+def test_timing_hooks(gpu):
+    from flyvec_amd import _lib, synthetic
+    V, K, w, B = 300, 64, 11, 256
+    tokens, offsets = small_corpus(20000, V)
+    t, _ = make_trainer(tokens, offsets, V, K, w, B, synthetic.synapses(K, V, sigma=0.02))
+    t.step(0, B, 1e-3)
+    total, per = t.time_steps(B, 3, 1e-3)
+    assert total > 0 and set(per) == set(_lib.TRAIN_KERNEL_NAMES) and all(v > 0 for v in per.values())
+    single = t.time_kernels(reps=3)
+    assert set(single) == set(_lib.TRAIN_KERNEL_NAMES) and all(v > 0 for v in single.values())
+    assert _lib.calibration_copy(1 << 20, 3) > 0
+    t.close()
 
 
 def test_partial_last_batch_and_epoch_driver(gpu, oracle_lib):
