@@ -30,7 +30,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # B/s, MI355X
 
-TRAIN = dict(K=400, V=20000, w=11, B=10000, n_tokens=10_000_000, lr0=2e-4, n_epochs=15, prec=1e-30)
+TRAIN = dict(K=400, V=20000, w=11, B=10000, n_tokens=10_000_000, lr0=2e-4, n_epochs=15, prec=1e-30,
+             zipf_s=1.07, mean_chunk=25)
+# the 400 MB matrix that exceeds the 256 MB Infinity Cache; the corpus is shortened from 200 M to
+# 20 M tokens (the step does not depend on its length)
+LARGE = dict(K=1000, V=50000, w=15, B=50000, n_tokens=20_000_000, lr0=2e-4, n_epochs=15, prec=1e-30,
+             zipf_s=1.0, mean_chunk=40)
+EPOCH = dict(K=400, V=20000, w=11, B=10000, n_tokens=100_000_000, lr0=2e-4, n_epochs=15, prec=1e-30,
+             zipf_s=1.07, mean_chunk=25)
 HASH = dict(K=400, V=20000, w=11, k=32, n=1 << 20)
 
 
@@ -69,10 +76,9 @@ def hash_bytes_per_window(K, w):
     return 4 * w * K + 4 * w + 8 * ((K + 63) // 64)
 
 
-def bench_train(steps, warmup, cpu_seconds):
+def bench_train(steps, warmup, cpu_seconds, c=TRAIN):
     from flyvec_amd import Trainer, synthetic
-    c = TRAIN
-    tokens, offsets = synthetic.corpus(c["n_tokens"], c["V"])
+    tokens, offsets = synthetic.corpus(c["n_tokens"], c["V"], s=c["zipf_s"], mean_chunk=c["mean_chunk"])
     W0 = synthetic.synapses(c["K"], c["V"], seed=5)
     t = Trainer(c["V"], c["K"], c["w"], c["B"], initial_learning_rate=c["lr0"], prec=c["prec"])
     t.set_corpus(tokens, offsets)
@@ -114,7 +120,8 @@ def bench_train(steps, warmup, cpu_seconds):
         "event_ms_per_step": ev_ms_per_step,
         "kernel_ms": kern_ms,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": MEASURED_TRAFFIC.get(dom),
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK,
+                     "traffic": MEASURED_TRAFFIC.get(dom) if c is TRAIN else None,
                      "algorithmic_bytes": per_kernel[dom]},
         "step_roofline_frac": (step_bytes / HBM_PEAK) / (ms_per_step * 1e-3),
         "step_algorithmic_bytes": step_bytes,
@@ -137,6 +144,47 @@ def bench_train(steps, warmup, cpu_seconds):
                                "sample": f"{done} steps of the same workload (B={c['B']}) by the C/OpenMP "
                                          f"restatement of the reference step, {dt:.1f} s"}
     return out
+
+
+def bench_epoch(c=EPOCH):
+    """One full epoch as flyvec_train runs it (flyvec/train_flyvec.py:253-263): reshuffle, every
+    minibatch of the corpus, then one checkpoint written as .npy; set-up is timed beside it."""
+    import tempfile
+    from flyvec_amd import Trainer, synthetic
+    t0 = time.perf_counter()
+    tokens, offsets = synthetic.corpus(c["n_tokens"], c["V"], s=c["zipf_s"], mean_chunk=c["mean_chunk"])
+    W0 = synthetic.synapses(c["K"], c["V"], seed=5)
+    t_gen = time.perf_counter() - t0
+    t = Trainer(c["V"], c["K"], c["w"], c["B"], initial_learning_rate=c["lr0"], prec=c["prec"])
+    t0 = time.perf_counter()
+    t.set_corpus(tokens, offsets)      # upload, window table, 1/frequency, identity order: all on the device
+    t.set_weights(W0)
+    t.sync()
+    t_setup = time.perf_counter() - t0
+    nwin = t.num_windows
+    t.shuffle(1)
+    t.run_epoch(0, c["n_epochs"])      # warm-up epoch: first-touch of every buffer
+    t0 = time.perf_counter()
+    t.shuffle(2)
+    t.sync()
+    t_shuffle = time.perf_counter() - t0
+    t1 = time.perf_counter()
+    t.run_epoch(1, c["n_epochs"])      # returns when the device has finished
+    t_steps = time.perf_counter() - t1
+    t2 = time.perf_counter()
+    W = t.get_weights()
+    with tempfile.TemporaryDirectory() as d:
+        np.save(os.path.join(d, "flyvec_model_1.npy"), W)
+    t_ckpt = time.perf_counter() - t2
+    total = time.perf_counter() - t0
+    t.close()
+    n_steps = (nwin + c["B"] - 1) // c["B"]
+    step_bytes, _ = train_bytes(c["K"], 2 * c["V"], c["w"], c["B"])
+    return {"value": nwin / total, "seconds_per_epoch": total, "n_windows": nwin, "n_steps": n_steps,
+            "ms_per_step": t_steps / n_steps * 1e3,
+            "breakdown_s": {"shuffle": t_shuffle, "minibatch_loop": t_steps, "checkpoint": t_ckpt,
+                            "setup_once": t_setup, "synthetic_corpus_generation": t_gen},
+            "step_roofline_frac": (step_bytes * (nwin / c["B"]) / HBM_PEAK) / t_steps}
 
 
 def bench_hash(reps, cpu_seconds):
@@ -190,6 +238,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample length (0 = skip)")
     ap.add_argument("--no-hash", action="store_true")
+    ap.add_argument("--workload", choices=["step", "large-step", "epoch"], default="step",
+                    help="step: the headline minibatch step (default); large-step: K=1000, V=50000, w=15, "
+                         "B=50000 (400 MB matrix); epoch: one full epoch over 100 M tokens with shuffle and "
+                         "checkpoint")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB copy kernel (yardstick for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -198,15 +250,30 @@ def main():
 
     from flyvec_amd import _lib
     info = _lib.device_info()
-    tr = bench_train(args.steps, args.warmup, args.cpu_seconds)
-    c = TRAIN
+    if args.workload == "epoch":
+        c = EPOCH
+        ep = bench_epoch(c)
+        print(json.dumps({
+            "metric": "train windows/s over one full epoch", "value": ep["value"], "unit": "windows/s",
+            "n_gpus": 1, "steps": ep["n_steps"], "warmup": ep["n_steps"], "ms_per_step": ep["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": f"full training epoch: {c['n_tokens']} Zipf(1.07) tokens, K={c['K']} "
+                                   f"Nvoc={c['V']} w={c['w']} B={c['B']}, {ep['n_windows']} windows, device "
+                                   f"shuffle before and one .npy checkpoint after"},
+            "device": info["name"].strip(), "seconds_per_epoch": ep["seconds_per_epoch"],
+            "breakdown_s": ep["breakdown_s"], "step_roofline_frac": ep["step_roofline_frac"]}))
+        return
+    c = LARGE if args.workload == "large-step" else TRAIN
+    if args.workload == "large-step":
+        args.steps, args.warmup, args.no_hash = min(args.steps, 50), min(args.warmup, 5), True
+    tr = bench_train(args.steps, args.warmup, args.cpu_seconds, c)
     line = {
-        "metric": "train windows/s at K=400,Nvoc=20k",
+        "metric": f"train windows/s at K={c['K']},Nvoc={c['V'] // 1000}k",
         "value": tr["value"], "unit": "windows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": tr["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"single training minibatch step: K={c['K']} Nvoc={c['V']} w={c['w']} B={c['B']}, "
-                               f"{c['n_tokens']} Zipf(1.07) tokens, geometric chunks (mean 25), "
+                               f"{c['n_tokens']} Zipf({c['zipf_s']}) tokens, geometric chunks (mean {c['mean_chunk']}), "
                                f"{tr['n_windows']} windows, lr 2e-4, fp32"},
         "device": info["name"].strip(),
         "roofline": tr["roofline"],

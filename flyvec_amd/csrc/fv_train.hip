@@ -29,9 +29,11 @@
 #include <math.h>
 #include <string.h>
 
+#include <utility>
 #include <vector>
 
 #include "fv_internal.h"
+#include "fv_permute.h"
 #include "fv_repeat_add.h"
 
 // Written over W[p] while the true weight of a sparse element waits in its slot record. A quiet
@@ -55,6 +57,7 @@ struct fv_trainer {
   int32_t *corpus;
   uint64_t n_tokens;
   uint64_t *starts, *perm;
+  uint64_t *perm_alt;  // second permutation buffer, allocated by the first shuffle
   uint64_t n_windows;
   float *invf;
   int32_t *idx;     // B x w column indices of the current minibatch
@@ -636,15 +639,35 @@ __global__ __launch_bounds__(256) void fv_row_norm_kernel(const float *__restric
   if (threadIdx.x == 0) out[h] = sqrt(part[0] + part[1] + part[2] + part[3]);
 }
 
+// ---- window order ------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void fv_identity_kernel(uint64_t *__restrict__ perm, uint64_t n) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) perm[i] = i;
+}
+
+// The reshuffle of flyvec/src/model_arrays.cu:451-465 rearranges the current order, cumulatively
+// over the epochs; here out[i] = in[sigma(i)] with sigma a keyed bijection computed per index.
+__global__ __launch_bounds__(256) void fv_shuffle_kernel(const uint64_t *__restrict__ in, uint64_t *__restrict__ out,
+                                                         uint64_t n, fv_feistel f) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256)
+    out[i] = in[fv_permute_index(&f, i, n)];
+}
+
+static unsigned fv_perm_blocks(uint64_t n) {
+  const uint64_t want = (n + 255) / 256;
+  return (unsigned)(want < 8192 ? want : 8192);
+}
+
 // ---- host side ------------------------------------------------------------------------------
 
 static void fv_trainer_free_corpus(fv_trainer *t) {
   (void)hipFree(t->corpus);
   (void)hipFree(t->starts);
   (void)hipFree(t->perm);
+  (void)hipFree(t->perm_alt);
   (void)hipFree(t->invf);
   t->corpus = nullptr;
-  t->starts = t->perm = nullptr;
+  t->starts = t->perm = t->perm_alt = nullptr;
   t->invf = nullptr;
   t->n_tokens = t->n_windows = 0;
   t->have_corpus = false;
@@ -786,10 +809,9 @@ extern "C" int fv_trainer_set_corpus(fv_trainer *t, const int32_t *tokens, uint6
     }
     if (rc == FV_OK) rc = fv_dev_build_window_starts(off_dev, n_chunks, t->w, t->starts, nwin, t->stream);
     if (rc == FV_OK) {
-      std::vector<uint64_t> ident(nwin);
-      for (uint64_t i = 0; i < nwin; ++i) ident[i] = i;
-      e = hipMemcpy(t->perm, ident.data(), nwin * sizeof(uint64_t), hipMemcpyHostToDevice);
-      if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "permutation upload failed: %s", hipGetErrorString(e));
+      hipLaunchKernelGGL(fv_identity_kernel, dim3(fv_perm_blocks(nwin)), dim3(256), 0, t->stream, t->perm, nwin);
+      e = hipStreamSynchronize(t->stream);
+      if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "permutation fill failed: %s", hipGetErrorString(e));
     }
   }
   (void)hipFree(off_dev);
@@ -844,30 +866,18 @@ extern "C" int fv_trainer_get_weights(fv_trainer *t, float *out_W) {
   return fv_download_weights(t->Wt, out_W, t->K, t->N, t->ldk, t->stream);
 }
 
-static inline uint64_t fv_splitmix64(uint64_t *state) {
-  uint64_t z = (*state += 0x9E3779B97F4A7C15ull);
-  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-  return z ^ (z >> 31);
-}
-
 extern "C" int fv_trainer_shuffle(fv_trainer *t, uint64_t seed) {
   FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
   FV_REQUIRE(t->have_corpus, FV_ERR_STATE, "no corpus set");
   const uint64_t n = t->n_windows;
   if (n == 0) return FV_OK;
-  FV_HIP(hipStreamSynchronize(t->stream));
-  std::vector<uint64_t> perm(n);
-  FV_HIP(hipMemcpy(perm.data(), t->perm, n * sizeof(uint64_t), hipMemcpyDeviceToHost));
-  uint64_t state = seed ^ (0xD1B54A32D192ED03ull * (t->shuffle_calls + 1));
-  for (uint64_t i = 0; i < n; ++i) {  // flyvec/src/model_arrays.cu:458-463
-    const uint64_t j = fv_splitmix64(&state) % n;
-    const uint64_t tmp = perm[i];
-    perm[i] = perm[j];
-    perm[j] = tmp;
-  }
+  if (!t->perm_alt) FV_HIP(hipMalloc((void **)&t->perm_alt, n * sizeof(uint64_t)));
+  // every call draws a different bijection, also under one seed
+  const fv_feistel f = fv_feistel_make(n, seed ^ (0xD1B54A32D192ED03ull * (t->shuffle_calls + 1)));
+  hipLaunchKernelGGL(fv_shuffle_kernel, dim3(fv_perm_blocks(n)), dim3(256), 0, t->stream, t->perm, t->perm_alt, n, f);
+  FV_HIP(hipGetLastError());
+  std::swap(t->perm, t->perm_alt);
   t->shuffle_calls++;
-  FV_HIP(hipMemcpy(t->perm, perm.data(), n * sizeof(uint64_t), hipMemcpyHostToDevice));
   return FV_OK;
 }
 

@@ -119,9 +119,10 @@ int fv_trainer_get_inverse_frequency(fv_trainer *t, float *out_invf);
 int fv_trainer_set_weights(fv_trainer *t, const float *W);
 int fv_trainer_get_weights(fv_trainer *t, float *out_W);
 
-/* flyvec/src/model_arrays.cu:442 do_reshuffle_indices: for i in order swap(perm[i],
- * perm[r_i mod Nwin]), cumulative across calls.  The reference draws r from cuRAND's
- * scrambled Sobol64; here r is a splitmix64 stream seeded by `seed`. */
+/* flyvec/src/model_arrays.cu:442 do_reshuffle_indices: rearranges the current window order,
+ * cumulatively across calls.  The reference runs a serial swap loop on the host fed by cuRAND's
+ * scrambled Sobol64; here the order becomes perm[sigma(i)] on the device, sigma a bijection of
+ * [0, Nwin) keyed by `seed` and the number of earlier calls.  Asynchronous. */
 int fv_trainer_shuffle(fv_trainer *t, uint64_t seed);
 /* Test hook replacing the random stream: install / read the window permutation. */
 int fv_trainer_set_permutation(fv_trainer *t, const uint64_t *perm, uint64_t n);

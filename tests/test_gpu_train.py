@@ -204,6 +204,31 @@ def test_repeatable_and_permutation_round_trip(gpu):
     assert np.array_equal(outs[0], outs[1])
 
 
+def test_device_shuffle_is_a_cumulative_bijection(gpu):
+    from flyvec_amd import Trainer
+    V, w = 300, 11
+    tokens, offsets = small_corpus(200000, V)
+    a, b = Trainer(V, 8, w, 64), Trainer(V, 8, w, 64)
+    a.set_corpus(tokens, offsets)
+    b.set_corpus(tokens, offsets)
+    n = a.num_windows
+    assert np.array_equal(a.get_permutation(), np.arange(n, dtype=np.uint64))   # identity after set_corpus
+    a.shuffle(3)
+    sigma = a.get_permutation()
+    assert np.array_equal(np.sort(sigma), np.arange(n, dtype=np.uint64))
+    assert np.mean(sigma == np.arange(n)) < 0.01
+    p0 = np.random.default_rng(1).permutation(n).astype(np.uint64)
+    b.set_permutation(p0)
+    b.shuffle(3)                                   # same seed, same call number: the same sigma
+    assert np.array_equal(b.get_permutation(), p0[sigma])
+    a.shuffle(3)                                   # a later call under the same seed draws another sigma
+    again = a.get_permutation()
+    assert np.array_equal(np.sort(again), np.arange(n, dtype=np.uint64))
+    assert not np.array_equal(again, sigma[sigma])
+    a.close()
+    b.close()
+
+
 def test_errors_are_reported_not_fatal(gpu):
     from flyvec_amd import Trainer, _lib, synthetic
     V, K = 50, 16
