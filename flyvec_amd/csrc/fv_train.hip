@@ -284,8 +284,10 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
   }
   __syncthreads();  // the neuron's part of order[] is now readable by the whole block
 
-  // xx[h] = fp32 sum of the scaled activations in window order
-  float xx = 0.0f;
+  // xx[h]: lane l of the first wave adds the neuron's scaled activations number l, l + 64, l + 128, ...
+  // (window order) onto 0, then the 64 partial sums are added onto 0 in lane order. For up to 64
+  // windows that is the plain sum in window order.
+  float part = 0.0f;
   for (uint32_t j0 = 0; j0 < c_h; j0 += FV_NB_ROUND) {
     const uint32_t mr = min(c_h - j0, (uint32_t)FV_NB_ROUND);
     for (uint32_t jb = tid; jb < mr; jb += 4 * T) {  // up to 4 independent loads per thread
@@ -300,19 +302,16 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
         if (jb + q * T < mr) scbuf[jb + q * T] = v[q];
     }
     __syncthreads();
-    if (tid == 0) {
-      uint32_t j = 0;
-      for (; j + 16 <= mr; j += 16) {  // 16 values fetched together, then the dependent adds
-        float4 v[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] = *(const float4 *)&scbuf[j + 4 * q];
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          xx = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(xx, v[q].x), v[q].y), v[q].z), v[q].w);
-      }
-      for (; j < mr; ++j) xx = __fadd_rn(xx, scbuf[j]);
-    }
+    if (tid < 64)
+      for (uint32_t j = tid; j < mr; j += 64) part = __fadd_rn(part, scbuf[j]);  // FV_NB_ROUND % 64 == 0
     __syncthreads();
+  }
+  float xx = 0.0f;
+  if (tid < 64) scbuf[tid] = part;
+  __syncthreads();
+  if (tid == 0) {
+    const uint32_t np = min(c_h, 64u);
+    for (uint32_t l = 0; l < np; ++l) xx = __fadd_rn(xx, scbuf[l]);
   }
   if (tid == 0) a.xx[h] = xx;
 }

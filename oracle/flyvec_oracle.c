@@ -19,8 +19,13 @@
  *       shapes, and numpy restatements of each stage.
  *
  * Order-dependent fp32 sums (the reference uses atomics whose order is not
- * defined) are realised here in increasing window order, then increasing
- * position inside the window.
+ * defined) are given a fixed order here.  The sparse term of ds: increasing
+ * window order, then increasing position inside the window.  The per-neuron
+ * totals xx: see fvo_xx_sums (64 interleaved partial sums in window order,
+ * then the partials in index order; for a neuron with at most 64 windows that
+ * is the plain sum in window order).  fvo_xx_sums is pinned by a numpy
+ * restatement of that order and by its agreement with plain window order (to
+ * rounding) in tests/test_oracle_train.py.
  */
 #include <math.h>
 #include <stdint.h>
@@ -167,6 +172,36 @@ float fvo_epoch_eps(float lr0, uint64_t epoch, uint64_t n_epochs) {
 }
 
 /*
+ * xx[h] = sum of sc[r] over the windows r won by h (flyvec/src/cuda_funcs.cu:722-744, fp32 atomics
+ * there).  order_kind 0: the j-th window of neuron h, counted in increasing window order, is added
+ * onto partial sum j mod 64 (each starting at 0); the partials that received a value are then
+ * added onto 0 in index order.  order_kind 1: every window added onto xx[h] in increasing window
+ * order.  The two agree for neurons with at most 64 windows.
+ */
+#define FVO_XX_LANES 64
+void fvo_xx_sums(const int32_t *win, const float *sc, uint64_t n, int K, int order_kind, float *xx) {
+  for (int h = 0; h < K; ++h) xx[h] = 0.0f;
+  if (order_kind == 1) {
+    for (uint64_t r = 0; r < n; ++r) xx[win[r]] = xx[win[r]] + sc[r];
+    return;
+  }
+  float *part = (float *)calloc((size_t)K * FVO_XX_LANES, sizeof(float));
+  uint64_t *cnt = (uint64_t *)calloc((size_t)K, sizeof(uint64_t));
+  for (uint64_t r = 0; r < n; ++r) {
+    const int h = win[r];
+    float *p = part + (size_t)h * FVO_XX_LANES + (cnt[h] % FVO_XX_LANES);
+    *p = *p + sc[r];
+    cnt[h]++;
+  }
+  for (int h = 0; h < K; ++h) {
+    const uint64_t used = cnt[h] < FVO_XX_LANES ? cnt[h] : FVO_XX_LANES;
+    for (uint64_t l = 0; l < used; ++l) xx[h] = xx[h] + part[(size_t)h * FVO_XX_LANES + l];
+  }
+  free(part);
+  free(cnt);
+}
+
+/*
  * One minibatch step on already inflated indices (idx is n x w).
  * Order follows flyvec/src/cuda_funcs.cu:1662-1803 for sparse_input = 1,
  * frequency_scaling = 1, Lmid = Lbase = 1, delta = 0, p = 2:
@@ -174,7 +209,7 @@ float fvo_epoch_eps(float lr0, uint64_t epoch, uint64_t n_epochs) {
  *   :1700-1701   scaled and raw activations   (from that copy, i.e. from W)
  *   :1715        xx <- 0
  *   :1719        winner = argmax of RAW
- *   :1721        xx[winner] += SCALED[r][winner]              (:722-744)
+ *   :1721        xx[winner] += SCALED[r][winner]              (:722-744; order: fvo_xx_sums kind 0)
  *   :1722        ds[h][:] = xx[h] != 0 ? -xx[h]*W[h][:] : 0   (:394-406)
  *   :1732        ds[winner][idx] += invf[idx % V]             (:657-672)
  *   :1792        rows with xx == 0 zero-filled; nc = max|ds|  (cu_special_reduction.cu:26-99)
@@ -189,7 +224,7 @@ void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx,
                     int32_t *winners, float *sc_at_winner, float *xx_out, float *nc_out) {
   int32_t *win = (int32_t *)malloc(sizeof(int32_t) * (n ? n : 1));
   float *scw = (float *)malloc(sizeof(float) * (n ? n : 1));
-  float *xx = (float *)calloc((size_t)K, sizeof(float));
+  float *xx = (float *)calloc((size_t)(K > 0 ? K : 1), sizeof(float));
   float *ds = ds_scratch;
 
 #pragma omp parallel
@@ -219,8 +254,7 @@ void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx,
     free(raw);
   }
 
-  /* xx: fp32 adds in increasing window order */
-  for (uint64_t r = 0; r < n; ++r) xx[win[r]] = xx[win[r]] + scw[r];
+  fvo_xx_sums(win, scw, n, K, 0, xx);
 
   /* ds = -xx*W or 0 */
 #pragma omp parallel for schedule(static)

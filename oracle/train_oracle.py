@@ -55,6 +55,8 @@ def lib():
         L.fvo_argmax_lowest.argtypes = [C.c_void_p, C.c_int]
         L.fvo_epoch_eps.restype = C.c_float
         L.fvo_epoch_eps.argtypes = [C.c_float, C.c_uint64, C.c_uint64]
+        L.fvo_xx_sums.restype = None
+        L.fvo_xx_sums.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_int, C.c_void_p]
         L.fvo_train_step.restype = None
         L.fvo_train_step.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, C.c_void_p, C.c_uint64,
                                      C.c_int, C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_void_p,
@@ -162,6 +164,16 @@ def argmax_reference(row):
 def argmax_lowest(row):
     row = np.ascontiguousarray(row, dtype=np.float32)
     return int(lib().fvo_argmax_lowest(_p(row), len(row)))
+
+
+def xx_sums(winners, sc, K, order_kind=0):
+    """Per-neuron totals of the scaled activations; order_kind 0 = the step's order (64 interleaved
+    partial sums), 1 = plain window order."""
+    winners = np.ascontiguousarray(winners, dtype=np.int32)
+    sc = np.ascontiguousarray(sc, dtype=np.float32)
+    xx = np.empty(K, dtype=np.float32)
+    lib().fvo_xx_sums(_p(winners), _p(sc), len(winners), K, order_kind, _p(xx))
+    return xx
 
 
 def epoch_eps(lr0, epoch, n_epochs):

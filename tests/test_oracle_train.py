@@ -301,3 +301,58 @@ def test_multi_step_driver_matches_single_steps():
     if tail:
         wt = to.train_steps(Wa, corpus, starts, perm, (len(perm) // B) * B, B, 1, w, invf, 1e-3)
         assert len(wt) == tail
+
+
+# ---- order of the per-neuron totals ---------------------------------------------------------------
+
+def xx_numpy(winners, sc, K):
+    """The step's order, restated: value j of a neuron (window order) joins partial j mod 64; the
+    partials in use are then added in index order. np.cumsum in float32 adds strictly left to right."""
+    out = np.zeros(K, dtype=f32)
+    for h in range(K):
+        v = sc[winners == h]
+        if len(v) == 0:
+            continue
+        parts = [np.cumsum(v[l::64], dtype=f32)[-1] for l in range(min(64, len(v)))]
+        out[h] = np.cumsum(np.array(parts, dtype=f32), dtype=f32)[-1]
+    return out
+
+
+@pytest.mark.parametrize("n,K", [(1, 3), (50, 4), (64, 1), (65, 1), (129, 2), (5000, 7), (40000, 3)])
+def test_xx_order_against_numpy(n, K):
+    rng = np.random.default_rng(n + K)
+    winners = rng.integers(0, K, size=n).astype(np.int32)
+    sc = (rng.standard_normal(n) * 10.0 ** rng.uniform(-3, 1, n)).astype(f32)
+    assert np.array_equal(to.xx_sums(winners, sc, K, 0), xx_numpy(winners, sc, K))
+    seq = np.zeros(K, dtype=f32)
+    for r in range(n):
+        seq[winners[r]] = f32(seq[winners[r]] + sc[r])
+    assert np.array_equal(to.xx_sums(winners, sc, K, 1), seq)
+
+
+def test_xx_order_is_window_order_up_to_64_windows_and_close_beyond():
+    rng = np.random.default_rng(5)
+    K = 40
+    winners = np.repeat(np.arange(K), 64).astype(np.int32)      # exactly 64 windows each
+    rng.shuffle(winners)
+    sc = rng.standard_normal(len(winners)).astype(f32)
+    assert np.array_equal(to.xx_sums(winners, sc, K, 0), to.xx_sums(winners, sc, K, 1))
+    winners = rng.integers(0, 3, size=30000).astype(np.int32)
+    sc = np.abs(rng.standard_normal(30000)).astype(f32)
+    a, b = to.xx_sums(winners, sc, 3, 0), to.xx_sums(winners, sc, 3, 1)
+    exact = np.array([sc[winners == h].astype(np.float64).sum() for h in range(3)])
+    assert not np.array_equal(a, b)                              # the orders do differ ...
+    assert np.all(np.abs(a - exact) <= 2e-5 * exact)             # ... by rounding only
+    assert np.all(np.abs(b - exact) <= 2e-5 * exact)
+
+
+def test_step_uses_the_interleaved_order():
+    rng = np.random.default_rng(8)
+    K, V, w, n = 3, 30, 5, 2000
+    W = rng.standard_normal((K, 2 * V)).astype(f32)
+    idx = rng.integers(0, V, size=(n, w)).astype(np.int32)
+    idx[:, w // 2] += V
+    invf = (1.0 / rng.integers(1, 50, size=V)).astype(f32)
+    res = to.train_step(W.copy(), idx, invf, 1e-3)
+    assert np.bincount(res["winners"], minlength=K).max() > 64
+    assert np.array_equal(res["xx"], xx_numpy(res["winners"], res["sc"], K))
