@@ -39,10 +39,9 @@
 // Written over W[p] while the true weight of a sparse element waits in its slot record. A quiet
 // NaN with a payload no arithmetic produces.
 #define FV_SENTINEL 0x7fc5ca1eu
-#define FV_SLOT_INVALID 0xffffffffu
 
 struct fv_slot {
-  uint32_t p;  // element index i * ldk + h, or FV_SLOT_INVALID
+  uint32_t p;  // element index i * ldk + h
   uint32_t n;  // pending additions of 1/f
   float wv;    // the weight the sentinel replaced
 };
@@ -66,6 +65,7 @@ struct fv_trainer {
   uint32_t *order;  // B window ids grouped by winner, ascending inside a group
   uint32_t *group_base, *group_count;  // K each
   fv_slot *slots;   // FV_NB_CLASSES regions of B x w slot records
+  uint32_t *slot_count;  // K * FV_NB_CLASSES
   float *xx;        // ldk
   float *bmax;      // max|ds| of each block of the absmax launch, then of each block of the sparse launch
   float *scalars;   // [0] max|ds| of the last step
@@ -171,6 +171,11 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
 #endif
 #define FV_NB_CLASSES (1 << FV_NB_CLASS_SHIFT)  // column classes per neuron (kernel 3)
 #define FV_NB_CNT_WORDS 5120    // LDS counter words per class block (20 KB)
+#define FV_SP_LIST_CAP 1024     // positions of non-zero counters collected in LDS at a time
+#define FV_SP_CHUNK 16          // window positions read by 16 neighbouring lanes (idx is padded by this much)
+#define FV_SP_STAGE 2048        // window ids staged in LDS at a time
+#define FV_SP_GROUP 8           // loads per lane are issued in groups of this many ...
+#define FV_SP_GROUPS 4          // ... and this many groups are in flight before the first is counted
 #define FV_NB_ROUND 2048        // scaled activations staged in LDS at a time
 #define FV_NB_LOADS 16          // independent loads issued together
 
@@ -328,18 +333,69 @@ struct fv_sparse_args {
   const uint32_t *order;
   const uint32_t *group_base;
   const uint32_t *group_count;
-  const int32_t *idx;
+  const int32_t *idx;  // readable FV_SP_CHUNK entries past its end
   float *Wt;
   fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records
   uint64_t slot_stride;
   const float *xx;
   const float *invf;
-  float *bmax_sparse;  // one maximum of |ds| per block
+  float *bmax_sparse;    // one maximum of |ds| per block
+  uint32_t *slot_count;  // records written per block
   uint32_t ldk, w, V;
 };
 
+// Barrier for data exchanged through LDS only: waits for the wave's LDS operations, not for its
+// global stores still in flight.
+__device__ __forceinline__ void fv_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// Counting pass of one class block over the windows whose ids are staged in LDS (ord[0 .. n_staged)).
+// Sixteen consecutive lanes read sixteen consecutive positions of one window, so a wave's load
+// touches four rows of the index matrix; positions past the window (the next row, or the padding
+// behind the last one) are loaded and dropped.
+template <bool NARROW>
+__device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const uint32_t *ord, uint32_t n_staged,
+                                                const int32_t *__restrict__ idx, uint32_t w, uint32_t n_cols,
+                                                uint32_t q, uint32_t lo, uint32_t span, uint32_t tid) {
+  const uint32_t c = tid & 15u, slot = tid >> 4;  // the block takes 16 windows per step
+  const uint32_t steps = (n_staged + 15) >> 4;
+  for (uint32_t c0 = 0; c0 < w; c0 += FV_SP_CHUNK) {
+    const uint32_t cc = c0 + c;
+    const bool col_ok = cc < w;
+    for (uint32_t s0 = 0; s0 < steps; s0 += FV_SP_GROUPS * FV_SP_GROUP) {
+      int32_t iv[FV_SP_GROUPS][FV_SP_GROUP];
+#pragma unroll
+      for (int g = 0; g < FV_SP_GROUPS; ++g) {
+        if (s0 + g * FV_SP_GROUP < steps) {  // the same answer in the whole block
+#pragma unroll
+          for (int b = 0; b < FV_SP_GROUP; ++b)
+            iv[g][b] = idx[ord[min((s0 + g * FV_SP_GROUP + b) * 16 + slot, n_staged - 1)] * w + cc];
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < FV_SP_GROUPS; ++g) {
+        if (s0 + g * FV_SP_GROUP < steps) {
+#pragma unroll
+          for (int b = 0; b < FV_SP_GROUP; ++b) {
+            const uint32_t i = (uint32_t)iv[g][b];
+            const uint32_t k = (i >> FV_NB_CLASS_SHIFT) - lo;
+            if (col_ok && (s0 + g * FV_SP_GROUP + b) * 16 + slot < n_staged && i < n_cols &&
+                (i & (FV_NB_CLASSES - 1)) == q && k < span) {
+              if (NARROW)
+                atomicAdd(&cnt[k >> 1], 1u << (16 * (k & 1)));
+              else
+                atomicAdd(&cnt[k], 1u);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
   __shared__ uint32_t cnt[FV_NB_CNT_WORDS];
+  __shared__ uint16_t list[FV_SP_LIST_CAP];
+  __shared__ uint32_t ord[FV_SP_STAGE];
   __shared__ uint32_t sh_pos;
   constexpr uint32_t T = 256;
   const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT;
@@ -347,21 +403,25 @@ __global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
   const uint32_t tid = threadIdx.x;
   const uint32_t c_h = a.group_count[h];
   if (c_h == 0) {
-    if (tid == 0) a.bmax_sparse[blockIdx.x] = 0.0f;
+    if (tid == 0) {
+      a.bmax_sparse[blockIdx.x] = 0.0f;
+      a.slot_count[blockIdx.x] = 0;
+    }
     return;
   }
   const uint32_t base = a.group_base[h];
   const float x_h = a.xx[h];
   float ds_max = 0.0f;
   const uint32_t *__restrict__ order = a.order + base;
-  const int32_t *__restrict__ idx = a.idx;
   const uint32_t n_cols = 2 * a.V;
   const uint32_t m_ent = c_h * a.w;
   fv_slot *slots = a.slots + (uint64_t)q * a.slot_stride + (uint64_t)base * a.w;
 
-  if (tid == 0) sh_pos = 0;
   for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
-  __syncthreads();
+  const bool staged_once = c_h <= FV_SP_STAGE;  // the usual case: the neuron's window ids are staged here
+  if (staged_once)
+    for (uint32_t i = tid; i < c_h; i += T) ord[i] = order[i];
+  fv_lds_barrier();
 
   // No counter can exceed the neuron's number of window positions: below 2^16 of them, two 16-bit
   // counters share a word and one pass covers twice as many columns.
@@ -371,84 +431,111 @@ __global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
   uint32_t emitted = 0;
 
   for (uint32_t lo = 0; lo < class_cols; lo += span) {
-    // count: one window position per thread at a time, FV_NB_LOADS of them in flight
-    for (uint32_t eb = tid; eb < m_ent; eb += FV_NB_LOADS * T) {
-      uint32_t rr[FV_NB_LOADS], cc[FV_NB_LOADS];
-      int32_t iv[FV_NB_LOADS];
-#pragma unroll
-      for (int u = 0; u < FV_NB_LOADS; ++u) {
-        const uint32_t e = min(eb + u * T, m_ent - 1);
-        const uint32_t j = e / a.w;
-        cc[u] = e - j * a.w;
-        rr[u] = order[j];
+    for (uint32_t j0 = 0; j0 < c_h; j0 += FV_SP_STAGE) {
+      const uint32_t n_staged = min(c_h - j0, (uint32_t)FV_SP_STAGE);
+      if (!staged_once) {
+        fv_lds_barrier();  // the previous part has been counted
+        for (uint32_t i = tid; i < n_staged; i += T) ord[i] = order[j0 + i];
+        fv_lds_barrier();
       }
+      if (narrow)
+        fv_sparse_count<true>(cnt, ord, n_staged, a.idx, a.w, n_cols, q, lo, span, tid);
+      else
+        fv_sparse_count<false>(cnt, ord, n_staged, a.idx, a.w, n_cols, q, lo, span, tid);
+    }
+    // Every non-zero counter is one distinct element. Their positions are collected in LDS, up to
+    // FV_SP_LIST_CAP at a time; a counter is cleared when its element is taken, so what did not fit
+    // is found again by the next round.
+    uint32_t found;
+    do {
+      if (tid == 0) sh_pos = 0;
+      fv_lds_barrier();
+      {
+        // bit 8 * i + u of `mine`: counter u of the thread's i-th group of four words is non-zero
+        static_assert(FV_NB_CNT_WORDS == 4 * 5 * 256, "five groups of four counter words per thread");
+        uint64_t mine = 0;
 #pragma unroll
-      for (int u = 0; u < FV_NB_LOADS; ++u) iv[u] = idx[(uint64_t)rr[u] * a.w + cc[u]];
+        for (int i = 0; i < 5; ++i) {
+          const uint4 c4 = ((const uint4 *)cnt)[tid + i * T];
+          const uint32_t cw[4] = {c4.x, c4.y, c4.z, c4.w};
+          uint32_t bits = 0;
 #pragma unroll
-      for (int u = 0; u < FV_NB_LOADS; ++u) {
-        const uint32_t i = (uint32_t)iv[u];
-        const uint32_t k = (i >> FV_NB_CLASS_SHIFT) - lo;
-        if (eb + u * T < m_ent && i < n_cols && (i & (FV_NB_CLASSES - 1)) == q && k < span) {
-          if (narrow)
-            atomicAdd(&cnt[k >> 1], 1u << (16 * (k & 1)));
-          else
-            atomicAdd(&cnt[k], 1u);
+          for (int u = 0; u < 4; ++u) {
+            if (narrow) {
+              bits |= ((cw[u] & 0xffffu) ? 1u : 0u) << (2 * u);
+              bits |= ((cw[u] >> 16) ? 1u : 0u) << (2 * u + 1);
+            } else {
+              bits |= (cw[u] ? 1u : 0u) << u;
+            }
+          }
+          mine |= (uint64_t)bits << (8 * i);
+        }
+        // list positions: prefix sum inside the wave, one LDS atomic per wave
+        const uint32_t my = (uint32_t)__popcll(mine);
+        const int lane = tid & 63;
+        uint32_t incl = my;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const uint32_t o = __shfl_up(incl, d, 64);
+          if (lane >= d) incl += o;
+        }
+        uint32_t wave_base = 0;
+        if (lane == 63 && incl) wave_base = atomicAdd(&sh_pos, incl);
+        wave_base = __shfl(wave_base, 63, 64);
+        uint32_t e = wave_base + incl - my;
+        while (mine) {
+          const uint32_t b = (uint32_t)__ffsll((long long)mine) - 1;
+          mine &= mine - 1;
+          if (e < FV_SP_LIST_CAP) list[e] = (uint16_t)((tid + (b >> 3) * T) * (narrow ? 8u : 4u) + (b & 7u));
+          ++e;
         }
       }
-    }
-    __syncthreads();
-    // every non-zero counter is one distinct element: append (element, count) to the slot records
-    // and reset the counter for the next pass ...
-    for (uint32_t k4 = tid; k4 < FV_NB_CNT_WORDS / 4; k4 += T) {
-      const uint4 c4 = ((const uint4 *)cnt)[k4];
-      if ((c4.x | c4.y | c4.z | c4.w) == 0) continue;
-      ((uint4 *)cnt)[k4] = make_uint4(0, 0, 0, 0);
-      const uint32_t cw[4] = {c4.x, c4.y, c4.z, c4.w};
-      const uint32_t per = narrow ? 8 : 4;  // counters in this uint4
+      fv_lds_barrier();
+      found = sh_pos;
+      const uint32_t take = min(found, (uint32_t)FV_SP_LIST_CAP);
+      // one element per thread (four in flight): save its weight and its count in a slot record,
+      // plant the sentinel, take |ds| (the dense term plus count additions of 1/f; a row with
+      // xx == 0 has ds == 0)
+      for (uint32_t eb = tid; eb < take; eb += 4 * T) {
+        uint32_t pe[4], ne[4];
+        float wv[4], fe[4];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        if (u >= (int)per) break;
-        const uint32_t c = narrow ? (cw[u >> 1] >> (16 * (u & 1))) & 0xffffu : cw[u];
-        if (c == 0) continue;
-        const uint32_t col = ((lo + k4 * per + u) << FV_NB_CLASS_SHIFT) | q;
-        const uint32_t e = atomicAdd(&sh_pos, 1u);
-        slots[e].p = col * a.ldk + h;
-        slots[e].n = c;
-      }
-    }
-    __syncthreads();
-    // ... then one element per thread: save its weight, plant the sentinel, and take |ds| of the
-    // element (the dense term plus count additions of 1/f; a row with xx == 0 has ds == 0)
-    const uint32_t end = sh_pos;
-    for (uint32_t eb = emitted + tid; eb < end; eb += 4 * T) {
-      uint32_t pe[4], ne[4];
-      float wv[4], fe[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const fv_slot *sl = &slots[min(eb + u * T, end - 1)];
-        pe[u] = sl->p;
-        ne[u] = sl->n;
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        wv[u] = a.Wt[pe[u]];
-        const uint32_t col = pe[u] / a.ldk;
-        fe[u] = a.invf[col >= a.V ? col - a.V : col];
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-        if (eb + u * T < end) {
-          slots[eb + u * T].wv = wv[u];
-          a.Wt[pe[u]] = __uint_as_float(FV_SENTINEL);
-          if (x_h != 0.0f) ds_max = fv_absmax_keep(ds_max, fv_sparse_ds(x_h, wv[u], fe[u], ne[u]));
+        for (int u = 0; u < 4; ++u) {
+          const uint32_t k = list[min(eb + u * T, take - 1)];
+          const uint32_t word = narrow ? cnt[k >> 1] : cnt[k];
+          ne[u] = narrow ? (word >> (16 * (k & 1))) & 0xffffu : word;
+          const uint32_t col = ((lo + k) << FV_NB_CLASS_SHIFT) | q;
+          pe[u] = col * a.ldk + h;
+          wv[u] = a.Wt[pe[u]];
+          fe[u] = a.invf[col >= a.V ? col - a.V : col];
+          if (eb + u * T < take) {
+            if (narrow)
+              atomicAnd(&cnt[k >> 1], 0xffff0000u >> (16 * (k & 1)));
+            else
+              cnt[k] = 0;
+          }
         }
-    }
-    emitted = end;
-    __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (eb + u * T < take) {
+            fv_slot rec;
+            rec.p = pe[u];
+            rec.n = ne[u];
+            rec.wv = wv[u];
+            slots[emitted + eb + u * T] = rec;
+            a.Wt[pe[u]] = __uint_as_float(FV_SENTINEL);
+            if (x_h != 0.0f) ds_max = fv_absmax_keep(ds_max, fv_sparse_ds(x_h, wv[u], fe[u], ne[u]));
+          }
+      }
+      emitted += take;
+      fv_lds_barrier();
+    } while (found > FV_SP_LIST_CAP);
   }
-  for (uint32_t e = emitted + tid; e < m_ent; e += T) slots[e].p = FV_SLOT_INVALID;
   const float bm = fv_block_max_nonneg(ds_max, (float *)cnt);
-  if (tid == 0) a.bmax_sparse[blockIdx.x] = bm;
+  if (tid == 0) {
+    a.bmax_sparse[blockIdx.x] = bm;
+    a.slot_count[blockIdx.x] = emitted;
+  }
 }
 
 // ---- kernels 3 and 4: dense passes over the matrix ------------------------------------------------
@@ -457,19 +544,15 @@ struct fv_dense_args {
   float4 *Wt4;
   const float *xx;
   const float *invf;
-  const fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records, n_slots used in each
+  const fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records
   uint64_t slot_stride;
+  const uint32_t *slot_count;  // records of each block of the sparse launch
+  const uint32_t *group_base;
   float *bmax;           // n_bmax block maxima of |ds|: dense blocks, then the sparse kernel's blocks
   float *scalars;
-  uint32_t total4, ldk4, ldk, V, K, n_slots, n_bmax, dense_blocks;
+  uint32_t total4, ldk4, ldk, V, K, w, n_bmax, dense_blocks;
   float eps, prec, update_cut;
 };
-
-// Slot record of flat index e over the FV_NB_CLASSES regions (e < FV_NB_CLASSES * n_slots).
-__device__ __forceinline__ const fv_slot *fv_slot_at(const fv_dense_args &a, uint32_t e) {
-  const uint32_t region = e / a.n_slots;
-  return a.slots + (uint64_t)region * a.slot_stride + (e - region * a.n_slots);
-}
 
 __device__ __forceinline__ bool fv_is_sentinel(float w) { return __float_as_uint(w) == FV_SENTINEL; }
 
@@ -605,20 +688,24 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
 // Kernel 6: the final value of every sparse element goes over its sentinel. Runs after the dense
 // update so no dense thread can mistake a finished element for an ordinary weight.
 __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
-  const uint32_t e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= FV_NB_CLASSES * a.n_slots) return;
-  const fv_slot sl = *fv_slot_at(a, e);
-  if (sl.p == FV_SLOT_INVALID) return;
-  const uint32_t i = sl.p / a.ldk, h = sl.p - i * a.ldk;
+  // block (h, q) of the sparse launch wrote slot_count records at the start of its part of region q
+  const uint32_t count = a.slot_count[blockIdx.x];
+  if (count == 0) return;
+  const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT, q = blockIdx.x & (FV_NB_CLASSES - 1);
+  const fv_slot *slots = a.slots + (uint64_t)q * a.slot_stride + (uint64_t)a.group_base[h] * a.w;
   const float x = a.xx[h];
-  float out = sl.wv;  // a row with xx == 0 is not updated: the saved weight goes back
-  if (x != 0.0f) {
-    const float nc = a.scalars[0];
-    const float s = a.prec > nc ? a.eps / a.prec : a.eps / nc;
-    const float d = __fmul_rn(s, fv_sparse_ds(x, sl.wv, a.invf[i >= a.V ? i - a.V : i], sl.n));
-    if (fabsf(d) > a.update_cut) out = __fadd_rn(sl.wv, d);
+  const float nc = a.scalars[0];
+  const float s = a.prec > nc ? a.eps / a.prec : a.eps / nc;
+  for (uint32_t e = threadIdx.x; e < count; e += 256) {
+    const fv_slot sl = slots[e];
+    float out = sl.wv;  // a row with xx == 0 is not updated: the saved weight goes back
+    if (x != 0.0f) {
+      const uint32_t i = sl.p / a.ldk;
+      const float d = __fmul_rn(s, fv_sparse_ds(x, sl.wv, a.invf[i >= a.V ? i - a.V : i], sl.n));
+      if (fabsf(d) > a.update_cut) out = __fadd_rn(sl.wv, d);
+    }
+    ((float *)a.Wt4)[sl.p] = out;
   }
-  ((float *)a.Wt4)[sl.p] = out;
 }
 
 // ---- row norms (log line of flyvec/src/cuda_funcs.cu:1234-1242) -------------------------------
@@ -679,6 +766,7 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   (void)hipFree(t->Wt);
   (void)hipFree(t->idx);
   (void)hipFree(t->slots);
+  (void)hipFree(t->slot_count);
   (void)hipFree(t->order);
   (void)hipFree(t->group_base);
   (void)hipFree(t->group_count);
@@ -696,13 +784,15 @@ static int fv_trainer_alloc(fv_trainer *t) {
   const size_t elems = (size_t)t->N * t->ldk;
   FV_HIP(hipStreamCreate(&t->stream));
   FV_HIP(hipMalloc((void **)&t->Wt, elems * sizeof(float)));
-  FV_HIP(hipMalloc((void **)&t->idx, (size_t)t->B * t->w * sizeof(int32_t)));
+  FV_HIP(hipMalloc((void **)&t->idx, ((size_t)t->B * t->w + FV_SP_CHUNK) * sizeof(int32_t)));
+  FV_HIP(hipMemsetAsync(t->idx, 0xff, ((size_t)t->B * t->w + FV_SP_CHUNK) * sizeof(int32_t), t->stream));
   FV_HIP(hipMalloc((void **)&t->win, ((size_t)t->B + 16) * sizeof(int32_t)));  // read in 16-byte pieces
   FV_HIP(hipMalloc((void **)&t->sc, (size_t)t->B * sizeof(float)));
   FV_HIP(hipMalloc((void **)&t->order, (size_t)t->B * sizeof(uint32_t)));
   FV_HIP(hipMalloc((void **)&t->group_base, (size_t)t->K * sizeof(uint32_t)));
   FV_HIP(hipMalloc((void **)&t->group_count, (size_t)t->K * sizeof(uint32_t)));
   FV_HIP(hipMalloc((void **)&t->slots, (size_t)FV_NB_CLASSES * t->B * t->w * sizeof(fv_slot)));
+  FV_HIP(hipMalloc((void **)&t->slot_count, (size_t)FV_NB_CLASSES * t->K * sizeof(uint32_t)));
   FV_HIP(hipMalloc((void **)&t->xx, (size_t)t->ldk * sizeof(float)));
   FV_HIP(hipMalloc((void **)&t->bmax, ((size_t)t->dense_blocks + (size_t)FV_NB_CLASSES * t->K) * sizeof(float)));
   FV_HIP(hipMemsetAsync(t->win, 0, ((size_t)t->B + 16) * sizeof(int32_t), t->stream));
@@ -968,6 +1058,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.xx = t->xx;
   sp.invf = t->invf;
   sp.bmax_sparse = t->bmax + t->dense_blocks;
+  sp.slot_count = t->slot_count;
   sp.ldk = t->ldk;
   sp.w = t->w;
   sp.V = (uint32_t)t->V;
@@ -978,6 +1069,9 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.xx = t->xx;
   d.invf = t->invf;
   d.slots = t->slots;
+  d.slot_count = t->slot_count;
+  d.group_base = t->group_base;
+  d.w = t->w;
   d.slot_stride = (uint64_t)t->B * t->w;
   d.bmax = t->bmax;
   d.scalars = t->scalars;
@@ -986,10 +1080,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.ldk = t->ldk;
   d.V = (uint32_t)t->V;
   d.K = t->K;
-  d.n_slots = n * t->w;
   d.n_bmax = t->dense_blocks + t->K * FV_NB_CLASSES;
   d.dense_blocks = t->dense_blocks;
-  const unsigned slot_blocks = (FV_NB_CLASSES * d.n_slots + 255) / 256;
   d.eps = eps;
   d.prec = t->cfg.prec;
   d.update_cut = t->update_cut;
@@ -999,7 +1091,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
   if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
-  if (which & 32u) hipLaunchKernelGGL(fv_slot_update_kernel, dim3(slot_blocks), dim3(256), 0, t->stream, d);
+  if (which & 32u) hipLaunchKernelGGL(fv_slot_update_kernel, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[6], t->stream));
   FV_HIP(hipGetLastError());
   t->last_n = n;
