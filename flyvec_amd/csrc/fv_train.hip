@@ -174,8 +174,12 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
 #define FV_SP_LIST_CAP 1024     // positions of non-zero counters collected in LDS at a time
 #define FV_SP_CHUNK 16          // window positions read by 16 neighbouring lanes (idx is padded by this much)
 #define FV_SP_STAGE 2048        // window ids staged in LDS at a time
-#define FV_SP_GROUP 8           // loads per lane are issued in groups of this many ...
-#define FV_SP_GROUPS 4          // ... and this many groups are in flight before the first is counted
+#ifndef FV_SP_THREADS
+#define FV_SP_THREADS 512       // threads of a class block
+#endif
+#ifndef FV_SP_LOADS
+#define FV_SP_LOADS 24          // most loads a lane has in flight in the counting pass
+#endif
 #define FV_NB_ROUND 2048        // scaled activations staged in LDS at a time
 #define FV_NB_LOADS 16          // independent loads issued together
 
@@ -199,13 +203,15 @@ __device__ __forceinline__ float fv_absmax_keep(float m, float v) {
   return a > m ? a : m;  // a NaN never replaces m, as in the reference's comparison
 }
 
-// Block-wide maximum of non-negative floats; result valid in thread 0.
-__device__ __forceinline__ float fv_block_max_nonneg(float m, float *smem4) {
+// Block-wide maximum of non-negative floats (blocks of up to 16 waves; smem holds one float per wave).
+__device__ __forceinline__ float fv_block_max_nonneg(float m, float *smem) {
   const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
   __syncthreads();
-  if ((threadIdx.x & 63) == 0) smem4[threadIdx.x >> 6] = __uint_as_float(wm);
+  if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = __uint_as_float(wm);
   __syncthreads();
-  return fmaxf(fmaxf(smem4[0], smem4[1]), fmaxf(smem4[2], smem4[3]));
+  float r = smem[0];
+  for (uint32_t i = 1; i < (blockDim.x >> 6); ++i) r = fmaxf(r, smem[i]);
+  return r;
 }
 
 // Sum over the block of one value per thread (result in every thread).
@@ -351,53 +357,58 @@ __device__ __forceinline__ void fv_lds_barrier() { asm volatile("s_waitcnt lgkmc
 // Counting pass of one class block over the windows whose ids are staged in LDS (ord[0 .. n_staged)).
 // Sixteen consecutive lanes read sixteen consecutive positions of one window, so a wave's load
 // touches four rows of the index matrix; positions past the window (the next row, or the padding
-// behind the last one) are loaded and dropped.
-template <bool NARROW>
+// behind the last one) are loaded and dropped. A lane issues LOADS loads back to back with no
+// branch between them (the compiler waits for every load in flight at a branch target), then counts.
+#define FV_SP_WPS (FV_SP_THREADS / 16)  // windows the block takes per step
+template <bool NARROW, int LOADS>
 __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const uint32_t *ord, uint32_t n_staged,
                                                 const int32_t *__restrict__ idx, uint32_t w, uint32_t n_cols,
                                                 uint32_t q, uint32_t lo, uint32_t span, uint32_t tid) {
-  const uint32_t c = tid & 15u, slot = tid >> 4;  // the block takes 16 windows per step
-  const uint32_t steps = (n_staged + 15) >> 4;
+  const uint32_t c = tid & 15u, slot = tid >> 4;
+  const uint32_t steps = (n_staged + FV_SP_WPS - 1) / FV_SP_WPS;
   for (uint32_t c0 = 0; c0 < w; c0 += FV_SP_CHUNK) {
     const uint32_t cc = c0 + c;
     const bool col_ok = cc < w;
-    for (uint32_t s0 = 0; s0 < steps; s0 += FV_SP_GROUPS * FV_SP_GROUP) {
-      int32_t iv[FV_SP_GROUPS][FV_SP_GROUP];
+    for (uint32_t s0 = 0; s0 < steps; s0 += LOADS) {
+      int32_t iv[LOADS];
 #pragma unroll
-      for (int g = 0; g < FV_SP_GROUPS; ++g) {
-        if (s0 + g * FV_SP_GROUP < steps) {  // the same answer in the whole block
+      for (int b = 0; b < LOADS; ++b) iv[b] = idx[ord[min((s0 + b) * FV_SP_WPS + slot, n_staged - 1)] * w + cc];
 #pragma unroll
-          for (int b = 0; b < FV_SP_GROUP; ++b)
-            iv[g][b] = idx[ord[min((s0 + g * FV_SP_GROUP + b) * 16 + slot, n_staged - 1)] * w + cc];
-        }
-      }
-#pragma unroll
-      for (int g = 0; g < FV_SP_GROUPS; ++g) {
-        if (s0 + g * FV_SP_GROUP < steps) {
-#pragma unroll
-          for (int b = 0; b < FV_SP_GROUP; ++b) {
-            const uint32_t i = (uint32_t)iv[g][b];
-            const uint32_t k = (i >> FV_NB_CLASS_SHIFT) - lo;
-            if (col_ok && (s0 + g * FV_SP_GROUP + b) * 16 + slot < n_staged && i < n_cols &&
-                (i & (FV_NB_CLASSES - 1)) == q && k < span) {
-              if (NARROW)
-                atomicAdd(&cnt[k >> 1], 1u << (16 * (k & 1)));
-              else
-                atomicAdd(&cnt[k], 1u);
-            }
-          }
+      for (int b = 0; b < LOADS; ++b) {
+        const uint32_t i = (uint32_t)iv[b];
+        const uint32_t k = (i >> FV_NB_CLASS_SHIFT) - lo;
+        if (col_ok && (s0 + b) * FV_SP_WPS + slot < n_staged && i < n_cols && (i & (FV_NB_CLASSES - 1)) == q &&
+            k < span) {
+          if (NARROW)
+            atomicAdd(&cnt[k >> 1], 1u << (16 * (k & 1)));
+          else
+            atomicAdd(&cnt[k], 1u);
         }
       }
     }
   }
 }
 
-__global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
+// The same with the number of loads in flight fitted to the number of windows.
+template <bool NARROW>
+__device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, const uint32_t *ord, uint32_t n_staged,
+                                                    const int32_t *__restrict__ idx, uint32_t w, uint32_t n_cols,
+                                                    uint32_t q, uint32_t lo, uint32_t span, uint32_t tid) {
+  if (n_staged <= FV_SP_WPS * 2)
+    fv_sparse_count<NARROW, 2>(cnt, ord, n_staged, idx, w, n_cols, q, lo, span, tid);
+  else if (n_staged <= FV_SP_WPS * 8)
+    fv_sparse_count<NARROW, 8>(cnt, ord, n_staged, idx, w, n_cols, q, lo, span, tid);
+  else
+    fv_sparse_count<NARROW, FV_SP_LOADS>(cnt, ord, n_staged, idx, w, n_cols, q, lo, span, tid);
+}
+
+__global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
   __shared__ uint32_t cnt[FV_NB_CNT_WORDS];
   __shared__ uint16_t list[FV_SP_LIST_CAP];
   __shared__ uint32_t ord[FV_SP_STAGE];
   __shared__ uint32_t sh_pos;
-  constexpr uint32_t T = 256;
+  __shared__ float wave_max[16];
+  constexpr uint32_t T = FV_SP_THREADS;
   const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT;
   const uint32_t q = blockIdx.x & (FV_NB_CLASSES - 1);
   const uint32_t tid = threadIdx.x;
@@ -439,9 +450,9 @@ __global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
         fv_lds_barrier();
       }
       if (narrow)
-        fv_sparse_count<true>(cnt, ord, n_staged, a.idx, a.w, n_cols, q, lo, span, tid);
+        fv_sparse_count_any<true>(cnt, ord, n_staged, a.idx, a.w, n_cols, q, lo, span, tid);
       else
-        fv_sparse_count<false>(cnt, ord, n_staged, a.idx, a.w, n_cols, q, lo, span, tid);
+        fv_sparse_count_any<false>(cnt, ord, n_staged, a.idx, a.w, n_cols, q, lo, span, tid);
     }
     // Every non-zero counter is one distinct element. Their positions are collected in LDS, up to
     // FV_SP_LIST_CAP at a time; a counter is cleared when its element is taken, so what did not fit
@@ -452,11 +463,14 @@ __global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
       fv_lds_barrier();
       {
         // bit 8 * i + u of `mine`: counter u of the thread's i-th group of four words is non-zero
-        static_assert(FV_NB_CNT_WORDS == 4 * 5 * 256, "five groups of four counter words per thread");
+        constexpr int n_groups = (FV_NB_CNT_WORDS / 4 + T - 1) / T;
+        static_assert(n_groups <= 8, "a 64-bit mask holds eight groups");
         uint64_t mine = 0;
 #pragma unroll
-        for (int i = 0; i < 5; ++i) {
-          const uint4 c4 = ((const uint4 *)cnt)[tid + i * T];
+        for (int i = 0; i < n_groups; ++i) {
+          const uint32_t g4 = min(tid + i * T, (uint32_t)FV_NB_CNT_WORDS / 4 - 1);
+          uint4 c4 = ((const uint4 *)cnt)[g4];
+          if (tid + i * T >= FV_NB_CNT_WORDS / 4) c4 = make_uint4(0, 0, 0, 0);
           const uint32_t cw[4] = {c4.x, c4.y, c4.z, c4.w};
           uint32_t bits = 0;
 #pragma unroll
@@ -531,7 +545,7 @@ __global__ __launch_bounds__(256) void fv_sparse_kernel(fv_sparse_args a) {
       fv_lds_barrier();
     } while (found > FV_SP_LIST_CAP);
   }
-  const float bm = fv_block_max_nonneg(ds_max, (float *)cnt);
+  const float bm = fv_block_max_nonneg(ds_max, wave_max);
   if (tid == 0) {
     a.bmax_sparse[blockIdx.x] = bm;
     a.slot_count[blockIdx.x] = emitted;
@@ -1062,7 +1076,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.ldk = t->ldk;
   sp.w = t->w;
   sp.V = (uint32_t)t->V;
-  if (which & 4u) hipLaunchKernelGGL(fv_sparse_kernel, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, sp);
+  if (which & 4u) hipLaunchKernelGGL(fv_sparse_kernel, dim3(t->K * FV_NB_CLASSES), dim3(FV_SP_THREADS), 0, t->stream, sp);
   if (ev) FV_HIP(hipEventRecord(ev[3], t->stream));
   fv_dense_args d;
   d.Wt4 = (float4 *)t->Wt;
