@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
 #define FV_SP_CHUNK 16          // window positions read by 16 neighbouring lanes (idx is padded by this much)
 #define FV_SP_STAGE 2048        // window ids staged in LDS at a time
 #ifndef FV_SP_THREADS
-#define FV_SP_THREADS 512       // threads of a class block
+#define FV_SP_THREADS 256       // threads of a class block
 #endif
 #ifndef FV_SP_LOADS
 #define FV_SP_LOADS 24          // most loads a lane has in flight in the counting pass
