@@ -61,10 +61,10 @@ def test_small_config_bit_exact(gpu, oracle_lib, tie):
 
 @pytest.mark.parametrize("K,w,V,B", [(5, 3, 40, 64), (63, 1, 100, 128), (64, 5, 100, 100), (65, 15, 200, 256),
                                      (130, 64, 300, 64), (1000, 15, 300, 512), (2048, 7, 64, 128),
-                                     (30, 11, 20000, 700), (30, 11, 30000, 700)])
+                                     (30, 11, 20000, 700), (30, 11, 30000, 700), (3, 5, 400000, 300)])
 def test_shapes_bit_exact(gpu, oracle_lib, K, w, V, B):
-    # K not a multiple of 64 / 4, every lane-count template, w from 1 to 64, and (last case) more
-    # columns per class than one LDS counting pass of the sparse kernel holds (2V / 4 > 10240)
+    # K not a multiple of 64 / 4, every lane-count template, w from 1 to 64; the last cases have more
+    # columns per class than one pass over the LDS counters of the sparse kernel holds (2V / 4 > 10240)
     n_tokens = 40000 if V < 20000 else 120000
     wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=V, K=K, w=w, B=B, steps=6, n_tokens=n_tokens, mean_chunk=40)
     assert np.array_equal(wg, wo)
