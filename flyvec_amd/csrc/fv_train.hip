@@ -40,10 +40,11 @@
 // NaN with a payload no arithmetic produces.
 #define FV_SENTINEL 0x7fc5ca1eu
 
-struct fv_slot {
+struct __attribute__((aligned(16))) fv_slot {
   uint32_t p;  // element index i * ldk + h
   uint32_t n;  // pending additions of 1/f
   float wv;    // the weight the sentinel replaced
+  float f;     // 1/f of the element's token
 };
 
 struct fv_trainer {
@@ -536,6 +537,7 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
             rec.p = pe[u];
             rec.n = ne[u];
             rec.wv = wv[u];
+            rec.f = fe[u];
             slots[emitted + eb + u * T] = rec;
             a.Wt[pe[u]] = __uint_as_float(FV_SENTINEL);
             if (x_h != 0.0f) ds_max = fv_absmax_keep(ds_max, fv_sparse_ds(x_h, wv[u], fe[u], ne[u]));
@@ -710,15 +712,20 @@ __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
   const float x = a.xx[h];
   const float nc = a.scalars[0];
   const float s = a.prec > nc ? a.eps / a.prec : a.eps / nc;
-  for (uint32_t e = threadIdx.x; e < count; e += 256) {
-    const fv_slot sl = slots[e];
-    float out = sl.wv;  // a row with xx == 0 is not updated: the saved weight goes back
-    if (x != 0.0f) {
-      const uint32_t i = sl.p / a.ldk;
-      const float d = __fmul_rn(s, fv_sparse_ds(x, sl.wv, a.invf[i >= a.V ? i - a.V : i], sl.n));
-      if (fabsf(d) > a.update_cut) out = __fadd_rn(sl.wv, d);
+  for (uint32_t eb = threadIdx.x; eb < count; eb += 4 * 256) {  // four records in flight per thread
+    fv_slot sl[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) sl[u] = slots[min(eb + u * 256, count - 1)];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (eb + u * 256 >= count) break;
+      float out = sl[u].wv;  // a row with xx == 0 is not updated: the saved weight goes back
+      if (x != 0.0f) {
+        const float d = __fmul_rn(s, fv_sparse_ds(x, sl[u].wv, sl[u].f, sl[u].n));
+        if (fabsf(d) > a.update_cut) out = __fadd_rn(sl[u].wv, d);
+      }
+      ((float *)a.Wt4)[sl[u].p] = out;
     }
-    ((float *)a.Wt4)[sl.p] = out;
   }
 }
 
