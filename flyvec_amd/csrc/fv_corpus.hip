@@ -322,3 +322,67 @@ extern "C" int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, ui
   (void)hipFree(df);
   return rc;
 }
+
+// ---- masking of token ids ---------------------------------------------------------------------------
+// The reference removes stop words from an encoded corpus off line, one pass over the whole corpus
+// per id (flyvec/src/remove_words.cpp:28-37: data[w] == id ? -1). Here a bit per vocabulary id
+// marks the ids to remove and one pass rewrites the corpus, a part of bounded size at a time so that a
+// corpus larger than the device's free memory streams through.
+
+__global__ __launch_bounds__(256) void fv_mark_ids_kernel(const int32_t *__restrict__ remove, uint64_t n_remove,
+                                                          uint64_t vocab, uint32_t *__restrict__ bits) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n_remove; i += (uint64_t)gridDim.x * 256) {
+    const int32_t id = remove[i];
+    if (id >= 0 && (uint64_t)id < vocab) atomicOr(&bits[id >> 5], 1u << (id & 31));
+  }
+}
+
+__global__ __launch_bounds__(256) void fv_mask_tokens_kernel(int32_t *__restrict__ tokens, uint64_t n,
+                                                             const uint32_t *__restrict__ bits, uint64_t vocab) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
+    const int32_t t = tokens[i];
+    if (t >= 0 && (uint64_t)t < vocab && ((bits[t >> 5] >> (t & 31)) & 1u)) tokens[i] = -1;
+  }
+}
+
+#define FV_MASK_PART (64ull << 20)  // tokens per part (256 MB)
+
+extern "C" int fv_mask_tokens(int32_t *tokens, uint64_t n_tokens, const int32_t *remove_ids, uint64_t n_remove,
+                              uint64_t vocab) {
+  FV_REQUIRE(tokens || n_tokens == 0, FV_ERR_INVALID, "fv_mask_tokens: null corpus");
+  FV_REQUIRE(remove_ids || n_remove == 0, FV_ERR_INVALID, "fv_mask_tokens: null id list");
+  FV_REQUIRE(vocab >= 1 && vocab <= (1ull << 31), FV_ERR_INVALID, "fv_mask_tokens: vocabulary of %llu ids",
+             (unsigned long long)vocab);
+  if (n_tokens == 0 || n_remove == 0) return FV_OK;
+  for (uint64_t i = 0; i < n_remove; ++i)
+    FV_REQUIRE(remove_ids[i] >= 0 && (uint64_t)remove_ids[i] < vocab, FV_ERR_DATA,
+               "fv_mask_tokens: id %d is outside the vocabulary of %llu", remove_ids[i], (unsigned long long)vocab);
+  const uint64_t words = (vocab + 31) / 32;
+  const uint64_t part = n_tokens < FV_MASK_PART ? n_tokens : FV_MASK_PART;
+  uint32_t *bits = nullptr;
+  int32_t *rem = nullptr, *buf = nullptr;
+  hipError_t e = hipMalloc((void **)&bits, words * sizeof(uint32_t));
+  if (e == hipSuccess) e = hipMalloc((void **)&rem, n_remove * sizeof(int32_t));
+  if (e == hipSuccess) e = hipMalloc((void **)&buf, part * sizeof(int32_t));
+  if (e == hipSuccess) e = hipMemset(bits, 0, words * sizeof(uint32_t));
+  if (e == hipSuccess) e = hipMemcpy(rem, remove_ids, n_remove * sizeof(int32_t), hipMemcpyHostToDevice);
+  if (e == hipSuccess) {
+    const unsigned blocks = (unsigned)((n_remove + 255) / 256 < 1024 ? (n_remove + 255) / 256 : 1024);
+    hipLaunchKernelGGL(fv_mark_ids_kernel, dim3(blocks), dim3(256), 0, 0, rem, n_remove, vocab, bits);
+    e = hipGetLastError();
+  }
+  for (uint64_t first = 0; e == hipSuccess && first < n_tokens; first += part) {
+    const uint64_t n = n_tokens - first < part ? n_tokens - first : part;
+    e = hipMemcpy(buf, tokens + first, n * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (e != hipSuccess) break;
+    const unsigned blocks = (unsigned)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
+    hipLaunchKernelGGL(fv_mask_tokens_kernel, dim3(blocks), dim3(256), 0, 0, buf, n, bits, vocab);
+    e = hipGetLastError();
+    if (e == hipSuccess) e = hipMemcpy(tokens + first, buf, n * sizeof(int32_t), hipMemcpyDeviceToHost);
+  }
+  (void)hipFree(bits);
+  (void)hipFree(rem);
+  (void)hipFree(buf);
+  if (e != hipSuccess) return fv_fail(FV_ERR_HIP, "fv_mask_tokens failed: %s", hipGetErrorString(e));
+  return FV_OK;
+}

@@ -79,6 +79,13 @@ int fv_build_window_starts(const uint64_t *offsets, uint64_t n_chunks, uint64_t 
  * reference's fp32 counter does. */
 int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, uint64_t vocab, float *out_invf);
 
+/* flyvec/src/remove_words.cpp:28-37 (an off-line tool of the reference: for every id of a stop list,
+ * data[w] == id ? -1): rewrites `tokens` in place, every occurrence of an id of `remove_ids`
+ * becomes -1 (masked: such a position contributes nothing to a window). One pass on the device,
+ * whatever the length of the list; ids must lie in [0, vocab). */
+int fv_mask_tokens(int32_t *tokens, uint64_t n_tokens, const int32_t *remove_ids, uint64_t n_remove,
+                   uint64_t vocab);
+
 /* ---- trainer ------------------------------------------------------------------ */
 
 typedef struct fv_trainer fv_trainer;

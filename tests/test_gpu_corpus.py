@@ -1,0 +1,62 @@
+"""Device half of flyvec_amd/corpus.py: stop-word masking (flyvec/src/remove_words.cpp:28-37) against
+numpy, and the encoder's shards carried through merge -> flyvec_train."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_mask_tokens_equals_numpy(gpu):
+    from flyvec_amd import corpus
+    rng = np.random.default_rng(0)
+    V = 5000
+    tokens = rng.integers(-1, V, size=300_001).astype(np.int32)
+    remove = rng.choice(V, size=419, replace=False).astype(np.int32)   # the reference's list has 419 ids
+    want = tokens.copy()
+    want[np.isin(want, remove)] = -1
+    got = corpus.mask_tokens(tokens.copy(), remove, vocab=V)
+    assert np.array_equal(got, want)
+    assert np.array_equal(corpus.mask_tokens(got.copy(), remove, vocab=V), want)          # idempotent
+    assert np.array_equal(corpus.mask_tokens(tokens.copy(), np.zeros(0, np.int32), vocab=V), tokens)
+    assert np.array_equal(corpus.mask_tokens(tokens.copy(), np.repeat(remove[:3], 5), vocab=V),
+                          np.where(np.isin(tokens, remove[:3]), -1, tokens))               # duplicates in the list
+
+
+def test_mask_tokens_errors(gpu):
+    from flyvec_amd import _lib, corpus
+    tokens = np.arange(10, dtype=np.int32)
+    with pytest.raises(_lib.FlyvecError) as e:
+        corpus.mask_tokens(tokens, np.array([3, 99], dtype=np.int32), vocab=10)
+    assert e.value.code == _lib.FV_ERR_DATA
+    with pytest.raises(ValueError):
+        corpus.mask_tokens(tokens.astype(np.int64), [1])
+
+
+def test_shards_to_checkpoint(gpu, tmp_path):
+    from flyvec_amd import corpus
+    from flyvec_amd.train_flyvec import main as train_main
+    rng = np.random.default_rng(3)
+    V = 200
+    shard_dir = tmp_path / "shards"
+    shard_dir.mkdir()
+    for stem in ("part0", "part1", "part2"):
+        lens = rng.integers(5, 40, size=150)
+        ids = rng.integers(1, V, size=int(lens.sum())).astype(np.int32)
+        ids[-1] = V - 1
+        np.save(shard_dir / f"{stem}.npy", ids)
+        np.save(shard_dir / f"{stem}_offsets.npy", np.cumsum(lens).astype(np.uint64))   # ends, no leading 0
+    stop = np.array([1, 2, 3], dtype=np.int32)
+    np.save(tmp_path / "stop.npy", stop)
+    corpus.main(["merge", str(shard_dir), "-o", str(tmp_path / "merged"), "--stop-ids", str(tmp_path / "stop.npy")])
+    tokens = np.load(tmp_path / "merged" / "encodings.npy")
+    offsets = np.load(tmp_path / "merged" / "offsets.npy")
+    assert not np.isin(tokens, stop).any() and (tokens == -1).any()
+    assert offsets[0] == 0 and offsets[-1] == len(tokens) and len(offsets) == 3 * 150 + 1
+    out = tmp_path / "ckpt"
+    assert train_main([str(tmp_path / "merged" / "encodings.npy"), str(tmp_path / "merged" / "offsets.npy"),
+                       "-o", str(out), "--hid", "32", "-b", "128", "--Nep", "1", "--seed", "0"]) == 0
+    (ckpt,) = list(out.iterdir())
+    W = np.load(ckpt)
+    assert W.shape == (32, 2 * V) and np.isfinite(W).all()
+    # masked ids never enter a window: their context and target columns keep their initial spread
+    assert np.abs(W[:, stop]).max() < 0.2
