@@ -54,6 +54,14 @@ class FlyVec:
         if normalize_synapses:
             self.hasher.normalize()  # flyvec/core.py:87
         self._synapses = None
+        self._stop_ids = None
+
+    @classmethod
+    def load(cls, force_redownload=False):
+        """flyvec/core.py:50-60 downloads the pretrained model from a bucket; this package fetches
+        nothing. Unpack the model directory yourself and use ``from_config``."""
+        raise NotImplementedError("FlyVec.load() downloads data in the reference; use FlyVec.from_config("
+                                  "'<model dir>/config.yaml', tokenizer=...) on a local copy")
 
     @classmethod
     def from_config(cls, fname: Union[Path, str], tokenizer=None):
@@ -89,8 +97,25 @@ class FlyVec:
         return list(self.tokenizer.vocab) if hasattr(self.tokenizer, "vocab") else \
             [self.tokenizer.id2token(i) for i in range(self.tokenizer.n_vocab())]
 
+    @property
+    def vocab(self):
+        return self.tokenizer.vocab
+
+    @property
+    def dictionary(self):
+        return self.tokenizer.dictionary
+
+    @property
     def stop_word_ids(self):
-        return set(np.load(self.stopword_file)) if self.stopword_file else set()
+        """Token ids the model should not respond to (flyvec/core.py:109-112); empty without a file."""
+        if self._stop_ids is None:
+            self._stop_ids = set(int(i) for i in np.load(self.stopword_file)) if self.stopword_file else set()
+        return self._stop_ids
+
+    @property
+    def stop_words(self):
+        """flyvec/core.py:114-117."""
+        return set(self.tokenizer.id2token(t) for t in self.stop_word_ids)
 
     @property
     def unknown_embedding_info(self):
@@ -145,7 +170,7 @@ class FlyVec:
         vocab = self.token_vocab
         ids = np.array([self.tokenizer.token2id(self.tokenizer.tokenize(t)[0]) if len(t) else -1
                         for t in vocab], dtype=np.int64)
-        stop = self.stop_word_ids() if exclude_stop_words else set()
+        stop = self.stop_word_ids if exclude_stop_words else set()
         good = ids > 0
         codes = self.hasher.hash_targets(ids[good].astype(np.int32), k) if good.any() else None
         out = {}
@@ -163,3 +188,12 @@ class FlyVec:
                 continue
             out[t] = list(vec) if output_list else vec
         return out
+
+    def export_simple_embeddings(self, path, k: int = 50, exclude_stop_words=False):
+        """Writes ``simple_word_vectors(k, output_list=True)`` as JSON: token -> list of 0/1, the
+        context-independent artefact the reference's README describes (README.md:132-138)."""
+        import json
+        vecs = self.simple_word_vectors(k, exclude_stop_words=exclude_stop_words, output_list=True)
+        with open(path, "w") as fp:
+            json.dump({t: [int(x) for x in v] for t, v in vecs.items()}, fp)
+        return len(vecs)

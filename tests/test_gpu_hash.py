@@ -154,3 +154,30 @@ def test_flyvec_wrapper_semantics(gpu, tmp_path):
     assert np.array_equal(vecs["world"], ho.sparse_code(Wn[:, V + 2], 20)) and not vecs["<UNK>"].any()
     win = np.array([[1, 2, V + 3, 4, -1]], dtype=np.int32)
     assert np.array_equal(model.get_context_embeddings(win, 30), ho.hash_windows(Wn, win, 30))
+
+
+def test_flyvec_wrapper_stop_words_and_export(gpu, tmp_path):
+    """stop_word_ids / stop_words are attributes as in the reference (flyvec/core.py:109-117);
+    exclude_stop_words drops them from the whole-vocabulary table; the table exports as JSON."""
+    import json
+    from flyvec_amd import FlyVec
+    from oracle import hash_oracle as ho
+    rng = np.random.default_rng(9)
+    vocab = ["<UNK>", "the", "of", "fly", "brain"] + [f"tok{i}" for i in range(45)]
+    K, V = 128, len(vocab)
+    W = rng.standard_normal((K, 2 * V)).astype(f32)
+    np.save(tmp_path / "model.npy", W)
+    np.save(tmp_path / "stop.npy", np.array([1, 2], dtype=np.int64))
+    (tmp_path / "config.yaml").write_text("synapses: model.npy\nstop_words: stop.npy\ntokenizer: tok.pkl\n")
+    model = FlyVec.from_config(tmp_path / "config.yaml", tokenizer=vocab)       # normalize_synapses defaults to False
+    assert model.stop_word_ids == {1, 2} and model.stop_words == {"the", "of"}
+    assert model.vocab == vocab and model.n_vocab == V and model.n_neurons == K
+    assert np.array_equal(model.synapses, W)
+    kept = model.simple_word_vectors(k=10, exclude_stop_words=True)
+    assert set(kept) == set(vocab) - {"the", "of"}
+    n = model.export_simple_embeddings(tmp_path / "simple.json", k=10)
+    table = json.loads((tmp_path / "simple.json").read_text())
+    assert n == V and set(table) == set(vocab)
+    assert table["brain"] == ho.sparse_code(W[:, V + 4], 10).astype(int).tolist() and sum(table["brain"]) == 10
+    with pytest.raises(NotImplementedError):
+        FlyVec.load()
