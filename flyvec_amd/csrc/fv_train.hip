@@ -57,6 +57,7 @@ struct fv_trainer {
   int32_t *corpus;
   uint64_t n_tokens;
   uint64_t *starts, *perm;
+  uint64_t *pstart;    // starts[perm[i]]: where the i-th window of the current order begins
   uint64_t *perm_alt;  // second permutation buffer, allocated by the first shuffle
   uint64_t n_windows;
   float *invf;
@@ -85,8 +86,7 @@ struct fv_trainer {
 struct fv_gather_args {
   const float *Wt;
   const int32_t *corpus;
-  const uint64_t *starts;
-  const uint64_t *perm;
+  const uint64_t *pstart;  // start of every window, in the current order
   const float *invf;
   int32_t *idx;
   int32_t *win;
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
   // sampler: lane c holds column index c of the window (flyvec/src/cuda_funcs.cu:915-936)
   int32_t idx = -1;
   if (lane < (int)a.w) {
-    const uint64_t s = a.starts[a.perm[a.first + r]];
+    const uint64_t s = a.pstart[a.first + r];
     const int32_t tok = a.corpus[s + lane];
     idx = tok < 0 ? -1 : (lane == (int)(a.w / 2) ? tok + (int32_t)a.V : tok);
     a.idx[(uint64_t)r * a.w + lane] = idx;
@@ -760,6 +760,14 @@ __global__ __launch_bounds__(256) void fv_shuffle_kernel(const uint64_t *__restr
     out[i] = in[fv_permute_index(&f, i, n)];
 }
 
+// The sampler's two look-ups (order -> window -> start) folded into one table whenever the order changes.
+__global__ __launch_bounds__(256) void fv_order_starts_kernel(const uint64_t *__restrict__ perm,
+                                                              const uint64_t *__restrict__ starts,
+                                                              uint64_t *__restrict__ pstart, uint64_t n) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256)
+    pstart[i] = starts[perm[i]];
+}
+
 static unsigned fv_perm_blocks(uint64_t n) {
   const uint64_t want = (n + 255) / 256;
   return (unsigned)(want < 8192 ? want : 8192);
@@ -772,9 +780,10 @@ static void fv_trainer_free_corpus(fv_trainer *t) {
   (void)hipFree(t->starts);
   (void)hipFree(t->perm);
   (void)hipFree(t->perm_alt);
+  (void)hipFree(t->pstart);
   (void)hipFree(t->invf);
   t->corpus = nullptr;
-  t->starts = t->perm = t->perm_alt = nullptr;
+  t->starts = t->perm = t->perm_alt = t->pstart = nullptr;
   t->invf = nullptr;
   t->n_tokens = t->n_windows = 0;
   t->have_corpus = false;
@@ -905,6 +914,7 @@ extern "C" int fv_trainer_set_corpus(fv_trainer *t, const int32_t *tokens, uint6
   if (rc == FV_OK && nwin) {
     e = hipMalloc((void **)&t->starts, nwin * sizeof(uint64_t));
     if (e == hipSuccess) e = hipMalloc((void **)&t->perm, nwin * sizeof(uint64_t));
+    if (e == hipSuccess) e = hipMalloc((void **)&t->pstart, nwin * sizeof(uint64_t));
     if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "window table allocation failed: %s", hipGetErrorString(e));
     if (rc == FV_OK) {
       // Starts are sums of chunk lengths: with non-decreasing offsets that span no more than the
@@ -920,6 +930,8 @@ extern "C" int fv_trainer_set_corpus(fv_trainer *t, const int32_t *tokens, uint6
     if (rc == FV_OK) rc = fv_dev_build_window_starts(off_dev, n_chunks, t->w, t->starts, nwin, t->stream);
     if (rc == FV_OK) {
       hipLaunchKernelGGL(fv_identity_kernel, dim3(fv_perm_blocks(nwin)), dim3(256), 0, t->stream, t->perm, nwin);
+      hipLaunchKernelGGL(fv_order_starts_kernel, dim3(fv_perm_blocks(nwin)), dim3(256), 0, t->stream, t->perm,
+                         t->starts, t->pstart, nwin);
       e = hipStreamSynchronize(t->stream);
       if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "permutation fill failed: %s", hipGetErrorString(e));
     }
@@ -987,6 +999,9 @@ extern "C" int fv_trainer_shuffle(fv_trainer *t, uint64_t seed) {
   hipLaunchKernelGGL(fv_shuffle_kernel, dim3(fv_perm_blocks(n)), dim3(256), 0, t->stream, t->perm, t->perm_alt, n, f);
   FV_HIP(hipGetLastError());
   std::swap(t->perm, t->perm_alt);
+  hipLaunchKernelGGL(fv_order_starts_kernel, dim3(fv_perm_blocks(n)), dim3(256), 0, t->stream, t->perm, t->starts,
+                     t->pstart, n);
+  FV_HIP(hipGetLastError());
   t->shuffle_calls++;
   return FV_OK;
 }
@@ -1003,6 +1018,9 @@ extern "C" int fv_trainer_set_permutation(fv_trainer *t, const uint64_t *perm, u
                (unsigned long long)i, (unsigned long long)perm[i]);
   FV_HIP(hipStreamSynchronize(t->stream));
   FV_HIP(hipMemcpy(t->perm, perm, n * sizeof(uint64_t), hipMemcpyHostToDevice));
+  hipLaunchKernelGGL(fv_order_starts_kernel, dim3(fv_perm_blocks(n)), dim3(256), 0, t->stream, t->perm, t->starts,
+                     t->pstart, n);
+  FV_HIP(hipGetLastError());
   return FV_OK;
 }
 
@@ -1031,8 +1049,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   fv_gather_args g;
   g.Wt = t->Wt;
   g.corpus = t->corpus;
-  g.starts = t->starts;
-  g.perm = t->perm;
+  g.pstart = t->pstart;
   g.invf = t->invf;
   g.idx = t->idx;
   g.win = t->win;
