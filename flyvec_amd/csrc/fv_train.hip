@@ -173,13 +173,14 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
 #define FV_NB_CLASSES (1 << FV_NB_CLASS_SHIFT)  // column classes per neuron (kernel 3)
 #define FV_NB_CNT_WORDS 5120    // LDS counter words per class block (20 KB)
 #define FV_SP_LIST_CAP 1024     // positions of non-zero counters collected in LDS at a time
-#define FV_SP_CHUNK 16          // window positions read by 16 neighbouring lanes (idx is padded by this much)
+#define FV_SP_CHUNK 16          // window positions read by 16 neighbouring lanes
+#define FV_IDX_PAD 80            // entries of -1 behind the index matrix: a padding row plus a chunk
 #define FV_SP_STAGE 2048        // window ids staged in LDS at a time
 #ifndef FV_SP_THREADS
 #define FV_SP_THREADS 256       // threads of a class block
 #endif
 #ifndef FV_SP_LOADS
-#define FV_SP_LOADS 24          // most loads a lane has in flight in the counting pass
+#define FV_SP_LOADS 16          // most loads a lane has in flight in the counting pass
 #endif
 #define FV_NB_ROUND 2048        // scaled activations staged in LDS at a time
 #define FV_NB_LOADS 16          // independent loads issued together
@@ -340,7 +341,7 @@ struct fv_sparse_args {
   const uint32_t *order;
   const uint32_t *group_base;
   const uint32_t *group_count;
-  const int32_t *idx;  // readable FV_SP_CHUNK entries past its end
+  const int32_t *idx;  // followed by FV_IDX_PAD entries of -1
   float *Wt;
   fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records
   uint64_t slot_stride;
@@ -348,59 +349,66 @@ struct fv_sparse_args {
   const float *invf;
   float *bmax_sparse;    // one maximum of |ds| per block
   uint32_t *slot_count;  // records written per block
-  uint32_t ldk, w, V;
+  uint32_t ldk, w, V, pad_row;  // pad_row: the row index just behind the index matrix
 };
 
 // Barrier for data exchanged through LDS only: waits for the wave's LDS operations, not for its
 // global stores still in flight.
 __device__ __forceinline__ void fv_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// Counting pass of one class block over the windows whose ids are staged in LDS (ord[0 .. n_staged)).
-// Sixteen consecutive lanes read sixteen consecutive positions of one window, so a wave's load
-// touches four rows of the index matrix; positions past the window (the next row, or the padding
-// behind the last one) are loaded and dropped. A lane issues LOADS loads back to back with no
-// branch between them (the compiler waits for every load in flight at a branch target), then counts.
+// Counting pass of one class block over the windows whose ids are staged in LDS: ord[0 .. n_staged),
+// followed up to the next multiple of 16 * LOADS by the id of the padding row behind the index
+// matrix (all -1). Sixteen consecutive lanes read sixteen consecutive positions of one window, so a
+// wave's load touches four rows; positions past the window (the next row or the padding) are
+// loaded and dropped. A lane issues LOADS loads back to back with no branch between them (the
+// compiler waits for every load in flight at a branch target), then counts. With the class in the
+// top bits and the column of the class below, one subtraction and one comparison tell whether an
+// entry is this block's: of class q, inside [lo, lo + span), not masked, not dropped.
 #define FV_SP_WPS (FV_SP_THREADS / 16)  // windows the block takes per step
 template <bool NARROW, int LOADS>
 __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const uint32_t *ord, uint32_t n_staged,
-                                                const int32_t *__restrict__ idx, uint32_t w, uint32_t n_cols,
-                                                uint32_t q, uint32_t lo, uint32_t span, uint32_t tid) {
+                                                const int32_t *__restrict__ idx, uint32_t w, uint32_t q,
+                                                uint32_t lo, uint32_t span, uint32_t tid) {
   const uint32_t c = tid & 15u, slot = tid >> 4;
   const uint32_t steps = (n_staged + FV_SP_WPS - 1) / FV_SP_WPS;
+  const uint32_t origin = (q << (32 - FV_NB_CLASS_SHIFT)) | lo;
   for (uint32_t c0 = 0; c0 < w; c0 += FV_SP_CHUNK) {
     const uint32_t cc = c0 + c;
-    const bool col_ok = cc < w;
+    const uint32_t drop = cc < w ? 0u : 0xffffffffu;
     for (uint32_t s0 = 0; s0 < steps; s0 += LOADS) {
       int32_t iv[LOADS];
 #pragma unroll
-      for (int b = 0; b < LOADS; ++b) iv[b] = idx[ord[min((s0 + b) * FV_SP_WPS + slot, n_staged - 1)] * w + cc];
+      for (int b = 0; b < LOADS; ++b) iv[b] = idx[ord[(s0 + b) * FV_SP_WPS + slot] * w + cc];
 #pragma unroll
       for (int b = 0; b < LOADS; ++b) {
-        const uint32_t i = (uint32_t)iv[b];
-        const uint32_t k = (i >> FV_NB_CLASS_SHIFT) - lo;
-        if (col_ok && (s0 + b) * FV_SP_WPS + slot < n_staged && i < n_cols && (i & (FV_NB_CLASSES - 1)) == q &&
-            k < span) {
+        const uint32_t t = __builtin_rotateright32((uint32_t)iv[b] | drop, FV_NB_CLASS_SHIFT) - origin;
+        if (t < span) {
           if (NARROW)
-            atomicAdd(&cnt[k >> 1], 1u << (16 * (k & 1)));
+            atomicAdd(&cnt[t >> 1], 1u << (16 * (t & 1)));
           else
-            atomicAdd(&cnt[k], 1u);
+            atomicAdd(&cnt[t], 1u);
         }
       }
     }
   }
 }
 
-// The same with the number of loads in flight fitted to the number of windows.
+// The same with the number of loads in flight fitted to the number of windows; pads ord[].
 template <bool NARROW>
-__device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, const uint32_t *ord, uint32_t n_staged,
-                                                    const int32_t *__restrict__ idx, uint32_t w, uint32_t n_cols,
-                                                    uint32_t q, uint32_t lo, uint32_t span, uint32_t tid) {
-  if (n_staged <= FV_SP_WPS * 2)
-    fv_sparse_count<NARROW, 2>(cnt, ord, n_staged, idx, w, n_cols, q, lo, span, tid);
-  else if (n_staged <= FV_SP_WPS * 8)
-    fv_sparse_count<NARROW, 8>(cnt, ord, n_staged, idx, w, n_cols, q, lo, span, tid);
+__device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, uint32_t *ord, uint32_t n_staged, uint32_t pad_row,
+                                                    const int32_t *__restrict__ idx, uint32_t w, uint32_t q,
+                                                    uint32_t lo, uint32_t span, uint32_t tid) {
+  static_assert(FV_SP_STAGE % (FV_SP_WPS * FV_SP_LOADS) == 0 && FV_SP_LOADS % 8 == 0, "padding of ord[] stays inside it");
+  const uint32_t per = FV_SP_WPS * (n_staged <= FV_SP_WPS * 2 ? 2 : n_staged <= FV_SP_WPS * 8 ? 8 : FV_SP_LOADS);
+  const uint32_t padded = (n_staged + per - 1) / per * per;
+  for (uint32_t i = n_staged + tid; i < padded; i += FV_SP_THREADS) ord[i] = pad_row;
+  fv_lds_barrier();
+  if (per == FV_SP_WPS * 2)
+    fv_sparse_count<NARROW, 2>(cnt, ord, n_staged, idx, w, q, lo, span, tid);
+  else if (per == FV_SP_WPS * 8)
+    fv_sparse_count<NARROW, 8>(cnt, ord, n_staged, idx, w, q, lo, span, tid);
   else
-    fv_sparse_count<NARROW, FV_SP_LOADS>(cnt, ord, n_staged, idx, w, n_cols, q, lo, span, tid);
+    fv_sparse_count<NARROW, FV_SP_LOADS>(cnt, ord, n_staged, idx, w, q, lo, span, tid);
 }
 
 __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
@@ -451,9 +459,9 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
         fv_lds_barrier();
       }
       if (narrow)
-        fv_sparse_count_any<true>(cnt, ord, n_staged, a.idx, a.w, n_cols, q, lo, span, tid);
+        fv_sparse_count_any<true>(cnt, ord, n_staged, a.pad_row, a.idx, a.w, q, lo, span, tid);
       else
-        fv_sparse_count_any<false>(cnt, ord, n_staged, a.idx, a.w, n_cols, q, lo, span, tid);
+        fv_sparse_count_any<false>(cnt, ord, n_staged, a.pad_row, a.idx, a.w, q, lo, span, tid);
     }
     // Every non-zero counter is one distinct element. Their positions are collected in LDS, up to
     // FV_SP_LIST_CAP at a time; a counter is cleared when its element is taken, so what did not fit
@@ -814,8 +822,8 @@ static int fv_trainer_alloc(fv_trainer *t) {
   const size_t elems = (size_t)t->N * t->ldk;
   FV_HIP(hipStreamCreate(&t->stream));
   FV_HIP(hipMalloc((void **)&t->Wt, elems * sizeof(float)));
-  FV_HIP(hipMalloc((void **)&t->idx, ((size_t)t->B * t->w + FV_SP_CHUNK) * sizeof(int32_t)));
-  FV_HIP(hipMemsetAsync(t->idx, 0xff, ((size_t)t->B * t->w + FV_SP_CHUNK) * sizeof(int32_t), t->stream));
+  FV_HIP(hipMalloc((void **)&t->idx, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t)));
+  FV_HIP(hipMemsetAsync(t->idx, 0xff, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t), t->stream));
   FV_HIP(hipMalloc((void **)&t->win, ((size_t)t->B + 16) * sizeof(int32_t)));  // read in 16-byte pieces
   FV_HIP(hipMalloc((void **)&t->sc, (size_t)t->B * sizeof(float)));
   FV_HIP(hipMalloc((void **)&t->order, (size_t)t->B * sizeof(uint32_t)));
@@ -1097,6 +1105,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.invf = t->invf;
   sp.bmax_sparse = t->bmax + t->dense_blocks;
   sp.slot_count = t->slot_count;
+  sp.pad_row = t->B;
   sp.ldk = t->ldk;
   sp.w = t->w;
   sp.V = (uint32_t)t->V;
