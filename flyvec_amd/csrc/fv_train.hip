@@ -63,6 +63,7 @@ struct fv_trainer {
   float *invf;
   int32_t *idx;     // B x w column indices of the current minibatch
   int32_t *win;     // B winners
+  uint16_t *win16;  // the same, 16 bits each (padded by 64)
   float *sc;        // B scaled activations at the winner
   uint32_t *order;  // B window ids grouped by winner, ascending inside a group
   uint32_t *group_base, *group_count;  // K each
@@ -90,6 +91,7 @@ struct fv_gather_args {
   const float *invf;
   int32_t *idx;
   int32_t *win;
+  uint16_t *win16;  // the same winners as 16-bit values, for the grouping kernel
   float *sc;
   uint64_t first;
   uint32_t n, K, ldk, w, V, tie_rule;
@@ -156,6 +158,7 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
   }
   if (lane == 0) {
     a.win[r] = (int32_t)hstar;
+    a.win16[r] = (uint16_t)hstar;
     a.sc[r] = (float)s;
   }
 }
@@ -183,10 +186,10 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
 #define FV_SP_LOADS 16          // most loads a lane has in flight in the counting pass
 #endif
 #define FV_NB_ROUND 2048        // scaled activations staged in LDS at a time
-#define FV_NB_LOADS 16          // independent loads issued together
+#define FV_NB_LOADS 32          // winners a thread of the grouping kernel fetches together
 
 struct fv_group_args {
-  const int32_t *win;  // padded: readable up to n rounded up to 16
+  const uint16_t *win;  // 16-bit winners, padded: readable up to n rounded up to 64
   const float *sc;
   uint32_t *order;
   uint32_t *group_base;
@@ -245,6 +248,39 @@ __device__ __forceinline__ uint32_t fv_block_exclusive_scan(uint32_t v, uint32_t
   return before + incl - v;
 }
 
+// Exclusive prefix sum and total of one value per thread over the block, in one pass.
+__device__ __forceinline__ uint32_t fv_block_scan_total(uint32_t v, uint32_t *smem /*17*/, uint32_t *total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+  uint32_t incl = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t o = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += o;
+  }
+  __syncthreads();
+  if (lane == 63) smem[wave] = incl;
+  __syncthreads();
+  uint32_t before = 0, all = 0;
+  for (int i = 0; i < n_waves; ++i) {
+    const uint32_t t = smem[i];
+    before += i < wave ? t : 0u;
+    all += t;
+  }
+  *total = all;
+  return before + incl - v;
+}
+
+// SMALL: a thread's run is at most 64 windows and the minibatch has fewer than 2^16. The run is then
+// fetched in one trip to memory (16 loads of 16 bytes in flight), the two counts travel through
+// one block scan as the halves of a word, and the scaled activations of a thread's first matches
+// are fetched while that scan runs.
+// Winner number q (0 .. 7) of a 16-byte load of 16-bit winners.
+__device__ __forceinline__ uint32_t fv_winner_of(const int4 &v, int q) {
+  const uint32_t word = (uint32_t)((q >> 1) == 0 ? v.x : (q >> 1) == 1 ? v.y : (q >> 1) == 2 ? v.z : v.w);
+  return (q & 1) ? word >> 16 : word & 0xffffu;
+}
+
+template <bool SMALL>
 __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_args a) {
   __shared__ float scbuf[FV_NB_ROUND];
   __shared__ uint32_t red[17];
@@ -252,72 +288,128 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
   const uint32_t h = blockIdx.x;
   const uint32_t tid = threadIdx.x, T = blockDim.x;
   const uint32_t n = a.n;
-  const int32_t *__restrict__ win = a.win;
+  const uint16_t *__restrict__ win = a.win;
 
-  // A thread's run is a multiple of 4 windows, read as 16-byte loads; matches among its first 64
-  // windows are kept as a bit mask.
-  const uint32_t seg = ((n + T - 1) / T + 3) & ~3u;
+  // A thread's run is a multiple of 8 windows, read as 16-byte loads of 8 winners; matches among
+  // its first 64 windows are kept as a bit mask.
+  const uint32_t seg = ((n + T - 1) / T + 7) & ~7u;
   const uint32_t r0 = min(tid * seg, n), r1 = min(r0 + seg, n);
-  const uint32_t n_pad = (n + 15) & ~15u;
+  const uint32_t n_pad = (n + 63) & ~63u;
   uint32_t lt = 0, eq = 0;
   uint64_t mask = 0;
-  for (uint32_t rb = r0; rb < r1; rb += FV_NB_LOADS) {
-    int4 wv4[FV_NB_LOADS / 4];
+  uint32_t base, my_off, c_h;
+  constexpr int PF = 8;
+  float pf[PF];
+  if (SMALL) {
+    int4 wv4[8];
 #pragma unroll
-    for (int q = 0; q < FV_NB_LOADS / 4; ++q) wv4[q] = *(const int4 *)(win + min(rb + 4 * q, n_pad - 4));
+    for (int q = 0; q < 8; ++q) wv4[q] = *(const int4 *)(win + min(r0 + 8 * q, n_pad - 8));
 #pragma unroll
-    for (int q = 0; q < FV_NB_LOADS; ++q) {
-      const int4 v4 = wv4[q >> 2];
-      const uint32_t wv = (uint32_t)((q & 3) == 0 ? v4.x : (q & 3) == 1 ? v4.y : (q & 3) == 2 ? v4.z : v4.w);
-      const bool in = rb + q < r1;
-      lt += in && wv < h;
-      const bool hit = in && wv == h;
-      eq += hit;
-      const uint32_t o = rb + q - r0;
-      mask |= o < 64 ? (uint64_t)hit << o : 0ull;
+    for (int g = 0; g < 4; ++g) {
+      if (g * 16 < (int)seg) {  // the same answer in the whole block
+#pragma unroll
+        for (int q = 16 * g; q < 16 * g + 16; ++q) {
+          const uint32_t wv = fv_winner_of(wv4[q >> 3], q & 7);
+          const bool in = r0 + q < r1;
+          lt += in && wv < h;
+          const bool hit = in && wv == h;
+          eq += hit;
+          mask |= (uint64_t)hit << q;
+        }
+      }
     }
+    uint64_t mm = mask;
+#pragma unroll
+    for (int q = 0; q < PF; ++q) {
+      const uint32_t r = mm ? r0 + (uint32_t)__ffsll((long long)mm) - 1 : r0;
+      pf[q] = a.sc[min(r, n - 1)];
+      mm &= mm - 1;
+    }
+    uint32_t total;
+    const uint32_t before = fv_block_scan_total(lt | (eq << 16), red, &total);
+    base = total & 0xffffu;
+    c_h = total >> 16;
+    my_off = before >> 16;
+  } else {
+    for (uint32_t rb = r0; rb < r1; rb += FV_NB_LOADS) {
+      int4 wv4[FV_NB_LOADS / 8];
+#pragma unroll
+      for (int q = 0; q < FV_NB_LOADS / 8; ++q) wv4[q] = *(const int4 *)(win + min(rb + 8 * q, n_pad - 8));
+#pragma unroll
+      for (int q = 0; q < FV_NB_LOADS; ++q) {
+        const uint32_t wv = fv_winner_of(wv4[q >> 3], q & 7);
+        const bool in = rb + q < r1;
+        lt += in && wv < h;
+        const bool hit = in && wv == h;
+        eq += hit;
+        const uint32_t o = rb + q - r0;
+        mask |= o < 64 ? (uint64_t)hit << o : 0ull;
+      }
+    }
+    base = fv_block_sum_u32(lt, red);  // windows won by lower neurons
+    my_off = fv_block_exclusive_scan(eq, red);
+    c_h = fv_block_sum_u32(eq, red);
   }
-  const uint32_t base = fv_block_sum_u32(lt, red);  // windows won by lower neurons
-  const uint32_t my_off = fv_block_exclusive_scan(eq, red);
-  const uint32_t c_h = fv_block_sum_u32(eq, red);
   if (tid == 0) {
     a.group_base[h] = base;
     a.group_count[h] = c_h;
   }
+  // SMALL and the neuron's values fit scbuf: they are placed by rank here, without a trip through order[]
+  const bool staged = SMALL && c_h <= FV_NB_ROUND;
   uint32_t *order = a.order + base;
   {
     uint32_t rank = my_off;
     uint64_t mm = mask;
+    if (SMALL) {
+#pragma unroll
+      for (int q = 0; q < PF; ++q) {
+        if (mm) {
+          order[rank] = r0 + (uint32_t)__ffsll((long long)mm) - 1;
+          if (staged) scbuf[rank] = pf[q];
+          ++rank;
+          mm &= mm - 1;
+        }
+      }
+    }
     while (mm) {
-      order[rank++] = r0 + (uint32_t)__ffsll((long long)mm) - 1;
+      const uint32_t r = r0 + (uint32_t)__ffsll((long long)mm) - 1;
+      order[rank] = r;
+      if (staged) scbuf[rank] = a.sc[r];
+      ++rank;
       mm &= mm - 1;
     }
     for (uint32_t r = r0 + 64; r < r1; ++r)
       if ((uint32_t)win[r] == h) order[rank++] = r;
   }
-  __syncthreads();  // the neuron's part of order[] is now readable by the whole block
+  __syncthreads();  // the neuron's part of order[] (and of scbuf) is now readable by the whole block
 
   // xx[h]: lane l of the first wave adds the neuron's scaled activations number l, l + 64, l + 128, ...
   // (window order) onto 0, then the 64 partial sums are added onto 0 in lane order. For up to 64
   // windows that is the plain sum in window order.
   float part = 0.0f;
-  for (uint32_t j0 = 0; j0 < c_h; j0 += FV_NB_ROUND) {
-    const uint32_t mr = min(c_h - j0, (uint32_t)FV_NB_ROUND);
-    for (uint32_t jb = tid; jb < mr; jb += 4 * T) {  // up to 4 independent loads per thread
-      uint32_t r[4];
-      float v[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) r[q] = order[j0 + min(jb + q * T, mr - 1)];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) v[q] = a.sc[r[q]];
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (jb + q * T < mr) scbuf[jb + q * T] = v[q];
-    }
-    __syncthreads();
+  if (staged) {
     if (tid < 64)
-      for (uint32_t j = tid; j < mr; j += 64) part = __fadd_rn(part, scbuf[j]);  // FV_NB_ROUND % 64 == 0
+      for (uint32_t j = tid; j < c_h; j += 64) part = __fadd_rn(part, scbuf[j]);
     __syncthreads();
+  } else {
+    for (uint32_t j0 = 0; j0 < c_h; j0 += FV_NB_ROUND) {
+      const uint32_t mr = min(c_h - j0, (uint32_t)FV_NB_ROUND);
+      for (uint32_t jb = tid; jb < mr; jb += 4 * T) {  // up to 4 independent loads per thread
+        uint32_t r[4];
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) r[q] = order[j0 + min(jb + q * T, mr - 1)];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = a.sc[r[q]];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (jb + q * T < mr) scbuf[jb + q * T] = v[q];
+      }
+      __syncthreads();
+      if (tid < 64)
+        for (uint32_t j = tid; j < mr; j += 64) part = __fadd_rn(part, scbuf[j]);  // FV_NB_ROUND % 64 == 0
+      __syncthreads();
+    }
   }
   float xx = 0.0f;
   if (tid < 64) scbuf[tid] = part;
@@ -810,6 +902,7 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   (void)hipFree(t->group_count);
   (void)hipFree(t->bmax);
   (void)hipFree(t->win);
+  (void)hipFree(t->win16);
   (void)hipFree(t->sc);
   (void)hipFree(t->xx);
   (void)hipFree(t->scalars);
@@ -834,6 +927,8 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMalloc((void **)&t->xx, (size_t)t->ldk * sizeof(float)));
   FV_HIP(hipMalloc((void **)&t->bmax, ((size_t)t->dense_blocks + (size_t)FV_NB_CLASSES * t->K) * sizeof(float)));
   FV_HIP(hipMemsetAsync(t->win, 0, ((size_t)t->B + 16) * sizeof(int32_t), t->stream));
+  FV_HIP(hipMalloc((void **)&t->win16, ((size_t)t->B + 64) * sizeof(uint16_t)));  // read in 16-byte pieces
+  FV_HIP(hipMemsetAsync(t->win16, 0, ((size_t)t->B + 64) * sizeof(uint16_t), t->stream));
   FV_HIP(hipMalloc((void **)&t->scalars, 16 * sizeof(float)));
   FV_HIP(hipMemsetAsync(t->Wt, 0, elems * sizeof(float), t->stream));
   FV_HIP(hipMemsetAsync(t->xx, 0, (size_t)t->ldk * sizeof(float), t->stream));
@@ -1061,6 +1156,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.invf = t->invf;
   g.idx = t->idx;
   g.win = t->win;
+  g.win16 = t->win16;
   g.sc = t->sc;
   g.first = first;
   g.n = n;
@@ -1082,7 +1178,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   }
   if (ev) FV_HIP(hipEventRecord(ev[1], t->stream));
   fv_group_args gr;
-  gr.win = t->win;
+  gr.win = t->win16;
   gr.sc = t->sc;
   gr.order = t->order;
   gr.group_base = t->group_base;
@@ -1091,7 +1187,12 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   gr.n = n;
   // a thread's run of the winner array should fit its 64-bit match mask
   const unsigned gr_threads = n <= 16384 ? 256 : FV_NB_MAX_THREADS;
-  if (which & 2u) hipLaunchKernelGGL(fv_group_kernel, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
+  if (which & 2u) {
+    if (n <= 64 * gr_threads && n < 65536)
+      hipLaunchKernelGGL(fv_group_kernel<true>, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
+    else
+      hipLaunchKernelGGL(fv_group_kernel<false>, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
+  }
   if (ev) FV_HIP(hipEventRecord(ev[2], t->stream));
   fv_sparse_args sp;
   sp.order = t->order;
