@@ -97,21 +97,45 @@ struct fv_gather_args {
   uint32_t n, K, ldk, w, V, tie_rule;
 };
 
+// FV_GATHER_WINDOWS windows per wavefront, one after the other: the grid then fits the machine in
+// one round (a second round of waves cost more than the longer life of each wave). The tokens of
+// all the wave's windows are fetched up front.
+#ifndef FV_GATHER_WINDOWS
+#define FV_GATHER_WINDOWS 1
+#endif
+
+template <int NV>
+__device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, uint32_t r, int32_t idx, int lane);
+
 template <int NV>
 __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a) {
   const int lane = threadIdx.x & 63;
-  const uint32_t r = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (r >= a.n) return;
+  const uint32_t g = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t per = (a.n + FV_GATHER_WINDOWS - 1) / FV_GATHER_WINDOWS;  // wave g takes windows g, g + per, ...
+  if (g >= per) return;
 
   // sampler: lane c holds column index c of the window (flyvec/src/cuda_funcs.cu:915-936)
-  int32_t idx = -1;
-  if (lane < (int)a.w) {
-    const uint64_t s = a.pstart[a.first + r];
-    const int32_t tok = a.corpus[s + lane];
-    idx = tok < 0 ? -1 : (lane == (int)(a.w / 2) ? tok + (int32_t)a.V : tok);
-    a.idx[(uint64_t)r * a.w + lane] = idx;
+  int32_t idx[FV_GATHER_WINDOWS];
+#pragma unroll
+  for (int k = 0; k < FV_GATHER_WINDOWS; ++k) {
+    const uint32_t r = g + k * per;
+    idx[k] = -1;
+    if (lane < (int)a.w && r < a.n) {
+      const uint64_t s = a.pstart[a.first + r];
+      const int32_t tok = a.corpus[s + lane];
+      idx[k] = tok < 0 ? -1 : (lane == (int)(a.w / 2) ? tok + (int32_t)a.V : tok);
+      a.idx[(uint64_t)r * a.w + lane] = idx[k];
+    }
   }
+#pragma unroll
+  for (int k = 0; k < FV_GATHER_WINDOWS; ++k) {
+    const uint32_t r = g + k * per;
+    if (r < a.n) fv_gather_one_window<NV>(a, r, idx[k], lane);
+  }
+}
 
+template <int NV>
+__device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, uint32_t r, int32_t idx, int lane) {
   double acc[NV];
 #pragma unroll
   for (int j = 0; j < NV; ++j) acc[j] = 0.0;
@@ -1142,7 +1166,8 @@ extern "C" int fv_trainer_get_permutation(fv_trainer *t, uint64_t *out_perm, uin
 
 template <int NV>
 static void fv_launch_gather(const fv_gather_args &a, hipStream_t stream) {
-  hipLaunchKernelGGL(fv_gather_winner_kernel<NV>, dim3((a.n + 3) / 4), dim3(256), 0, stream, a);
+  const uint32_t waves = (a.n + FV_GATHER_WINDOWS - 1) / FV_GATHER_WINDOWS;
+  hipLaunchKernelGGL(fv_gather_winner_kernel<NV>, dim3((waves + 3) / 4), dim3(256), 0, stream, a);
 }
 
 // Enqueues the kernels of one step (those whose bit is set in `which`); ev (nullable) receives
