@@ -59,7 +59,7 @@ def test_small_config_bit_exact(gpu, oracle_lib, tie):
     assert np.array_equal(Wg, Wo)
 
 
-@pytest.mark.parametrize("K,w,V,B", [(5, 3, 40, 64), (63, 1, 100, 128), (64, 5, 100, 100), (65, 15, 200, 256),
+@pytest.mark.parametrize("K,w,V,B", [(1, 1, 5, 1), (3, 2, 7, 3), (5, 3, 40, 64), (63, 1, 100, 128), (64, 5, 100, 100), (65, 15, 200, 256),
                                      (130, 64, 300, 64), (1000, 15, 300, 512), (2048, 7, 64, 128),
                                      (30, 11, 20000, 700), (30, 11, 30000, 700), (3, 5, 400000, 300)])
 def test_shapes_bit_exact(gpu, oracle_lib, K, w, V, B):
