@@ -13,7 +13,7 @@
  *   fvo_count_windows / fvo_window_starts : the reference's own prune_input.cpp
  *       compiled into oracle/_ref (bit-exact on random and edge-case offsets).
  *   fvo_inverse_frequency, fvo_inflate, fvo_activations, fvo_argmax_*,
- *   fvo_train_step : closed forms (one-window batch, W = 0 fixed point,
+ *   fvo_train_step, fvo_train_step_delta (the anti-Hebbian term), fvo_epoch_delta : closed forms (one-window batch, W = 0 fixed point,
  *       invariance to a global rescale of 1/frequency by a power of two,
  *       max|dW| == eps), a from-scratch brute force in Python floats on tiny
  *       shapes, and numpy restatements of each stage.
@@ -219,11 +219,14 @@ void fvo_xx_sums(const int32_t *win, const float *sc, uint64_t n, int K, int ord
  * Outputs (any may be NULL): winners[n], sc_at_winner[n], xx[K], *nc_out.
  * ds_scratch must hold K*N floats.
  */
-void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx, uint64_t n, int w,
-                    const float *invf, float eps, float prec, int tie_rule, float *ds_scratch,
-                    int32_t *winners, float *sc_at_winner, float *xx_out, float *nc_out) {
+void fvo_train_step_delta(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx, uint64_t n, int w,
+                          const float *invf, float eps, float prec, int tie_rule, float delta, float *ds_scratch,
+                          int32_t *winners, float *sc_at_winner, int32_t *seconds, float *sc_at_second,
+                          float *xx_out, float *nc_out) {
   int32_t *win = (int32_t *)malloc(sizeof(int32_t) * (n ? n : 1));
   float *scw = (float *)malloc(sizeof(float) * (n ? n : 1));
+  int32_t *win2 = (int32_t *)malloc(sizeof(int32_t) * (n ? n : 1));
+  float *scw2 = (float *)malloc(sizeof(float) * (n ? n : 1));
   float *xx = (float *)calloc((size_t)(K > 0 ? K : 1), sizeof(float));
   float *ds = ds_scratch;
 
@@ -250,11 +253,40 @@ void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx,
         }
       win[r] = best;
       scw[r] = (float)ss;
+      win2[r] = best;
+      scw2[r] = 0.0f;
+      if (delta != 0) {
+        /* flyvec/src/cuda_funcs.cu:495-548 with num_m = 2: the winner's entry is overwritten with
+         * -9999.9999 and the same search runs again on the row */
+        raw[best] = (float)-9999.9999;
+        int second = tie_rule ? fvo_argmax_reference(raw, K) : fvo_argmax_lowest(raw, K);
+        const float *row2 = W + (uint64_t)second * N;
+        double s2 = 0.0;
+        for (int c = 0; c < w; ++c)
+          if (ix[c] != -1) {
+            float prod = row2[ix[c]] * invf[(uint64_t)ix[c] % V];
+            s2 += (double)prod;
+          }
+        win2[r] = second;
+        scw2[r] = (float)s2;
+      }
     }
     free(raw);
   }
 
   fvo_xx_sums(win, scw, n, K, 0, xx);
+  if (delta != 0) {
+    /* flyvec/src/cuda_funcs.cu:726-734: xx[second] += -delta * scaled[second]. Fixed order: the
+     * anti-Hebbian contributions of a neuron are summed like the Hebbian ones (fvo_xx_sums), and the
+     * two totals are then added. */
+    float *neg = (float *)malloc(sizeof(float) * (n ? n : 1));
+    float *xx2 = (float *)calloc((size_t)(K > 0 ? K : 1), sizeof(float));
+    for (uint64_t r = 0; r < n; ++r) neg[r] = -delta * scw2[r];
+    fvo_xx_sums(win2, neg, n, K, 0, xx2);
+    for (int h = 0; h < K; ++h) xx[h] = xx[h] + xx2[h];
+    free(neg);
+    free(xx2);
+  }
 
   /* ds = -xx*W or 0 */
 #pragma omp parallel for schedule(static)
@@ -275,6 +307,19 @@ void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx,
     const int32_t *ix = idx + r * (uint64_t)w;
     for (int c = 0; c < w; ++c)
       if (ix[c] != -1) d[ix[c]] = d[ix[c]] + invf[(uint64_t)ix[c] % V];
+  }
+  if (delta != 0) {
+    /* flyvec/src/cuda_funcs.cu:668: ds[second][idx] += -delta * 1/f. Fixed order: after every
+     * Hebbian addition, in increasing (window, position) order. */
+    for (uint64_t r = 0; r < n; ++r) {
+      float *d = ds + (uint64_t)win2[r] * N;
+      const int32_t *ix = idx + r * (uint64_t)w;
+      for (int c = 0; c < w; ++c)
+        if (ix[c] != -1) {
+          float g = -delta * invf[(uint64_t)ix[c] % V];
+          d[ix[c]] = d[ix[c]] + g;
+        }
+    }
   }
 
   /* rows with xx == 0 are zero-filled (drops their sparse term); nc = max|ds| */
@@ -309,11 +354,28 @@ void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx,
 
   if (winners) memcpy(winners, win, sizeof(int32_t) * n);
   if (sc_at_winner) memcpy(sc_at_winner, scw, sizeof(float) * n);
+  if (seconds) memcpy(seconds, win2, sizeof(int32_t) * n);
+  if (sc_at_second) memcpy(sc_at_second, scw2, sizeof(float) * n);
   if (xx_out) memcpy(xx_out, xx, sizeof(float) * (size_t)K);
   if (nc_out) *nc_out = nc;
   free(win);
   free(scw);
+  free(win2);
+  free(scw2);
   free(xx);
+}
+
+/* The step without the anti-Hebbian term (delta = 0, the trainer's default). */
+void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx, uint64_t n, int w,
+                    const float *invf, float eps, float prec, int tie_rule, float *ds_scratch,
+                    int32_t *winners, float *sc_at_winner, float *xx_out, float *nc_out) {
+  fvo_train_step_delta(W, K, N, V, idx, n, w, invf, eps, prec, tie_rule, 0.0f, ds_scratch, winners, sc_at_winner,
+                       NULL, NULL, xx_out, nc_out);
+}
+
+/* flyvec/src/cuda_funcs.cu:1230: the anti-Hebbian strength of an epoch */
+float fvo_epoch_delta(float delta, uint64_t epoch, uint64_t n_epochs) {
+  return (float)(delta * 0.5 * (1.0 + tanh((((float)epoch) - (0.125 * n_epochs)) / 10.0)));
 }
 
 /*
@@ -324,10 +386,10 @@ void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx,
  * remainder only).  winners (if given) receives the winners of every step
  * back to back.  Returns the number of windows processed.
  */
-uint64_t fvo_train_steps(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
-                         const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
-                         uint64_t n_steps, int w, const float *invf, float eps, float prec,
-                         int tie_rule, int32_t *winners) {
+uint64_t fvo_train_steps_delta(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
+                               const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
+                               uint64_t n_steps, int w, const float *invf, float eps, float prec,
+                               int tie_rule, float delta, int32_t *winners) {
   const uint64_t N = 2 * V;
   float *ds = (float *)malloc(sizeof(float) * (size_t)K * N);
   int32_t *idx = (int32_t *)malloc(sizeof(int32_t) * B * (uint64_t)w);
@@ -337,11 +399,19 @@ uint64_t fvo_train_steps(float *W, int K, uint64_t V, const int32_t *corpus, con
     if (k0 >= n_windows) break;
     uint64_t n = (k0 + B <= n_windows) ? B : n_windows - k0;
     fvo_inflate(corpus, starts, perm, k0, n, w, V, idx);
-    fvo_train_step(W, K, N, V, idx, n, w, invf, eps, prec, tie_rule, ds,
-                   winners ? winners + done : NULL, NULL, NULL, NULL);
+    fvo_train_step_delta(W, K, N, V, idx, n, w, invf, eps, prec, tie_rule, delta, ds,
+                         winners ? winners + done : NULL, NULL, NULL, NULL, NULL, NULL);
     done += n;
   }
   free(ds);
   free(idx);
   return done;
+}
+
+uint64_t fvo_train_steps(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
+                         const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
+                         uint64_t n_steps, int w, const float *invf, float eps, float prec,
+                         int tie_rule, int32_t *winners) {
+  return fvo_train_steps_delta(W, K, V, corpus, starts, perm, n_windows, first, B, n_steps, w, invf, eps, prec,
+                               tie_rule, 0.0f, winners);
 }

@@ -61,6 +61,17 @@ def lib():
         L.fvo_train_step.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, C.c_void_p, C.c_uint64,
                                      C.c_int, C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_void_p,
                                      C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.fvo_epoch_delta.restype = C.c_float
+        L.fvo_epoch_delta.argtypes = [C.c_float, C.c_uint64, C.c_uint64]
+        L.fvo_train_step_delta.restype = None
+        L.fvo_train_step_delta.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, C.c_void_p, C.c_uint64,
+                                           C.c_int, C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_float,
+                                           C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                           C.c_void_p, C.c_void_p]
+        L.fvo_train_steps_delta.restype = C.c_uint64
+        L.fvo_train_steps_delta.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                            C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_void_p,
+                                            C.c_float, C.c_float, C.c_int, C.c_float, C.c_void_p]
         L.fvo_train_steps.restype = C.c_uint64
         L.fvo_train_steps.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p,
                                       C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_void_p,
@@ -180,8 +191,13 @@ def epoch_eps(lr0, epoch, n_epochs):
     return float(lib().fvo_epoch_eps(lr0, epoch, n_epochs))
 
 
-def train_step(W, idx, invf, eps, prec=1e-30, tie_rule=0):
-    """In-place step on W (K, 2V) fp32 C-order.  Returns dict(winners, sc, xx, nc)."""
+def epoch_delta(delta, epoch, n_epochs):
+    return float(lib().fvo_epoch_delta(delta, epoch, n_epochs))
+
+
+def train_step(W, idx, invf, eps, prec=1e-30, tie_rule=0, delta=0.0):
+    """In-place step on W (K, 2V) fp32 C-order.  Returns dict(winners, sc, seconds, sc2, xx, nc, ds);
+    delta is the anti-Hebbian strength of the step (0 = none)."""
     assert W.dtype == np.float32 and W.flags.c_contiguous
     idx = np.ascontiguousarray(idx, dtype=np.int32)
     invf = np.ascontiguousarray(invf, dtype=np.float32)
@@ -192,12 +208,14 @@ def train_step(W, idx, invf, eps, prec=1e-30, tie_rule=0):
     sc = np.empty(n, dtype=np.float32)
     xx = np.empty(K, dtype=np.float32)
     nc = np.zeros(1, dtype=np.float32)
-    lib().fvo_train_step(_p(W), K, N, len(invf), _p(idx), n, w, _p(invf), eps, prec, tie_rule,
-                         _p(ds), _p(win), _p(sc), _p(xx), _p(nc))
-    return dict(winners=win, sc=sc, xx=xx, nc=float(nc[0]), ds=ds)
+    win2 = np.empty(n, dtype=np.int32)
+    sc2 = np.empty(n, dtype=np.float32)
+    lib().fvo_train_step_delta(_p(W), K, N, len(invf), _p(idx), n, w, _p(invf), eps, prec, tie_rule, delta,
+                               _p(ds), _p(win), _p(sc), _p(win2), _p(sc2), _p(xx), _p(nc))
+    return dict(winners=win, sc=sc, seconds=win2, sc2=sc2, xx=xx, nc=float(nc[0]), ds=ds)
 
 
-def train_steps(W, corpus, starts, perm, first, B, n_steps, w, invf, eps, prec=1e-30, tie_rule=0):
+def train_steps(W, corpus, starts, perm, first, B, n_steps, w, invf, eps, prec=1e-30, tie_rule=0, delta=0.0):
     """In-place n_steps minibatches; returns the winners of all processed windows."""
     assert W.dtype == np.float32 and W.flags.c_contiguous
     corpus = np.ascontiguousarray(corpus, dtype=np.int32)
@@ -209,6 +227,6 @@ def train_steps(W, corpus, starts, perm, first, B, n_steps, w, invf, eps, prec=1
     nwin = len(perm)
     cap = max(0, min(n_steps * B, nwin - first))
     win = np.empty(cap, dtype=np.int32)
-    done = lib().fvo_train_steps(_p(W), K, V, _p(corpus), _p(starts), _p(perm), nwin, first, B, n_steps,
-                                 w, _p(invf), eps, prec, tie_rule, _p(win))
+    done = lib().fvo_train_steps_delta(_p(W), K, V, _p(corpus), _p(starts), _p(perm), nwin, first, B, n_steps,
+                                       w, _p(invf), eps, prec, tie_rule, delta, _p(win))
     return win[:done]

@@ -27,13 +27,26 @@ def brute_argmax_lowest(raw):
     return best
 
 
-def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest):
-    """flyvec/src/cuda_funcs.cu:1662-1803 (sparse, frequency scaling, delta = 0) in Python scalars."""
+def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest, delta=0.0):
+    """flyvec/src/cuda_funcs.cu:1662-1803 (sparse, frequency scaling) in Python scalars. With
+    delta != 0 the second neuron of every window (the search repeated with the winner's activation
+    overwritten by -9999.9999, :495-548) receives the anti-Hebbian terms (:668, :726-734); their
+    place in the order of additions: after the Hebbian ones."""
     W = W.copy()
     K, N = W.shape
     V = N // 2
     n, w = idx.shape
-    win, sc = [], []
+    delta = f32(delta)
+
+    def scaled(h, r):
+        ss = 0.0
+        for c in range(w):
+            i = idx[r, c]
+            if i != -1:
+                ss += float(f32(W[h, i] * invf[i % V]))  # fp32 product, double sum
+        return f32(ss)
+
+    win, sc, win2, sc2 = [], [], [], []
     for r in range(n):
         raw = []
         for h in range(K):
@@ -44,16 +57,21 @@ def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest):
                     s += float(W[h, i])
             raw.append(f32(s))
         b = argmax(raw)
-        ss = 0.0
-        for c in range(w):
-            i = idx[r, c]
-            if i != -1:
-                ss += float(f32(W[b, i] * invf[i % V]))  # fp32 product, double sum
         win.append(b)
-        sc.append(f32(ss))
+        sc.append(scaled(b, r))
+        if delta != 0:
+            raw[b] = f32(-9999.9999)
+            b2 = argmax(raw)
+            win2.append(b2)
+            sc2.append(scaled(b2, r))
     xx = [f32(0)] * K
     for r in range(n):
         xx[win[r]] = f32(xx[win[r]] + sc[r])
+    if delta != 0:
+        xx2 = [f32(0)] * K
+        for r in range(n):
+            xx2[win2[r]] = f32(xx2[win2[r]] + f32(-delta * sc2[r]))
+        xx = [f32(a + b) for a, b in zip(xx, xx2)]
     ds = np.zeros((K, N), dtype=f32)
     for h in range(K):
         if xx[h] != 0:
@@ -64,6 +82,12 @@ def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest):
             i = idx[r, c]
             if i != -1:
                 ds[win[r], i] = f32(ds[win[r], i] + invf[i % V])
+    if delta != 0:
+        for r in range(n):
+            for c in range(w):
+                i = idx[r, c]
+                if i != -1:
+                    ds[win2[r], i] = f32(ds[win2[r], i] + f32(-delta * invf[i % V]))
     nc = f32(0)
     for h in range(K):
         if xx[h] != 0:
@@ -77,6 +101,8 @@ def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest):
                 v = f32(s * ds[h, c])
                 if abs(float(v)) > 1.0e-10:
                     W[h, c] = f32(W[h, c] + v)
+    if delta != 0:
+        return W, np.array(win, dtype=np.int32), np.array(xx, dtype=f32), float(nc), np.array(win2, dtype=np.int32)
     return W, np.array(win, dtype=np.int32), np.array(xx, dtype=f32), float(nc)
 
 
@@ -356,3 +382,69 @@ def test_step_uses_the_interleaved_order():
     res = to.train_step(W.copy(), idx, invf, 1e-3)
     assert np.bincount(res["winners"], minlength=K).max() > 64
     assert np.array_equal(res["xx"], xx_numpy(res["winners"], res["sc"], K))
+
+
+# ---- anti-Hebbian term (delta != 0) -----------------------------------------------------------------
+
+@pytest.mark.parametrize("seed", range(8))
+def test_delta_step_against_brute_force(seed):
+    rng = np.random.default_rng(100 + seed)
+    K, V, w, n = int(rng.integers(1, 5)), int(rng.integers(3, 7)), 3, int(rng.integers(1, 9))
+    W = rng.standard_normal((K, 2 * V)).astype(f32)
+    idx = rng.integers(0, V, size=(n, w)).astype(np.int32)
+    idx[:, w // 2] += V
+    idx[rng.random((n, w)) < 0.15] = -1
+    invf = (1.0 / rng.integers(1, 50, size=V)).astype(f32)
+    eps, prec, delta = 2e-2, 1e-30, 0.4
+    want_W, want_win, want_xx, want_nc, want_win2 = brute_step(W, idx, invf, eps, prec, delta=delta)
+    got_W = W.copy()
+    res = to.train_step(got_W, idx, invf, eps, prec, tie_rule=0, delta=delta)
+    assert np.array_equal(res["winners"], want_win) and np.array_equal(res["seconds"], want_win2)
+    assert np.array_equal(res["xx"], want_xx)
+    assert res["nc"] == want_nc
+    assert np.array_equal(got_W, want_W)
+
+
+def test_delta_single_window_closed_form():
+    W, idx, invf = setup_small(0, n=1)
+    V = W.shape[1] // 2
+    W0 = W.copy()
+    delta = f32(0.25)
+    res = to.train_step(W, idx, invf, 1e-3, delta=float(delta))
+    mu, nu = int(res["winners"][0]), int(res["seconds"][0])
+    raw = W0[:, idx[0]].astype(np.float64).sum(axis=1).astype(f32)
+    assert mu == int(np.argmax(raw)) and mu != nu
+    assert nu == int(np.argsort(-raw, kind="stable")[1])          # the runner-up of the window
+    sc = lambda h: f32((W0[h, idx[0]] * invf[idx[0] % V]).astype(f32).astype(np.float64).sum())
+    assert res["xx"][mu] == sc(mu) and res["xx"][nu] == f32(-delta * sc(nu)) and np.count_nonzero(res["xx"]) == 2
+    ds_nu = f32(-res["xx"][nu]) * W0[nu]
+    for i in idx[0]:
+        ds_nu[i] = f32(ds_nu[i] + f32(-delta * invf[i % V]))
+    assert np.array_equal(res["ds"][nu], ds_nu)
+    changed = np.flatnonzero((W != W0).any(axis=1))
+    assert sorted(changed.tolist()) == sorted([mu, nu])
+
+
+def test_delta_zero_is_the_plain_step_and_one_neuron_meets_itself():
+    W, idx, invf = setup_small(5)
+    Wa, Wb = W.copy(), W.copy()
+    ra = to.train_step(Wa, idx, invf, 1e-3)
+    rb = to.train_step(Wb, idx, invf, 1e-3, delta=0.0)
+    assert np.array_equal(Wa, Wb) and np.array_equal(ra["winners"], rb["winners"])
+    # with a single neuron the second search finds the same neuron again: it receives both terms
+    rng = np.random.default_rng(2)
+    W1 = rng.standard_normal((1, 12)).astype(f32)
+    idx1 = np.array([[1, 8, 3]], dtype=np.int32)
+    invf1 = np.full(6, 0.5, dtype=f32)
+    want = brute_step(W1, idx1, invf1, 1e-2, 1e-30, delta=0.3)
+    got = W1.copy()
+    res = to.train_step(got, idx1, invf1, 1e-2, delta=0.3)
+    assert res["seconds"][0] == 0 and np.array_equal(got, want[0])
+
+
+def test_epoch_delta_schedule():
+    # flyvec/src/cuda_funcs.cu:1230: delta * 0.5 * (1 + tanh((ep - 0.125 Nep) / 10)), rounded to fp32 once
+    import math
+    for delta, ep, nep in [(0.4, 0, 15), (0.4, 7, 15), (0.4, 14, 15), (1.0, 100, 200), (0.0, 3, 15)]:
+        want = f32(float(f32(delta)) * 0.5 * (1.0 + math.tanh((float(f32(ep)) - 0.125 * nep) / 10.0)))
+        assert to.epoch_delta(delta, ep, nep) == want
