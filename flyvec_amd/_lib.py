@@ -70,6 +70,9 @@ SIGNATURES = {
     "fv_trainer_set_permutation": [_vp, _vp, _u64],
     "fv_trainer_get_permutation": [_vp, _vp, _u64],
     "fv_trainer_step": [_vp, _u64, _u32, _f32],
+    "fv_trainer_step_delta": [_vp, _u64, _u32, _f32, _f32],
+    "fv_trainer_epoch_delta": [_vp, _u64, _u64, _vp],
+    "fv_trainer_get_second_winners": [_vp, _vp, _u32],
     "fv_trainer_run_epoch": [_vp, _u64, _u64],
     "fv_trainer_epoch_eps": [_vp, _u64, _u64, C.POINTER(_f32)],
     "fv_trainer_sync": [_vp],

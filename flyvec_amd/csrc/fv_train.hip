@@ -64,6 +64,15 @@ struct fv_trainer {
   int32_t *idx;     // B x w column indices of the current minibatch
   int32_t *win;     // B winners
   uint16_t *win16;  // the same, 16 bits each (padded by 64)
+  // anti-Hebbian form (delta != 0), allocated with the first such step: the second neuron of every
+  // window, its scaled activation, the windows grouped by it, the second count of every slot record
+  int32_t *win2;
+  uint16_t *win2_16;
+  float *sc2;
+  uint32_t *order2, *group_base2, *group_count2;
+  uint32_t *slot_n2;
+  fv_slot *slots2;  // records of a step with delta != 0: twice the room
+  float last_delta;
   float *sc;        // B scaled activations at the winner
   uint32_t *order;  // B window ids grouped by winner, ascending inside a group
   uint32_t *group_base, *group_count;  // K each
@@ -93,6 +102,10 @@ struct fv_gather_args {
   int32_t *win;
   uint16_t *win16;  // the same winners as 16-bit values, for the grouping kernel
   float *sc;
+  // anti-Hebbian form only: the second neuron of every window and its scaled activation
+  int32_t *win2;
+  uint16_t *win2_16;
+  float *sc2;
   uint64_t first;
   uint32_t n, K, ldk, w, V, tie_rule;
 };
@@ -104,10 +117,12 @@ struct fv_gather_args {
 #define FV_GATHER_WINDOWS 1
 #endif
 
-template <int NV>
+template <int NV, bool DELTA>
 __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, uint32_t r, int32_t idx, int lane);
 
-template <int NV>
+// DELTA: also the window's second neuron (flyvec/src/cuda_funcs.cu:495-548 with num_m = 2), which
+// receives the anti-Hebbian terms.
+template <int NV, bool DELTA>
 __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a) {
   const int lane = threadIdx.x & 63;
   const uint32_t g = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -130,46 +145,44 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
 #pragma unroll
   for (int k = 0; k < FV_GATHER_WINDOWS; ++k) {
     const uint32_t r = g + k * per;
-    if (r < a.n) fv_gather_one_window<NV>(a, r, idx[k], lane);
+    if (r < a.n) fv_gather_one_window<NV, DELTA>(a, r, idx[k], lane);
   }
 }
 
+// Argmax over the wave's K values (neuron h = lane + 64 j in acc[j]); the entry of neuron `replaced`
+// (none if >= K) counts as -9999.9999. Ties: the smaller tie key wins. Key = neuron index (lowest
+// index wins), or the position of the neuron in the reference's reduction order: its 64 threads
+// each scan a stride-64 class (= this lane's values, ascending), warp 0 beats warp 1, and inside a
+// warp the shuffle-down tree prefers lanes in bit-reversed order.
 template <int NV>
-__device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, uint32_t r, int32_t idx, int lane) {
-  double acc[NV];
-#pragma unroll
-  for (int j = 0; j < NV; ++j) acc[j] = 0.0;
-  fv_gather_accumulate<NV, fv_rows_per_batch<NV>::value, double>(a.Wt, a.ldk, a.K, 2 * a.V, lane,
-                                                                 (int)a.w, idx, acc);
-
-  // argmax of the raw activation. Ties: the smaller tie key wins. Key = neuron index (lowest
-  // index wins), or the position of the neuron in the reference's reduction order: its 64
-  // threads each scan a stride-64 class (= this lane's values, ascending), warp 0 beats warp 1,
-  // and inside a warp the shuffle-down tree prefers lanes in bit-reversed order.
+__device__ __forceinline__ uint32_t fv_wave_argmax(const double (&acc)[NV], uint32_t K, uint32_t tie_rule, int lane,
+                                                   uint32_t replaced) {
   const uint32_t lane_rank = ((uint32_t)lane & 32u) | (__brev((uint32_t)lane & 31u) >> 27);
   uint64_t best = 0;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const uint32_t h = lane + 64 * j;
-    const bool valid = (j < NV - 1) || h < a.K;
-    const uint32_t key = a.tie_rule ? ((lane_rank << 16) | (uint32_t)j) : h;
-    const uint64_t pk = ((uint64_t)fv_ord_key((float)acc[j]) << 32) | (0xffffffffu - key);
+    const bool valid = (j < NV - 1) || h < K;
+    const uint32_t key = tie_rule ? ((lane_rank << 16) | (uint32_t)j) : h;
+    const float v = h == replaced ? (float)-9999.9999 : (float)acc[j];
+    const uint64_t pk = ((uint64_t)fv_ord_key(v) << 32) | (0xffffffffu - key);
     best = (valid && pk > best) ? pk : best;
   }
   best = fv_wave_max_u64(best);
   const uint32_t bkey = 0xffffffffu - (uint32_t)best;
-  uint32_t hstar;
-  if (a.tie_rule) {
+  if (tie_rule) {
     const uint32_t rank = bkey >> 16;
-    hstar = (bkey & 0xffffu) * 64 + ((rank & 32u) | (__brev(rank & 31u) >> 27));
-  } else {
-    hstar = bkey;
+    return (bkey & 0xffffu) * 64 + ((rank & 32u) | (__brev(rank & 31u) >> 27));
   }
+  return bkey;
+}
 
-  // frequency-scaled activation of the winner: fp32 products, double sum in window order
+// Frequency-scaled activation of neuron h for the window whose column index c sits in lane c:
+// fp32 products, double sum in window order, one rounding (flyvec/src/cuda_funcs.cu:289-305).
+__device__ __forceinline__ float fv_scaled_activation(const fv_gather_args &a, int32_t idx, uint32_t h) {
   double pd = 0.0;
   if ((uint32_t)idx < 2 * a.V) {
-    const float wv = a.Wt[(uint64_t)idx * a.ldk + hstar];
+    const float wv = a.Wt[(uint64_t)idx * a.ldk + h];
     const float f = a.invf[(uint32_t)idx >= a.V ? (uint32_t)idx - a.V : (uint32_t)idx];
     pd = (double)__fmul_rn(wv, f);
   }
@@ -180,10 +193,32 @@ __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, ui
                          fv_readlane((uint32_t)bits, c);
     s = s + __longlong_as_double((long long)got);
   }
+  return (float)s;
+}
+
+template <int NV, bool DELTA>
+__device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, uint32_t r, int32_t idx, int lane) {
+  double acc[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) acc[j] = 0.0;
+  fv_gather_accumulate<NV, fv_rows_per_batch<NV>::value, double>(a.Wt, a.ldk, a.K, 2 * a.V, lane,
+                                                                 (int)a.w, idx, acc);
+  const uint32_t hstar = fv_wave_argmax<NV>(acc, a.K, a.tie_rule, lane, 0xffffffffu);
+  // the scaled activation is only ever read at the chosen neurons (flyvec/src/cuda_funcs.cu:731)
+  const float s = fv_scaled_activation(a, idx, hstar);
   if (lane == 0) {
     a.win[r] = (int32_t)hstar;
     a.win16[r] = (uint16_t)hstar;
-    a.sc[r] = (float)s;
+    a.sc[r] = s;
+  }
+  if (DELTA) {
+    const uint32_t second = fv_wave_argmax<NV>(acc, a.K, a.tie_rule, lane, hstar);
+    const float s2 = fv_scaled_activation(a, idx, second);
+    if (lane == 0) {
+      a.win2[r] = (int32_t)second;
+      a.win2_16[r] = (uint16_t)second;
+      a.sc2[r] = s2;
+    }
   }
 }
 
@@ -220,6 +255,8 @@ struct fv_group_args {
   uint32_t *group_count;
   float *xx;
   uint32_t n;
+  float scale;          // every scaled activation is multiplied by this first (1, or -delta for the second neurons)
+  uint32_t accumulate;  // add the total to xx[h] instead of storing it
 };
 
 // ds of one sparse element: the dense term, then n sequential additions of 1/f.
@@ -230,6 +267,12 @@ __device__ __forceinline__ float fv_sparse_ds(float xx, float wv, float f, uint3
 __device__ __forceinline__ float fv_absmax_keep(float m, float v) {
   const float a = fabsf(v);
   return a > m ? a : m;  // a NaN never replaces m, as in the reference's comparison
+}
+
+// ds of one sparse element with the anti-Hebbian term: after the n additions of 1/f, n2 additions
+// of -delta * 1/f (flyvec/src/cuda_funcs.cu:667-668; this order of the additions is the checker's).
+__device__ __forceinline__ float fv_sparse_ds2(float xx, float wv, float f, uint32_t n, float delta, uint32_t n2) {
+  return fv_add_repeat(fv_sparse_ds(xx, wv, f, n), __fmul_rn(-delta, f), n2);
 }
 
 // Block-wide maximum of non-negative floats (blocks of up to 16 waves; smem holds one float per wave).
@@ -346,7 +389,7 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
 #pragma unroll
     for (int q = 0; q < PF; ++q) {
       const uint32_t r = mm ? r0 + (uint32_t)__ffsll((long long)mm) - 1 : r0;
-      pf[q] = a.sc[min(r, n - 1)];
+      pf[q] = __fmul_rn(a.scale, a.sc[min(r, n - 1)]);
       mm &= mm - 1;
     }
     uint32_t total;
@@ -398,7 +441,7 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
     while (mm) {
       const uint32_t r = r0 + (uint32_t)__ffsll((long long)mm) - 1;
       order[rank] = r;
-      if (staged) scbuf[rank] = a.sc[r];
+      if (staged) scbuf[rank] = __fmul_rn(a.scale, a.sc[r]);
       ++rank;
       mm &= mm - 1;
     }
@@ -424,7 +467,7 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
 #pragma unroll
         for (int q = 0; q < 4; ++q) r[q] = order[j0 + min(jb + q * T, mr - 1)];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] = a.sc[r[q]];
+        for (int q = 0; q < 4; ++q) v[q] = __fmul_rn(a.scale, a.sc[r[q]]);
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           if (jb + q * T < mr) scbuf[jb + q * T] = v[q];
@@ -442,7 +485,7 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
     const uint32_t np = min(c_h, 64u);
     for (uint32_t l = 0; l < np; ++l) xx = __fadd_rn(xx, scbuf[l]);
   }
-  if (tid == 0) a.xx[h] = xx;
+  if (tid == 0) a.xx[h] = a.accumulate ? __fadd_rn(a.xx[h], xx) : xx;
 }
 
 // ---- kernel 3: sparse elements -----------------------------------------------------------------------
@@ -466,6 +509,13 @@ struct fv_sparse_args {
   float *bmax_sparse;    // one maximum of |ds| per block
   uint32_t *slot_count;  // records written per block
   uint32_t ldk, w, V, pad_row;  // pad_row: the row index just behind the index matrix
+  // anti-Hebbian form only: the windows in which the neuron came second, grouped like the others;
+  // the count of those occurrences of an element goes to slot_n2 beside its record
+  const uint32_t *order2;
+  const uint32_t *group_base2;
+  const uint32_t *group_count2;
+  uint32_t *slot_n2;
+  float delta;
 };
 
 // Barrier for data exchanged through LDS only: waits for the wave's LDS operations, not for its
@@ -527,8 +577,12 @@ __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, uint32_t *ord
     fv_sparse_count<NARROW, FV_SP_LOADS>(cnt, ord, n_staged, idx, w, q, lo, span, tid);
 }
 
+// DELTA: the neuron's elements are counted over two lists of windows, those it won and those in
+// which it came second, into two counter arrays; a record carries both counts.
+template <bool DELTA>
 __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
   __shared__ uint32_t cnt[FV_NB_CNT_WORDS];
+  __shared__ uint32_t cnt2[DELTA ? FV_NB_CNT_WORDS : 4];
   __shared__ uint16_t list[FV_SP_LIST_CAP];
   __shared__ uint32_t ord[FV_SP_STAGE];
   __shared__ uint32_t sh_pos;
@@ -538,7 +592,8 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
   const uint32_t q = blockIdx.x & (FV_NB_CLASSES - 1);
   const uint32_t tid = threadIdx.x;
   const uint32_t c_h = a.group_count[h];
-  if (c_h == 0) {
+  const uint32_t c2_h = DELTA ? a.group_count2[h] : 0u;
+  if (c_h == 0 && c2_h == 0) {
     if (tid == 0) {
       a.bmax_sparse[blockIdx.x] = 0.0f;
       a.slot_count[blockIdx.x] = 0;
@@ -546,15 +601,20 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
     return;
   }
   const uint32_t base = a.group_base[h];
+  const uint32_t base2 = DELTA ? a.group_base2[h] : 0u;
   const float x_h = a.xx[h];
   float ds_max = 0.0f;
   const uint32_t *__restrict__ order = a.order + base;
   const uint32_t n_cols = 2 * a.V;
-  const uint32_t m_ent = c_h * a.w;
-  fv_slot *slots = a.slots + (uint64_t)q * a.slot_stride + (uint64_t)base * a.w;
+  const uint32_t m_ent = max(c_h, c2_h) * a.w;
+  // the block's records: no more than (c_h + c2_h) * w of them, behind those of the lower neurons
+  const uint64_t slot_first = (uint64_t)q * a.slot_stride + (uint64_t)(base + base2) * a.w;
+  fv_slot *slots = a.slots + slot_first;
 
   for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
-  const bool staged_once = c_h <= FV_SP_STAGE;  // the usual case: the neuron's window ids are staged here
+  if (DELTA)
+    for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt2)[i] = make_uint4(0, 0, 0, 0);
+  const bool staged_once = !DELTA && c_h <= FV_SP_STAGE;  // the usual case: the neuron's window ids are staged here
   if (staged_once)
     for (uint32_t i = tid; i < c_h; i += T) ord[i] = order[i];
   fv_lds_barrier();
@@ -567,17 +627,22 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
   uint32_t emitted = 0;
 
   for (uint32_t lo = 0; lo < class_cols; lo += span) {
-    for (uint32_t j0 = 0; j0 < c_h; j0 += FV_SP_STAGE) {
-      const uint32_t n_staged = min(c_h - j0, (uint32_t)FV_SP_STAGE);
-      if (!staged_once) {
-        fv_lds_barrier();  // the previous part has been counted
-        for (uint32_t i = tid; i < n_staged; i += T) ord[i] = order[j0 + i];
-        fv_lds_barrier();
+    for (int l = 0; l < (DELTA ? 2 : 1); ++l) {
+      const uint32_t *__restrict__ ids = l == 0 ? order : a.order2 + base2;
+      const uint32_t n_ids = l == 0 ? c_h : c2_h;
+      uint32_t *counters = l == 0 ? cnt : cnt2;
+      for (uint32_t j0 = 0; j0 < n_ids; j0 += FV_SP_STAGE) {
+        const uint32_t n_staged = min(n_ids - j0, (uint32_t)FV_SP_STAGE);
+        if (!staged_once) {
+          fv_lds_barrier();  // the previous part has been counted
+          for (uint32_t i = tid; i < n_staged; i += T) ord[i] = ids[j0 + i];
+          fv_lds_barrier();
+        }
+        if (narrow)
+          fv_sparse_count_any<true>(counters, ord, n_staged, a.pad_row, a.idx, a.w, q, lo, span, tid);
+        else
+          fv_sparse_count_any<false>(counters, ord, n_staged, a.pad_row, a.idx, a.w, q, lo, span, tid);
       }
-      if (narrow)
-        fv_sparse_count_any<true>(cnt, ord, n_staged, a.pad_row, a.idx, a.w, q, lo, span, tid);
-      else
-        fv_sparse_count_any<false>(cnt, ord, n_staged, a.pad_row, a.idx, a.w, q, lo, span, tid);
     }
     // Every non-zero counter is one distinct element. Their positions are collected in LDS, up to
     // FV_SP_LIST_CAP at a time; a counter is cleared when its element is taken, so what did not fit
@@ -595,6 +660,15 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
         for (int i = 0; i < n_groups; ++i) {
           const uint32_t g4 = min(tid + i * T, (uint32_t)FV_NB_CNT_WORDS / 4 - 1);
           uint4 c4 = ((const uint4 *)cnt)[g4];
+          if (DELTA) {
+            const uint4 d4 = ((const uint4 *)cnt2)[g4];
+            if (narrow) {
+              // a 16-bit half is non-zero in the union if it is in either word: OR keeps that
+              c4.x |= d4.x; c4.y |= d4.y; c4.z |= d4.z; c4.w |= d4.w;
+            } else {
+              c4.x |= d4.x; c4.y |= d4.y; c4.z |= d4.z; c4.w |= d4.w;
+            }
+          }
           if (tid + i * T >= FV_NB_CNT_WORDS / 4) c4 = make_uint4(0, 0, 0, 0);
           const uint32_t cw[4] = {c4.x, c4.y, c4.z, c4.w};
           uint32_t bits = 0;
@@ -636,22 +710,30 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
       // plant the sentinel, take |ds| (the dense term plus count additions of 1/f; a row with
       // xx == 0 has ds == 0)
       for (uint32_t eb = tid; eb < take; eb += 4 * T) {
-        uint32_t pe[4], ne[4];
+        uint32_t pe[4], ne[4], n2e[4];
         float wv[4], fe[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           const uint32_t k = list[min(eb + u * T, take - 1)];
           const uint32_t word = narrow ? cnt[k >> 1] : cnt[k];
           ne[u] = narrow ? (word >> (16 * (k & 1))) & 0xffffu : word;
+          n2e[u] = 0;
+          if (DELTA) {
+            const uint32_t word2 = narrow ? cnt2[k >> 1] : cnt2[k];
+            n2e[u] = narrow ? (word2 >> (16 * (k & 1))) & 0xffffu : word2;
+          }
           const uint32_t col = ((lo + k) << FV_NB_CLASS_SHIFT) | q;
           pe[u] = col * a.ldk + h;
           wv[u] = a.Wt[pe[u]];
           fe[u] = a.invf[col >= a.V ? col - a.V : col];
           if (eb + u * T < take) {
-            if (narrow)
+            if (narrow) {
               atomicAnd(&cnt[k >> 1], 0xffff0000u >> (16 * (k & 1)));
-            else
+              if (DELTA) atomicAnd(&cnt2[k >> 1], 0xffff0000u >> (16 * (k & 1)));
+            } else {
               cnt[k] = 0;
+              if (DELTA) cnt2[k] = 0;
+            }
           }
         }
 #pragma unroll
@@ -663,8 +745,11 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
             rec.wv = wv[u];
             rec.f = fe[u];
             slots[emitted + eb + u * T] = rec;
+            if (DELTA) a.slot_n2[slot_first + emitted + eb + u * T] = n2e[u];
             a.Wt[pe[u]] = __uint_as_float(FV_SENTINEL);
-            if (x_h != 0.0f) ds_max = fv_absmax_keep(ds_max, fv_sparse_ds(x_h, wv[u], fe[u], ne[u]));
+            if (x_h != 0.0f)
+              ds_max = fv_absmax_keep(ds_max, DELTA ? fv_sparse_ds2(x_h, wv[u], fe[u], ne[u], a.delta, n2e[u])
+                                                    : fv_sparse_ds(x_h, wv[u], fe[u], ne[u]));
           }
       }
       emitted += take;
@@ -688,6 +773,9 @@ struct fv_dense_args {
   uint64_t slot_stride;
   const uint32_t *slot_count;  // records of each block of the sparse launch
   const uint32_t *group_base;
+  const uint32_t *group_base2;  // anti-Hebbian form only, like slot_n2 and delta
+  const uint32_t *slot_n2;
+  float delta;
   float *bmax;           // n_bmax block maxima of |ds|: dense blocks, then the sparse kernel's blocks
   float *scalars;
   uint32_t total4, ldk4, ldk, V, K, w, n_bmax, dense_blocks;
@@ -827,25 +915,34 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
 
 // Kernel 6: the final value of every sparse element goes over its sentinel. Runs after the dense
 // update so no dense thread can mistake a finished element for an ordinary weight.
+template <bool DELTA>
 __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
   // block (h, q) of the sparse launch wrote slot_count records at the start of its part of region q
   const uint32_t count = a.slot_count[blockIdx.x];
   if (count == 0) return;
   const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT, q = blockIdx.x & (FV_NB_CLASSES - 1);
-  const fv_slot *slots = a.slots + (uint64_t)q * a.slot_stride + (uint64_t)a.group_base[h] * a.w;
+  const uint64_t slot_first =
+      (uint64_t)q * a.slot_stride + (uint64_t)(a.group_base[h] + (DELTA ? a.group_base2[h] : 0u)) * a.w;
+  const fv_slot *slots = a.slots + slot_first;
   const float x = a.xx[h];
   const float nc = a.scalars[0];
   const float s = a.prec > nc ? a.eps / a.prec : a.eps / nc;
   for (uint32_t eb = threadIdx.x; eb < count; eb += 4 * 256) {  // four records in flight per thread
     fv_slot sl[4];
+    uint32_t n2[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) sl[u] = slots[min(eb + u * 256, count - 1)];
+    for (int u = 0; u < 4; ++u) {
+      sl[u] = slots[min(eb + u * 256, count - 1)];
+      n2[u] = DELTA ? a.slot_n2[slot_first + min(eb + u * 256, count - 1)] : 0u;
+    }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       if (eb + u * 256 >= count) break;
       float out = sl[u].wv;  // a row with xx == 0 is not updated: the saved weight goes back
       if (x != 0.0f) {
-        const float d = __fmul_rn(s, fv_sparse_ds(x, sl[u].wv, sl[u].f, sl[u].n));
+        const float ds = DELTA ? fv_sparse_ds2(x, sl[u].wv, sl[u].f, sl[u].n, a.delta, n2[u])
+                               : fv_sparse_ds(x, sl[u].wv, sl[u].f, sl[u].n);
+        const float d = __fmul_rn(s, ds);
         if (fabsf(d) > a.update_cut) out = __fadd_rn(sl[u].wv, d);
       }
       ((float *)a.Wt4)[sl[u].p] = out;
@@ -927,6 +1024,14 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   (void)hipFree(t->bmax);
   (void)hipFree(t->win);
   (void)hipFree(t->win16);
+  (void)hipFree(t->win2);
+  (void)hipFree(t->win2_16);
+  (void)hipFree(t->sc2);
+  (void)hipFree(t->order2);
+  (void)hipFree(t->group_base2);
+  (void)hipFree(t->group_count2);
+  (void)hipFree(t->slot_n2);
+  (void)hipFree(t->slots2);
   (void)hipFree(t->sc);
   (void)hipFree(t->xx);
   (void)hipFree(t->scalars);
@@ -973,8 +1078,11 @@ extern "C" int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_tr
   FV_REQUIRE(cfg->vocab >= 1 && cfg->vocab < (1ull << 30), FV_ERR_INVALID,
              "vocab = %llu is out of range", (unsigned long long)cfg->vocab);
   FV_REQUIRE(cfg->tie_rule <= 1, FV_ERR_INVALID, "tie_rule must be 0 or 1");
-  FV_REQUIRE(cfg->delta == 0.0f, FV_ERR_INVALID,
-             "delta != 0 (anti-Hebbian term on the m-th winner) is not implemented");
+  FV_REQUIRE(cfg->delta == cfg->delta && fabsf(cfg->delta) <= 1.0e6f, FV_ERR_INVALID, "delta = %g is out of range",
+             (double)cfg->delta);
+  // the slot regions of a step with delta != 0 hold twice as many records
+  FV_REQUIRE(cfg->delta == 0.0f || (uint64_t)cfg->batch * cfg->window < (1ull << 30), FV_ERR_INVALID,
+             "batch x window = %llu is out of range for delta != 0", (unsigned long long)cfg->batch * cfg->window);
   const uint32_t ldk = fv_ldk(cfg->hid);
   const uint64_t N = 2 * cfg->vocab;
   FV_REQUIRE(N * ldk < 0xffffffffull - (1u << 24), FV_ERR_INVALID,
@@ -1165,15 +1273,36 @@ extern "C" int fv_trainer_get_permutation(fv_trainer *t, uint64_t *out_perm, uin
 
 
 template <int NV>
-static void fv_launch_gather(const fv_gather_args &a, hipStream_t stream) {
+static void fv_launch_gather(const fv_gather_args &a, bool with_second, hipStream_t stream) {
   const uint32_t waves = (a.n + FV_GATHER_WINDOWS - 1) / FV_GATHER_WINDOWS;
-  hipLaunchKernelGGL(fv_gather_winner_kernel<NV>, dim3((waves + 3) / 4), dim3(256), 0, stream, a);
+  if (with_second)
+    hipLaunchKernelGGL((fv_gather_winner_kernel<NV, true>), dim3((waves + 3) / 4), dim3(256), 0, stream, a);
+  else
+    hipLaunchKernelGGL((fv_gather_winner_kernel<NV, false>), dim3((waves + 3) / 4), dim3(256), 0, stream, a);
 }
 
 // Enqueues the kernels of one step (those whose bit is set in `which`); ev (nullable) receives
 // FV_TRAIN_KERNELS + 1 events recorded around them.
-static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps, hipEvent_t *ev,
+// Buffers of the anti-Hebbian form, on first use.
+static int fv_trainer_alloc_delta(fv_trainer *t) {
+  if (t->win2) return FV_OK;
+  const size_t B = t->B, bw = (size_t)t->B * t->w;
+  FV_HIP(hipMalloc((void **)&t->win2, B * sizeof(int32_t)));
+  FV_HIP(hipMalloc((void **)&t->win2_16, (B + 64) * sizeof(uint16_t)));
+  FV_HIP(hipMemsetAsync(t->win2_16, 0, (B + 64) * sizeof(uint16_t), t->stream));
+  FV_HIP(hipMalloc((void **)&t->sc2, B * sizeof(float)));
+  FV_HIP(hipMalloc((void **)&t->order2, B * sizeof(uint32_t)));
+  FV_HIP(hipMalloc((void **)&t->group_base2, (size_t)t->K * sizeof(uint32_t)));
+  FV_HIP(hipMalloc((void **)&t->group_count2, (size_t)t->K * sizeof(uint32_t)));
+  FV_HIP(hipMalloc((void **)&t->slots2, 2 * FV_NB_CLASSES * bw * sizeof(fv_slot)));
+  FV_HIP(hipMalloc((void **)&t->slot_n2, 2 * FV_NB_CLASSES * bw * sizeof(uint32_t)));
+  return FV_OK;
+}
+
+static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps, float delta, hipEvent_t *ev,
                            unsigned which = 0x3f) {
+  const bool anti = delta != 0.0f;  // the second neuron of every window takes part (flyvec/src/cuda_funcs.cu:726-734)
+  if (anti) FV_TRY(fv_trainer_alloc_delta(t));
   fv_gather_args g;
   g.Wt = t->Wt;
   g.corpus = t->corpus;
@@ -1183,6 +1312,9 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.win = t->win;
   g.win16 = t->win16;
   g.sc = t->sc;
+  g.win2 = t->win2;
+  g.win2_16 = t->win2_16;
+  g.sc2 = t->sc2;
   g.first = first;
   g.n = n;
   g.K = t->K;
@@ -1192,7 +1324,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.tie_rule = t->cfg.tie_rule;
   if (ev) FV_HIP(hipEventRecord(ev[0], t->stream));
   if (which & 1u) switch ((t->K + 63) / 64) {
-#define FV_CASE(NV) case NV: fv_launch_gather<NV>(g, t->stream); break;
+#define FV_CASE(NV) case NV: fv_launch_gather<NV>(g, anti, t->stream); break;
     FV_CASE(1) FV_CASE(2) FV_CASE(3) FV_CASE(4) FV_CASE(5) FV_CASE(6) FV_CASE(7) FV_CASE(8)
     FV_CASE(9) FV_CASE(10) FV_CASE(11) FV_CASE(12) FV_CASE(13) FV_CASE(14) FV_CASE(15) FV_CASE(16)
     FV_CASE(17) FV_CASE(18) FV_CASE(19) FV_CASE(20) FV_CASE(21) FV_CASE(22) FV_CASE(23) FV_CASE(24)
@@ -1210,13 +1342,28 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   gr.group_count = t->group_count;
   gr.xx = t->xx;
   gr.n = n;
+  gr.scale = 1.0f;
+  gr.accumulate = 0;
   // a thread's run of the winner array should fit its 64-bit match mask
   const unsigned gr_threads = n <= 16384 ? 256 : FV_NB_MAX_THREADS;
-  if (which & 2u) {
-    if (n <= 64 * gr_threads && n < 65536)
-      hipLaunchKernelGGL(fv_group_kernel<true>, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
-    else
-      hipLaunchKernelGGL(fv_group_kernel<false>, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
+  // with delta != 0 a second launch groups the windows by their second neuron and adds
+  // -delta * (their scaled activations) to xx
+  for (int l = 0; l < (anti ? 2 : 1); ++l) {
+    if (l == 1) {
+      gr.win = t->win2_16;
+      gr.sc = t->sc2;
+      gr.order = t->order2;
+      gr.group_base = t->group_base2;
+      gr.group_count = t->group_count2;
+      gr.scale = -delta;
+      gr.accumulate = 1;
+    }
+    if (which & 2u) {
+      if (n <= 64 * gr_threads && n < 65536)
+        hipLaunchKernelGGL(fv_group_kernel<true>, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
+      else
+        hipLaunchKernelGGL(fv_group_kernel<false>, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
+    }
   }
   if (ev) FV_HIP(hipEventRecord(ev[2], t->stream));
   fv_sparse_args sp;
@@ -1225,8 +1372,13 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.group_count = t->group_count;
   sp.idx = t->idx;
   sp.Wt = t->Wt;
-  sp.slots = t->slots;
-  sp.slot_stride = (uint64_t)t->B * t->w;
+  sp.slots = anti ? t->slots2 : t->slots;
+  sp.slot_stride = (uint64_t)t->B * t->w * (anti ? 2 : 1);
+  sp.order2 = t->order2;
+  sp.group_base2 = t->group_base2;
+  sp.group_count2 = t->group_count2;
+  sp.slot_n2 = t->slot_n2;
+  sp.delta = delta;
   sp.xx = t->xx;
   sp.invf = t->invf;
   sp.bmax_sparse = t->bmax + t->dense_blocks;
@@ -1235,17 +1387,25 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.ldk = t->ldk;
   sp.w = t->w;
   sp.V = (uint32_t)t->V;
-  if (which & 4u) hipLaunchKernelGGL(fv_sparse_kernel, dim3(t->K * FV_NB_CLASSES), dim3(FV_SP_THREADS), 0, t->stream, sp);
+  if (which & 4u) {
+    if (anti)
+      hipLaunchKernelGGL(fv_sparse_kernel<true>, dim3(t->K * FV_NB_CLASSES), dim3(FV_SP_THREADS), 0, t->stream, sp);
+    else
+      hipLaunchKernelGGL(fv_sparse_kernel<false>, dim3(t->K * FV_NB_CLASSES), dim3(FV_SP_THREADS), 0, t->stream, sp);
+  }
   if (ev) FV_HIP(hipEventRecord(ev[3], t->stream));
   fv_dense_args d;
   d.Wt4 = (float4 *)t->Wt;
   d.xx = t->xx;
   d.invf = t->invf;
-  d.slots = t->slots;
+  d.slots = anti ? t->slots2 : t->slots;
   d.slot_count = t->slot_count;
   d.group_base = t->group_base;
+  d.group_base2 = t->group_base2;
+  d.slot_n2 = t->slot_n2;
+  d.delta = delta;
   d.w = t->w;
-  d.slot_stride = (uint64_t)t->B * t->w;
+  d.slot_stride = (uint64_t)t->B * t->w * (anti ? 2 : 1);
   d.bmax = t->bmax;
   d.scalars = t->scalars;
   d.total4 = t->total4;
@@ -1264,12 +1424,18 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
   if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
-  if (which & 32u) hipLaunchKernelGGL(fv_slot_update_kernel, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, d);
+  if (which & 32u) {
+    if (anti)
+      hipLaunchKernelGGL(fv_slot_update_kernel<true>, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, d);
+    else
+      hipLaunchKernelGGL(fv_slot_update_kernel<false>, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, d);
+  }
   if (ev) FV_HIP(hipEventRecord(ev[6], t->stream));
   FV_HIP(hipGetLastError());
   t->last_n = n;
   t->last_first = first;
   t->last_eps = eps;
+  t->last_delta = delta;
   return FV_OK;
 }
 
@@ -1287,7 +1453,30 @@ static int fv_check_step(fv_trainer *t, uint64_t first, uint64_t n) {
 
 extern "C" int fv_trainer_step(fv_trainer *t, uint64_t first_window, uint32_t n_windows, float eps) {
   FV_TRY(fv_check_step(t, first_window, n_windows));
-  return fv_enqueue_step(t, first_window, n_windows, eps, nullptr);
+  return fv_enqueue_step(t, first_window, n_windows, eps, 0.0f, nullptr);
+}
+
+extern "C" int fv_trainer_step_delta(fv_trainer *t, uint64_t first_window, uint32_t n_windows, float eps,
+                                     float delta) {
+  FV_TRY(fv_check_step(t, first_window, n_windows));
+  return fv_enqueue_step(t, first_window, n_windows, eps, delta, nullptr);
+}
+
+extern "C" int fv_trainer_epoch_delta(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs, float *out_delta) {
+  FV_REQUIRE(t && out_delta, FV_ERR_INVALID, "null argument");
+  // flyvec/src/cuda_funcs.cu:1230: double arithmetic on the fp32 epoch, rounded to fp32 once
+  *out_delta = (float)(t->cfg.delta * 0.5 * (1.0 + tanh((((float)epoch_id) - (0.125 * n_epochs)) / 10.0)));
+  return FV_OK;
+}
+
+extern "C" int fv_trainer_get_second_winners(fv_trainer *t, int32_t *out_seconds, uint32_t capacity) {
+  FV_REQUIRE(t && out_seconds, FV_ERR_INVALID, "null argument");
+  FV_REQUIRE(t->win2 && t->last_delta != 0.0f, FV_ERR_STATE, "the last step had no anti-Hebbian term");
+  FV_REQUIRE(capacity >= t->last_n, FV_ERR_INVALID, "capacity %u below the %u windows of the last step", capacity,
+             t->last_n);
+  FV_HIP(hipStreamSynchronize(t->stream));
+  FV_HIP(hipMemcpy(out_seconds, t->win2, (size_t)t->last_n * sizeof(int32_t), hipMemcpyDeviceToHost));
+  return FV_OK;
 }
 
 extern "C" int fv_trainer_epoch_eps(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs, float *out_eps) {
@@ -1302,11 +1491,12 @@ extern "C" int fv_trainer_run_epoch(fv_trainer *t, uint64_t epoch_id, uint64_t n
   FV_REQUIRE(t->have_corpus, FV_ERR_STATE, "no corpus set");
   FV_REQUIRE(t->have_weights, FV_ERR_STATE, "no weights set");
   FV_REQUIRE(n_epochs > 0, FV_ERR_INVALID, "n_epochs must be positive");
-  float eps = 0.0f;
+  float eps = 0.0f, delta = 0.0f;
   FV_TRY(fv_trainer_epoch_eps(t, epoch_id, n_epochs, &eps));
+  FV_TRY(fv_trainer_epoch_delta(t, epoch_id, n_epochs, &delta));
   for (uint64_t k = 0; k < t->n_windows; k += t->B) {
     const uint64_t n = t->n_windows - k < t->B ? t->n_windows - k : t->B;
-    FV_TRY(fv_enqueue_step(t, k, (uint32_t)n, eps, nullptr));
+    FV_TRY(fv_enqueue_step(t, k, (uint32_t)n, eps, delta, nullptr));
   }
   FV_HIP(hipStreamSynchronize(t->stream));
   return FV_OK;
@@ -1369,7 +1559,7 @@ extern "C" int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint3
   FV_HIP(hipStreamSynchronize(t->stream));
   FV_HIP(hipEventRecord(e0, t->stream));
   for (uint32_t s = 0; s < n_steps && rc == FV_OK; ++s)
-    rc = fv_enqueue_step(t, first_window + (uint64_t)s * t->B, t->B, eps, nullptr);
+    rc = fv_enqueue_step(t, first_window + (uint64_t)s * t->B, t->B, eps, 0.0f, nullptr);
   FV_HIP(hipEventRecord(e1, t->stream));
   FV_HIP(hipStreamSynchronize(t->stream));
   FV_HIP(hipEventElapsedTime(out_total_ms, e0, e1));
@@ -1381,7 +1571,7 @@ extern "C" int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint3
   std::vector<hipEvent_t> ev((size_t)n_steps * per);
   for (auto &e : ev) FV_HIP(hipEventCreate(&e));
   for (uint32_t s = 0; s < n_steps && rc == FV_OK; ++s)
-    rc = fv_enqueue_step(t, first_window + (uint64_t)s * t->B, t->B, eps, &ev[(size_t)s * per]);
+    rc = fv_enqueue_step(t, first_window + (uint64_t)s * t->B, t->B, eps, 0.0f, &ev[(size_t)s * per]);
   FV_HIP(hipStreamSynchronize(t->stream));
   for (int k = 0; k < FV_TRAIN_KERNELS; ++k) out_kernel_ms[k] = 0.0f;
   if (rc == FV_OK) {
@@ -1404,10 +1594,10 @@ extern "C" int fv_trainer_time_kernel(fv_trainer *t, uint32_t kernel_index, uint
   FV_HIP(hipEventCreate(&e0));
   FV_HIP(hipEventCreate(&e1));
   FV_HIP(hipStreamSynchronize(t->stream));
-  int rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, nullptr, 1u << kernel_index);  // warm-up
+  int rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, t->last_delta, nullptr, 1u << kernel_index);  // warm-up
   FV_HIP(hipEventRecord(e0, t->stream));
   for (uint32_t r = 0; r < reps && rc == FV_OK; ++r)
-    rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, nullptr, 1u << kernel_index);
+    rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, t->last_delta, nullptr, 1u << kernel_index);
   FV_HIP(hipEventRecord(e1, t->stream));
   FV_HIP(hipStreamSynchronize(t->stream));
   float ms = 0.0f;

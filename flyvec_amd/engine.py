@@ -113,8 +113,23 @@ class Trainer:
         return out
 
     # -- the hot path ------------------------------------------------------------------------
-    def step(self, first_window, n_windows, eps):
-        check(self.lib.fv_trainer_step(self.handle, int(first_window), int(n_windows), float(eps)))
+    def step(self, first_window, n_windows, eps, delta=0.0):
+        """One minibatch; delta != 0 adds the anti-Hebbian term on the second neuron of every window."""
+        if delta:
+            check(self.lib.fv_trainer_step_delta(self.handle, int(first_window), int(n_windows), float(eps),
+                                                 float(delta)))
+        else:
+            check(self.lib.fv_trainer_step(self.handle, int(first_window), int(n_windows), float(eps)))
+
+    def epoch_delta(self, epoch_id, n_epochs):
+        out = C.c_float(0)
+        check(self.lib.fv_trainer_epoch_delta(self.handle, int(epoch_id), int(n_epochs), C.byref(out)))
+        return out.value
+
+    def second_winners(self, n):
+        out = np.empty(int(n), dtype=np.int32)
+        check(self.lib.fv_trainer_get_second_winners(self.handle, ptr(out), len(out)))
+        return out
 
     def run_epoch(self, epoch_id, n_epochs):
         check(self.lib.fv_trainer_run_epoch(self.handle, int(epoch_id), int(n_epochs)))

@@ -41,7 +41,7 @@ def build_parser():
     p.add_argument("--W", default=11, type=int, help="Size of the W-gram sliding window")
     p.add_argument("--hid", default=400, type=int, help="Number of hidden units (neurons)")
     p.add_argument("--initial_learning_rate", default=0.002, type=float, help="Initial learning rate")
-    p.add_argument("--delta", default=0.0, type=float, help="Anti-Hebbian strength (only 0 is built)")
+    p.add_argument("--delta", default=0.0, type=float, help="Anti-Hebbian strength on the second neuron of a window (flyvec/src/cuda_funcs.cu:1230 schedules it over the epochs)")
     p.add_argument("--mu", default=0.0, type=float, help="Mean of the random normal initialisation")
     p.add_argument("--sigma", default=0.02, type=float, help="Stdev of the random normal initialisation")
     p.add_argument("--Nep", default=15, type=int, help="Maximum number of epochs, fewer if starting from a checkpoint")

@@ -100,7 +100,7 @@ typedef struct fv_train_config {
   uint32_t tie_rule;           /* argmax ties: 0 lowest index, 1 the reference's lane-tree order
                                   (flyvec/src/cuda_funcs.cu:488-561) */
   float initial_learning_rate; /* "initial_learning_rate" */
-  float delta;                 /* "delta": must be 0 (anti-Hebbian term not built) */
+  float delta;                 /* "delta": strength of the anti-Hebbian term on the second neuron (0 = none) */
   float prec;                  /* "prec" */
   uint32_t reserved;           /* 0 */
 } fv_train_config;
@@ -138,6 +138,17 @@ int fv_trainer_get_permutation(fv_trainer *t, uint64_t *out_perm, uint64_t capac
 /* One pass of the minibatch loop body, flyvec/src/cuda_funcs.cu:1662-1803, on windows
  * perm[first_window .. first_window + n_windows) with n_windows <= batch. Asynchronous. */
 int fv_trainer_step(fv_trainer *t, uint64_t first_window, uint32_t n_windows, float eps);
+
+/* The same step with the anti-Hebbian term of strength `delta` (flyvec/src/cuda_funcs.cu:495-548,
+ * 667-668, 726-734): the second neuron of every window -- the winner search repeated with the
+ * winner's activation overwritten by -9999.9999 -- receives -delta times what the winner receives.
+ * fv_trainer_step is this with delta = 0. */
+int fv_trainer_step_delta(fv_trainer *t, uint64_t first_window, uint32_t n_windows, float eps, float delta);
+/* flyvec/src/cuda_funcs.cu:1230: delta_epoch = delta * 0.5 * (1 + tanh((epoch - 0.125 n_epochs) / 10))
+ * with delta from the configuration; fv_trainer_run_epoch uses it. */
+int fv_trainer_epoch_delta(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs, float *out_delta);
+/* Test hook: the second neurons of the last step (only after a step with delta != 0). */
+int fv_trainer_get_second_winners(fv_trainer *t, int32_t *out_seconds, uint32_t capacity);
 
 /* flyvec/src/cuda_funcs.cu:1220 launch_epoch_INPUT_AS_INT: eps = lr0 * (1 - epoch/n_epochs),
  * then every minibatch of the current permutation (the last one takes the remainder only).

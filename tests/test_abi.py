@@ -57,7 +57,7 @@ def test_argument_errors_need_no_device():
                            delta=0.0, prec=1e-30, reserved=0)
     assert lib.fv_trainer_create(C.byref(cfg), C.byref(out)) == _lib.FV_ERR_INVALID
     assert b"hid" in lib.fv_last_error()
-    cfg.hid, cfg.delta = 400, 0.5
+    cfg.hid, cfg.delta = 400, float("nan")
     assert lib.fv_trainer_create(C.byref(cfg), C.byref(out)) == _lib.FV_ERR_INVALID
     assert b"delta" in lib.fv_last_error()
 

@@ -324,3 +324,87 @@ def test_large_config_shape(gpu, oracle_lib):
     wo = to.train_steps(Wo, tokens, starts, perm, 0, B, steps, w, invf, eps)
     assert np.array_equal(np.concatenate(wins), wo)
     assert np.array_equal(Wg, Wo)
+
+
+# ---- anti-Hebbian term (delta != 0) -----------------------------------------------------------------
+
+def run_both_delta(to, V, K, w, B, steps, delta, tie=0, n_tokens=60000, W0=None, sigma=0.02, seed=0):
+    from flyvec_amd import synthetic
+    tokens, offsets = small_corpus(n_tokens, V, seed=seed)
+    if W0 is None:
+        W0 = synthetic.synapses(K, V, seed=5 + seed, sigma=sigma)
+    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, tie=tie)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    eps = t.epoch_eps(0, 15)
+    steps = min(steps, t.num_windows // B)
+    Wo = W0.copy()
+    for s in range(steps):
+        t.step(s * B, B, eps, delta=delta)
+        idx = to.inflate(tokens, starts, perm, s * B, B, w, V)
+        ref = to.train_step(Wo, idx, invf, eps, tie_rule=tie, delta=delta)
+        assert np.array_equal(t.winners(B), ref["winners"]), f"winners, step {s}"
+        assert np.array_equal(t.second_winners(B), ref["seconds"]), f"second neurons, step {s}"
+        xx, nc = t.step_stats()
+        assert np.array_equal(xx, ref["xx"]) and nc == ref["nc"], f"xx / max|ds|, step {s}"
+    Wg = t.get_weights()
+    t.close()
+    return Wg, Wo
+
+
+@pytest.mark.parametrize("tie", [0, 1])
+def test_delta_small_config_bit_exact(gpu, oracle_lib, tie):
+    Wg, Wo = run_both_delta(oracle_lib, V=500, K=400, w=11, B=512, steps=10, delta=0.4, tie=tie)
+    assert np.array_equal(Wg, Wo)
+
+
+@pytest.mark.parametrize("K,w,V,B", [(1, 1, 5, 1), (2, 3, 9, 7), (65, 15, 200, 256), (130, 64, 300, 64),
+                                     (30, 11, 30000, 700)])
+def test_delta_shapes_bit_exact(gpu, oracle_lib, K, w, V, B):
+    n_tokens = 40000 if V < 20000 else 120000
+    Wg, Wo = run_both_delta(oracle_lib, V=V, K=K, w=w, B=B, steps=4, delta=0.25, n_tokens=n_tokens)
+    assert np.array_equal(Wg, Wo)
+
+
+def test_delta_with_ties_and_heavy_neurons(gpu, oracle_lib):
+    # coarse weights: ties in both searches; then two neurons that take every first and second place
+    # of 7000 windows (32-bit counters in both counter arrays)
+    from flyvec_amd import synthetic
+    rng = np.random.default_rng(11)
+    V, K = 60, 200
+    W0 = (rng.integers(-2, 3, size=(K, 2 * V)) * 0.25).astype(f32)
+    for tie in (0, 1):
+        Wg, Wo = run_both_delta(oracle_lib, V=V, K=K, w=5, B=256, steps=4, delta=0.5, tie=tie, W0=W0)
+        assert np.array_equal(Wg, Wo)
+    V, K, B = 300, 6, 7000
+    W0 = synthetic.synapses(K, V, sigma=0.01)
+    W0[2] = np.abs(W0[2]) + 1.0
+    W0[4] = np.abs(W0[4]) + 0.5
+    Wg, Wo = run_both_delta(oracle_lib, V=V, K=K, w=11, B=B, steps=2, delta=0.3, W0=W0, n_tokens=120000)
+    assert np.array_equal(Wg, Wo)
+
+
+def test_delta_epoch_schedule_and_driver(gpu, oracle_lib):
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    V, K, w, B = 200, 96, 11, 300
+    tokens, offsets = small_corpus(9000, V, n_masked=10)
+    W0 = synthetic.synapses(K, V, sigma=0.02)
+    t = Trainer(V, K, w, B, initial_learning_rate=2e-3, delta=0.4)
+    t.set_corpus(tokens, offsets)
+    perm = np.random.default_rng(6).permutation(t.num_windows).astype(np.uint64)
+    t.set_permutation(perm)
+    t.set_weights(W0)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    nwin = t.num_windows
+    Wo = W0.copy()
+    for ep in (0, 7, 14):
+        delta = to.epoch_delta(0.4, ep, 15)
+        assert t.epoch_delta(ep, 15) == delta and delta > 0
+        t.run_epoch(ep, 15)
+        to.train_steps(Wo, tokens, starts, perm, 0, B, nwin // B + 1, w, invf, to.epoch_eps(2e-3, ep, 15),
+                       delta=delta)
+        assert np.array_equal(t.get_weights(), Wo), f"epoch {ep}"
+    t.step(0, B, 1e-3)                       # a plain step afterwards still works
+    with pytest.raises(Exception):
+        t.second_winners(B)                  # and has no second neurons to show
+    t.close()
