@@ -45,3 +45,21 @@ def test_cli_trains_saves_resumes(gpu, oracle_lib, tmp_path):
     # a trained checkpoint feeds the hashing wrapper
     model = FlyVec(out / names[1], tokenizer=["<UNK>"] + [f"t{i}" for i in range(1, V)], normalize_synapses=False)
     assert model.get_sparse_embedding("t5", 10)["embedding"].sum() <= 10
+
+
+def test_cli_with_anti_hebbian_term(gpu, tmp_path):
+    """--delta reaches the trainer and follows the epoch schedule of flyvec/src/cuda_funcs.cu:1230."""
+    from flyvec_amd.train_flyvec import main
+    V = 300
+    tokens, offsets = small_corpus(20000, V)
+    np.save(tmp_path / "encodings.npy", tokens)
+    np.save(tmp_path / "offsets.npy", offsets)
+    outs = {}
+    for name, delta in (("plain", "0"), ("anti", "0.4")):
+        out = tmp_path / name
+        assert main([str(tmp_path / "encodings.npy"), str(tmp_path / "offsets.npy"), "-o", str(out), "--hid", "64",
+                     "-b", "256", "--Nep", "2", "--save_every", "2", "--seed", "1", "--delta", delta]) == 0
+        (ckpt,) = list(out.iterdir())
+        outs[name] = np.load(ckpt)
+        assert np.isfinite(outs[name]).all()
+    assert not np.array_equal(outs["plain"], outs["anti"])
