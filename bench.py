@@ -47,13 +47,13 @@ HASH = dict(K=400, V=20000, w=11, k=32, n=1 << 20)
 # WRITE_SIZE reads them all: x1.0). Traffic below the algorithmic bytes means the rest was served
 # by the L2 caches.
 MEASURED_TRAFFIC = {
-    "update": (31376.0 * 2.0 + 62504.1) * 1024,
-    "absmax_ds": (31277.9 * 2.0 + 64.0) * 1024,
-    "gather_winner": (26644.9 * 2.0 + 703.3) * 1024,
-    "sparse_owners": (4567.9 * 2.0 + 2483.7) * 1024,
-    "group_xx": (303.0 * 2.0 + 87.2) * 1024,
-    "slot_update": (619.5 * 2.0 + 1501.2) * 1024,
-    "hash": (2245698.3 * 2.0 + 78826.3) * 1024,
+    "update": (31376.0 * 2.0 + 62508.3) * 1024,
+    "absmax_ds": (31272.4 * 2.0 + 64.0) * 1024,
+    "gather_winner": (26651.2 * 2.0 + 723.0) * 1024,
+    "sparse_owners": (4569.6 * 2.0 + 2483.8) * 1024,
+    "group_xx": (305.5 * 2.0 + 87.2) * 1024,
+    "slot_update": (620.0 * 2.0 + 1501.2) * 1024,
+    "hash": (2245608.2 * 2.0 + 78841.5) * 1024,
 }
 
 
