@@ -996,6 +996,8 @@ static unsigned fv_perm_blocks(uint64_t n) {
 
 // ---- host side ------------------------------------------------------------------------------
 
+static void fv_trainer_free_delta(fv_trainer *t);
+
 static void fv_trainer_free_corpus(fv_trainer *t) {
   (void)hipFree(t->corpus);
   (void)hipFree(t->starts);
@@ -1024,14 +1026,7 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   (void)hipFree(t->bmax);
   (void)hipFree(t->win);
   (void)hipFree(t->win16);
-  (void)hipFree(t->win2);
-  (void)hipFree(t->win2_16);
-  (void)hipFree(t->sc2);
-  (void)hipFree(t->order2);
-  (void)hipFree(t->group_base2);
-  (void)hipFree(t->group_count2);
-  (void)hipFree(t->slot_n2);
-  (void)hipFree(t->slots2);
+  fv_trainer_free_delta(t);
   (void)hipFree(t->sc);
   (void)hipFree(t->xx);
   (void)hipFree(t->scalars);
@@ -1284,8 +1279,25 @@ static void fv_launch_gather(const fv_gather_args &a, bool with_second, hipStrea
 // Enqueues the kernels of one step (those whose bit is set in `which`); ev (nullable) receives
 // FV_TRAIN_KERNELS + 1 events recorded around them.
 // Buffers of the anti-Hebbian form, on first use.
+static void fv_trainer_free_delta(fv_trainer *t) {
+  (void)hipFree(t->win2);
+  (void)hipFree(t->win2_16);
+  (void)hipFree(t->sc2);
+  (void)hipFree(t->order2);
+  (void)hipFree(t->group_base2);
+  (void)hipFree(t->group_count2);
+  (void)hipFree(t->slots2);
+  (void)hipFree(t->slot_n2);
+  t->win2 = nullptr;
+  t->win2_16 = nullptr;
+  t->sc2 = nullptr;
+  t->order2 = t->group_base2 = t->group_count2 = t->slot_n2 = nullptr;
+  t->slots2 = nullptr;
+}
+
 static int fv_trainer_alloc_delta(fv_trainer *t) {
-  if (t->win2) return FV_OK;
+  if (t->slot_n2) return FV_OK;  // the last one allocated: all are there
+  fv_trainer_free_delta(t);      // what an earlier, failed attempt left
   const size_t B = t->B, bw = (size_t)t->B * t->w;
   FV_HIP(hipMalloc((void **)&t->win2, B * sizeof(int32_t)));
   FV_HIP(hipMalloc((void **)&t->win2_16, (B + 64) * sizeof(uint16_t)));
