@@ -792,24 +792,14 @@ __device__ __forceinline__ float fv_dense_ds(float x, float w) {
 // changes only where |s * ds| exceeds the cut; sentinel positions belong to the slot kernel.
 __device__ __forceinline__ void fv_update_four(const fv_dense_args &a, uint32_t p4, float4 w, const float4 x,
                                                const float s) {
-  const bool s0 = fv_is_sentinel(w.x), s1 = fv_is_sentinel(w.y), s2 = fv_is_sentinel(w.z),
-             s3 = fv_is_sentinel(w.w);
-  bool c0 = false, c1 = false, c2 = false, c3 = false;
+  bool changed = false;
   float d;
-  d = __fmul_rn(s, fv_dense_ds(x.x, w.x)); if (fabsf(d) > a.update_cut) { w.x = __fadd_rn(w.x, d); c0 = true; }
-  d = __fmul_rn(s, fv_dense_ds(x.y, w.y)); if (fabsf(d) > a.update_cut) { w.y = __fadd_rn(w.y, d); c1 = true; }
-  d = __fmul_rn(s, fv_dense_ds(x.z, w.z)); if (fabsf(d) > a.update_cut) { w.z = __fadd_rn(w.z, d); c2 = true; }
-  d = __fmul_rn(s, fv_dense_ds(x.w, w.w)); if (fabsf(d) > a.update_cut) { w.w = __fadd_rn(w.w, d); c3 = true; }
-  if (s0 | s1 | s2 | s3) {
-    // store the other components one by one
-    float *wp = (float *)&a.Wt4[p4];
-    if (c0) wp[0] = w.x;
-    if (c1) wp[1] = w.y;
-    if (c2) wp[2] = w.z;
-    if (c3) wp[3] = w.w;
-  } else if (c0 | c1 | c2 | c3) {
-    a.Wt4[p4] = w;
-  }
+  d = __fmul_rn(s, fv_dense_ds(x.x, w.x)); if (fabsf(d) > a.update_cut) { w.x = __fadd_rn(w.x, d); changed = true; }
+  d = __fmul_rn(s, fv_dense_ds(x.y, w.y)); if (fabsf(d) > a.update_cut) { w.y = __fadd_rn(w.y, d); changed = true; }
+  d = __fmul_rn(s, fv_dense_ds(x.z, w.z)); if (fabsf(d) > a.update_cut) { w.z = __fadd_rn(w.z, d); changed = true; }
+  d = __fmul_rn(s, fv_dense_ds(x.w, w.w)); if (fabsf(d) > a.update_cut) { w.w = __fadd_rn(w.w, d); changed = true; }
+  // A sentinel has ds = 0 here and goes back as it came: the slot kernel, a later launch, replaces it.
+  if (changed) a.Wt4[p4] = w;
 }
 
 // 16-byte loads a thread of a dense pass has in flight, and the blocks per compute unit of its launch
