@@ -76,6 +76,9 @@ SIGNATURES = {
     "fv_trainer_run_epoch": [_vp, _u64, _u64],
     "fv_trainer_epoch_eps": [_vp, _u64, _u64, C.POINTER(_f32)],
     "fv_trainer_sync": [_vp],
+    "fv_trainer_set_dense_launches": [_vp, _u32],
+    "fv_trainer_get_dense_launches": [_vp, C.POINTER(_u32)],
+    "fv_trainer_set_wait_limit": [_vp, _u32],
     "fv_trainer_get_winners": [_vp, _vp, _u32],
     "fv_trainer_get_step_stats": [_vp, _vp, C.POINTER(_f32)],
     "fv_trainer_row_norms": [_vp, _u32, _vp],

@@ -80,7 +80,7 @@ struct fv_trainer {
   uint32_t *slot_count;  // K * FV_NB_CLASSES
   float *xx;        // ldk
   float *bmax;      // max|ds| of each block of the absmax launch, then of each block of the sparse launch
-  float *scalars;   // [0] max|ds| of the last step
+  float *scalars;   // [0] max|ds| of the last step, [1] non-zero once a single-launch dense pass has given up
   uint32_t last_n;
   uint64_t last_first;
   float last_eps;
@@ -88,6 +88,15 @@ struct fv_trainer {
   bool have_corpus, have_weights;
   unsigned dense_blocks;   // blocks of the absmax launch
   unsigned update_blocks;  // blocks of the dense update launch
+  // one launch for both dense passes (a matrix that fits the machine's registers): blocks, 16-byte
+  // groups per thread (0 = two launches), the arrival word of every block, launches so far, and a
+  // host-visible word a block sets when it gave up waiting for the others
+  unsigned onepass_blocks, onepass_unroll;
+  bool onepass;  // in use (fv_trainer_set_dense_launches)
+  unsigned long long *arrive;
+  uint32_t onepass_epoch;
+  uint32_t onepass_spin_limit;
+  uint32_t *onepass_status;
   float update_cut;  // largest fp32 <= 1e-10
 };
 
@@ -780,6 +789,10 @@ struct fv_dense_args {
   float *scalars;
   uint32_t total4, ldk4, ldk, V, K, w, n_bmax, dense_blocks;
   float eps, prec, update_cut;
+  // single-launch form only
+  unsigned long long *arrive;
+  uint32_t *status;
+  uint32_t epoch, spin_limit;
 };
 
 __device__ __forceinline__ bool fv_is_sentinel(float w) { return __float_as_uint(w) == FV_SENTINEL; }
@@ -903,6 +916,121 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
   }
 }
 
+// Kernels 4 and 5 as ONE launch, for a matrix that fits the register file of the machine: one block
+// per compute unit, every thread keeps its U 16-byte groups of W in registers from the maximum pass
+// to the update, so W is read once and written once in a step. Between the passes every block
+// publishes its maximum of |ds| as (launch number, value) in one 64-bit word and one wave of it
+// reads the words of all blocks until each carries this launch's number; the values it read are the
+// maxima, no second look-up follows. The wait is bounded: a block that does not see the others
+// within spin_limit rounds (they are not resident together: the launch was given fewer compute
+// units than it was sized for) marks its word as abandoned, so that blocks arriving later give up
+// as well, sets the status word and leaves its part of W as it is.
+#ifndef FV_ONEPASS_THREADS
+#define FV_ONEPASS_THREADS 1024
+#endif
+#define FV_ONEPASS_BLOCKS_PER_CU (1024 / FV_ONEPASS_THREADS)
+#define FV_ONEPASS_MAX_UNROLL 16
+#define FV_ONEPASS_SPIN_LIMIT (1u << 14)  // rounds of a few microseconds each: tens of milliseconds
+#define FV_ONEPASS_ABANDONED 0xffffffffu  // in place of a block's maximum (no maximum is a NaN): it gave up
+
+template <int U>
+__global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv_dense_args a) {
+  extern __shared__ float4 xs4[];
+  __shared__ float smem16[16];
+  __shared__ float sh_s;
+  __shared__ uint32_t sh_ok;
+  constexpr uint32_t T = FV_ONEPASS_THREADS;
+  const uint32_t stride = gridDim.x * T;
+  const uint32_t p4 = blockIdx.x * T + threadIdx.x;
+  const uint32_t dq = stride % a.ldk4;
+  const uint32_t q0 = p4 % a.ldk4;
+  float4 w[U];
+  fv_dense_load(a, p4, stride, w);
+  // after one launch has given up, the launches already enqueued behind it do not wait at all
+  const uint32_t limit = a.scalars[1] != 0.0f ? 0u : a.spin_limit;
+  for (uint32_t i = threadIdx.x; i < a.ldk4; i += T) xs4[i] = ((const float4 *)a.xx)[i];
+  // the sparse launch has finished: its block maxima go into this block's value
+  float m = 0.0f;
+  for (uint32_t i = a.dense_blocks + threadIdx.x; i < a.n_bmax; i += T) m = fmaxf(m, a.bmax[i]);
+  __syncthreads();
+  uint32_t q = q0;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (p4 + u * stride < a.total4) {
+      const float4 x = xs4[q];
+      m = fv_absmax_keep(m, fv_dense_ds(x.x, w[u].x));
+      m = fv_absmax_keep(m, fv_dense_ds(x.y, w[u].y));
+      m = fv_absmax_keep(m, fv_dense_ds(x.z, w[u].z));
+      m = fv_absmax_keep(m, fv_dense_ds(x.w, w[u].w));
+    }
+    q += dq;
+    if (q >= a.ldk4) q -= a.ldk4;
+  }
+  const float bm = fv_block_max_nonneg(m, smem16);
+  if (threadIdx.x == 0)
+    __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | __float_as_uint(bm),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x < 64) {
+    uint32_t mx = 0;
+    bool done = false, abandoned = false;
+    for (uint32_t spin = 0; spin < limit && !done && !abandoned; ++spin) {
+      bool ok = true, bad = false;
+      mx = 0;
+      for (uint32_t i = threadIdx.x; i < gridDim.x; i += 64) {
+        const unsigned long long v = __hip_atomic_load(&a.arrive[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = ok && (uint32_t)(v >> 32) == a.epoch;
+        bad = bad || ((uint32_t)(v >> 32) == a.epoch && (uint32_t)v == FV_ONEPASS_ABANDONED);
+        mx = max(mx, (uint32_t)v);  // non-negative floats order like their bit patterns
+      }
+      abandoned = __any(bad);
+      done = !abandoned && __all(ok);
+      if (!done && !abandoned) __builtin_amdgcn_s_sleep(2);
+    }
+    mx = fv_wave_max_u32(mx);
+    if (threadIdx.x == 0) {
+      const float nc = __uint_as_float(mx);
+      sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
+      sh_ok = done;
+      if (!done) {
+        // blocks that arrive later must not update either
+        __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | FV_ONEPASS_ABANDONED,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *a.status = 1u;
+        a.scalars[0] = __uint_as_float(0x7fc00000u);  // tells the slot kernel to put the saved weights back
+        a.scalars[1] = 1.0f;
+      } else if (blockIdx.x == 0) {
+        a.scalars[0] = nc;
+      }
+    }
+  }
+  __syncthreads();
+  if (!sh_ok) return;
+  const float s = sh_s;
+  q = q0;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (p4 + u * stride < a.total4) fv_update_four(a, p4 + u * stride, w[u], xs4[q], s);
+    q += dq;
+    if (q >= a.ldk4) q -= a.ldk4;
+  }
+}
+
+template <int U>
+static void fv_launch_onepass(const fv_dense_args &d, unsigned blocks, size_t smem, hipStream_t stream) {
+  hipLaunchKernelGGL(fv_dense_onepass_kernel<U>, dim3(blocks), dim3(FV_ONEPASS_THREADS), smem, stream, d);
+}
+
+template <int U>
+static int fv_onepass_fits(size_t smem) {
+  int nb = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fv_dense_onepass_kernel<U>, FV_ONEPASS_THREADS, smem) !=
+      hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return nb >= FV_ONEPASS_BLOCKS_PER_CU;
+}
+
 // Kernel 6: the final value of every sparse element goes over its sentinel. Runs after the dense
 // update so no dense thread can mistake a finished element for an ordinary weight.
 template <bool DELTA>
@@ -929,7 +1057,7 @@ __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
     for (int u = 0; u < 4; ++u) {
       if (eb + u * 256 >= count) break;
       float out = sl[u].wv;  // a row with xx == 0 is not updated: the saved weight goes back
-      if (x != 0.0f) {
+      if (x != 0.0f && nc == nc) {  // nc is a NaN after a dense pass that gave up: nothing is updated
         const float ds = DELTA ? fv_sparse_ds2(x, sl[u].wv, sl[u].f, sl[u].n, a.delta, n2[u])
                                : fv_sparse_ds(x, sl[u].wv, sl[u].f, sl[u].n);
         const float d = __fmul_rn(s, ds);
@@ -1002,6 +1130,19 @@ static void fv_trainer_free_corpus(fv_trainer *t) {
   t->have_corpus = false;
 }
 
+// Waits for the trainer's stream; reports a single-launch dense pass that gave up waiting for its
+// other blocks (the step it belonged to did not update the matrix).
+static int fv_trainer_wait(fv_trainer *t) {
+  FV_HIP(hipStreamSynchronize(t->stream));
+  if (t->onepass_status && *(volatile uint32_t *)t->onepass_status) {
+    *t->onepass_status = 0;
+    t->onepass = false;  // later steps take two launches
+    return fv_fail(FV_ERR_STATE, "a single-launch dense pass gave up waiting for its blocks (not resident together): "
+                                 "that step did not update the matrix; later steps use two launches");
+  }
+  return FV_OK;
+}
+
 extern "C" int fv_trainer_destroy(fv_trainer *t) {
   if (!t) return FV_OK;
   if (t->stream) (void)hipStreamSynchronize(t->stream);
@@ -1020,6 +1161,8 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   (void)hipFree(t->sc);
   (void)hipFree(t->xx);
   (void)hipFree(t->scalars);
+  (void)hipFree(t->arrive);
+  if (t->onepass_status) (void)hipHostFree(t->onepass_status);
   if (t->stream) (void)hipStreamDestroy(t->stream);
   delete t;
   return FV_OK;
@@ -1047,8 +1190,33 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMemsetAsync(t->Wt, 0, elems * sizeof(float), t->stream));
   FV_HIP(hipMemsetAsync(t->xx, 0, (size_t)t->ldk * sizeof(float), t->stream));
   FV_HIP(hipMemsetAsync(t->scalars, 0, 16 * sizeof(float), t->stream));
+  if (t->onepass_unroll) {
+    FV_HIP(hipMalloc((void **)&t->arrive, (size_t)t->onepass_blocks * sizeof(unsigned long long)));
+    FV_HIP(hipMemsetAsync(t->arrive, 0, (size_t)t->onepass_blocks * sizeof(unsigned long long), t->stream));
+    FV_HIP(hipHostMalloc((void **)&t->onepass_status, sizeof(uint32_t), hipHostMallocDefault));
+    *t->onepass_status = 0;
+  }
   FV_HIP(hipStreamSynchronize(t->stream));
   return FV_OK;
+}
+
+// One launch for both dense passes when every compute unit can hold a block whose threads keep the
+// whole matrix in registers between them; otherwise (onepass_unroll = 0) the two launches.
+static void fv_choose_onepass(fv_trainer *t, uint64_t cu) {
+  t->onepass_blocks = t->onepass_unroll = 0;
+  t->onepass_spin_limit = FV_ONEPASS_SPIN_LIMIT;
+  uint64_t blocks = ((uint64_t)t->total4 + FV_ONEPASS_THREADS - 1) / FV_ONEPASS_THREADS;
+  if (blocks > cu * FV_ONEPASS_BLOCKS_PER_CU) blocks = cu * FV_ONEPASS_BLOCKS_PER_CU;
+  const uint64_t need = ((uint64_t)t->total4 + blocks * FV_ONEPASS_THREADS - 1) / (blocks * FV_ONEPASS_THREADS);
+  if (need > FV_ONEPASS_MAX_UNROLL) return;
+  const unsigned unroll = need <= 4 ? 4 : need <= 8 ? 8 : need <= 12 ? 12 : 16;
+  const size_t smem = (size_t)t->ldk * sizeof(float);
+  const int fits = unroll == 4 ? fv_onepass_fits<4>(smem) : unroll == 8 ? fv_onepass_fits<8>(smem)
+                 : unroll == 12 ? fv_onepass_fits<12>(smem) : fv_onepass_fits<16>(smem);
+  if (!fits) return;
+  t->onepass_blocks = (unsigned)blocks;
+  t->onepass_unroll = unroll;
+  t->onepass = true;
 }
 
 extern "C" int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_trainer) {
@@ -1095,6 +1263,7 @@ extern "C" int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_tr
     const uint64_t cu = (uint64_t)(cus > 0 ? cus : 256);
     t->dense_blocks = (unsigned)(want < cu * FV_ABSMAX_BLOCKS_PER_CU ? want : cu * FV_ABSMAX_BLOCKS_PER_CU);
     t->update_blocks = (unsigned)(want < cu * FV_UPDATE_BLOCKS_PER_CU ? want : cu * FV_UPDATE_BLOCKS_PER_CU);
+    fv_choose_onepass(t, cu);
     rc = fv_trainer_alloc(t);
   }
   if (rc != FV_OK) {
@@ -1205,6 +1374,7 @@ extern "C" int fv_trainer_set_weights(fv_trainer *t, const float *W) {
 extern "C" int fv_trainer_get_weights(fv_trainer *t, float *out_W) {
   FV_REQUIRE(t && out_W, FV_ERR_INVALID, "null argument");
   FV_REQUIRE(t->have_weights, FV_ERR_STATE, "no weights set");
+  FV_TRY(fv_trainer_wait(t));
   return fv_download_weights(t->Wt, out_W, t->K, t->N, t->ldk, t->stream);
 }
 
@@ -1407,6 +1577,9 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.slot_n2 = t->slot_n2;
   d.delta = delta;
   d.w = t->w;
+  d.arrive = nullptr;
+  d.status = nullptr;
+  d.epoch = d.spin_limit = 0;
   d.slot_stride = (uint64_t)t->B * t->w * (anti ? 2 : 1);
   d.bmax = t->bmax;
   d.scalars = t->scalars;
@@ -1421,10 +1594,28 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.prec = t->cfg.prec;
   d.update_cut = t->update_cut;
   const size_t smem = (size_t)t->ldk * sizeof(float);
-  if (which & 8u)
-    hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
-  if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
-  if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
+  if (t->onepass) {
+    // both dense passes in the launch that takes the place of the first one
+    if (which & 8u) {
+      if (++t->onepass_epoch == 0) t->onepass_epoch = 1;
+      d.arrive = t->arrive;
+      d.status = t->onepass_status;
+      d.epoch = t->onepass_epoch;
+      d.spin_limit = t->onepass_spin_limit;
+      switch (t->onepass_unroll) {
+        case 4: fv_launch_onepass<4>(d, t->onepass_blocks, smem, t->stream); break;
+        case 8: fv_launch_onepass<8>(d, t->onepass_blocks, smem, t->stream); break;
+        case 12: fv_launch_onepass<12>(d, t->onepass_blocks, smem, t->stream); break;
+        default: fv_launch_onepass<16>(d, t->onepass_blocks, smem, t->stream); break;
+      }
+    }
+    if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
+  } else {
+    if (which & 8u)
+      hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
+    if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
+    if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
+  }
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
   if (which & 32u) {
     if (anti)
@@ -1500,14 +1691,35 @@ extern "C" int fv_trainer_run_epoch(fv_trainer *t, uint64_t epoch_id, uint64_t n
     const uint64_t n = t->n_windows - k < t->B ? t->n_windows - k : t->B;
     FV_TRY(fv_enqueue_step(t, k, (uint32_t)n, eps, delta, nullptr));
   }
-  FV_HIP(hipStreamSynchronize(t->stream));
+  return fv_trainer_wait(t);
+}
+
+extern "C" int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches) {
+  FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
+  FV_REQUIRE(launches <= 2, FV_ERR_INVALID, "launches must be 0 (choose), 1 or 2");
+  FV_REQUIRE(launches != 1 || t->onepass_unroll, FV_ERR_INVALID,
+             "a %llu x %u matrix does not fit the registers of this device: the dense passes need two launches",
+             (unsigned long long)t->N, t->K);
+  t->onepass = launches == 2 ? false : t->onepass_unroll != 0;
+  FV_HIP(hipMemsetAsync(t->scalars + 1, 0, sizeof(float), t->stream));  // "a launch has given up"
+  return FV_OK;
+}
+
+extern "C" int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches) {
+  FV_REQUIRE(t && out_launches, FV_ERR_INVALID, "null argument");
+  *out_launches = t->onepass ? 1u : 2u;
+  return FV_OK;
+}
+
+extern "C" int fv_trainer_set_wait_limit(fv_trainer *t, uint32_t rounds) {
+  FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
+  t->onepass_spin_limit = rounds;
   return FV_OK;
 }
 
 extern "C" int fv_trainer_sync(fv_trainer *t) {
   FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
-  FV_HIP(hipStreamSynchronize(t->stream));
-  return FV_OK;
+  return fv_trainer_wait(t);
 }
 
 extern "C" int fv_trainer_get_winners(fv_trainer *t, int32_t *out_winners, uint32_t capacity) {

@@ -142,6 +142,20 @@ class Trainer:
     def sync(self):
         check(self.lib.fv_trainer_sync(self.handle))
 
+    def set_dense_launches(self, launches):
+        """1: both passes over the matrix in one launch (it must fit the device's registers),
+        2: two launches, 0: as chosen at creation.  Same results either way."""
+        check(self.lib.fv_trainer_set_dense_launches(self.handle, int(launches)))
+
+    @property
+    def dense_launches(self):
+        out = C.c_uint32(0)
+        check(self.lib.fv_trainer_get_dense_launches(self.handle, C.byref(out)))
+        return out.value
+
+    def _set_wait_limit(self, rounds):
+        check(self.lib.fv_trainer_set_wait_limit(self.handle, int(rounds)))
+
     def winners(self, n):
         out = np.empty(int(n), dtype=np.int32)
         check(self.lib.fv_trainer_get_winners(self.handle, ptr(out), len(out)))

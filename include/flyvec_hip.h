@@ -157,7 +157,21 @@ int fv_trainer_run_epoch(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs);
 /* eps of flyvec/src/cuda_funcs.cu:1229 for this trainer's learning rate. */
 int fv_trainer_epoch_eps(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs, float *out_eps);
 
+/* Waits for the trainer's stream. FV_ERR_STATE if a single-launch dense pass (below) gave up
+ * waiting for its other blocks: the step it belonged to did not update the matrix. */
 int fv_trainer_sync(fv_trainer *t);
+
+/* The two passes over the matrix of a step (max|ds|, flyvec/src/cu_special_reduction.cu:241, and
+ * the update, flyvec/src/cuda_funcs.cu:1787-1806) run as ONE launch that keeps the matrix in
+ * registers between them when it fits the device (64 MiB on 256 compute units), else as two.
+ * launches = 1 or 2 forces the form (1 fails with FV_ERR_INVALID when the matrix does not fit),
+ * 0 returns to the choice made at creation. Results are bit-identical either way. */
+int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches);
+int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches); /* 1 or 2: the form in use */
+/* Test hook: between its two passes a single-launch dense pass waits for all its blocks, at most
+ * `rounds` polling rounds (2^14 by default, tens of milliseconds); 0 makes every block give up at once, which
+ * is how the error path of fv_trainer_sync is exercised. No counterpart in the reference. */
+int fv_trainer_set_wait_limit(fv_trainer *t, uint32_t rounds);
 
 /* Parity hooks on the last step: winner per window (max_IDs[r][0], flyvec/src/cuda_funcs.cu:
  * 1719), per-neuron totals xx (:1721) and max|ds| (flyvec/src/cu_special_reduction.cu:241). */

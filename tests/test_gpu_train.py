@@ -14,9 +14,10 @@ pytestmark = pytest.mark.gpu
 f32 = np.float32
 
 
-def make_trainer(tokens, offsets, V, K, w, B, W0, tie=0, lr0=2e-4, perm_seed=6, prec=1e-30):
+def make_trainer(tokens, offsets, V, K, w, B, W0, tie=0, lr0=2e-4, perm_seed=6, prec=1e-30, launches=0):
     from flyvec_amd import Trainer
     t = Trainer(V, K, w, B, initial_learning_rate=lr0, tie_rule=tie, prec=prec)
+    t.set_dense_launches(launches)  # 0: as chosen at creation, 1 / 2: both passes over W in one launch / in two
     t.set_corpus(tokens, offsets)
     perm = np.random.default_rng(perm_seed).permutation(t.num_windows).astype(np.uint64)
     t.set_permutation(perm)
@@ -29,13 +30,13 @@ def oracle_inputs(to, tokens, offsets, V, w):
 
 
 def run_both(gpu, oracle_lib, V, K, w, B, steps, tie=0, sigma=0.02, n_tokens=60000, W0=None, lr0=2e-4,
-             mean_chunk=25, n_masked=40, seed=0):
+             mean_chunk=25, n_masked=40, seed=0, launches=0):
     from flyvec_amd import synthetic
     to = oracle_lib
     tokens, offsets = small_corpus(n_tokens, V, seed=seed, mean_chunk=mean_chunk, n_masked=n_masked)
     if W0 is None:
         W0 = synthetic.synapses(K, V, seed=5 + seed, sigma=sigma)
-    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, tie=tie, lr0=lr0)
+    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, tie=tie, lr0=lr0, launches=launches)
     starts, invf = oracle_inputs(to, tokens, offsets, V, w)
     assert t.num_windows == len(starts)
     eps = t.epoch_eps(0, 15)
@@ -52,9 +53,10 @@ def run_both(gpu, oracle_lib, V, K, w, B, steps, tie=0, sigma=0.02, n_tokens=600
     return np.concatenate(wins), wo, Wg, Wo
 
 
+@pytest.mark.parametrize("launches", [1, 2])
 @pytest.mark.parametrize("tie", [0, 1])
-def test_small_config_bit_exact(gpu, oracle_lib, tie):
-    wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=500, K=400, w=11, B=512, steps=30, tie=tie)
+def test_small_config_bit_exact(gpu, oracle_lib, tie, launches):
+    wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=500, K=400, w=11, B=512, steps=30, tie=tie, launches=launches)
     assert np.array_equal(wg, wo)
     assert np.array_equal(Wg, Wo)
 
@@ -69,6 +71,85 @@ def test_shapes_bit_exact(gpu, oracle_lib, K, w, V, B):
     wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=V, K=K, w=w, B=B, steps=6, n_tokens=n_tokens, mean_chunk=40)
     assert np.array_equal(wg, wo)
     assert np.array_equal(Wg, Wo)
+
+
+@pytest.mark.parametrize("K,w,V,B", [(1, 1, 5, 1), (65, 15, 200, 256), (1000, 15, 300, 512), (2048, 7, 64, 128),
+                                     (30, 11, 30000, 700), (200, 11, 20000, 2000), (400, 11, 20000, 3000),
+                                     (400, 11, 20970, 3000), (3, 5, 400000, 300)])
+def test_shapes_bit_exact_with_two_dense_launches(gpu, oracle_lib, K, w, V, B):
+    # the shapes above take the single launch wherever the matrix fits the registers of the device;
+    # here the same step with the maximum pass and the update as two launches, on matrices of every
+    # size class of the single launch (4, 8, 12, 16 groups of 16 bytes per thread, and the largest that fits)
+    n_tokens = 40000 if V < 20000 else 120000
+    wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=V, K=K, w=w, B=B, steps=4, n_tokens=n_tokens, mean_chunk=40,
+                              launches=2)
+    assert np.array_equal(wg, wo)
+    assert np.array_equal(Wg, Wo)
+
+
+@pytest.mark.parametrize("K,V", [(200, 20000), (300, 20000), (400, 20000), (400, 20970)])
+def test_single_dense_launch_size_classes(gpu, oracle_lib, K, V):
+    # 32, 48, 64 and 67.1 MB of W: a thread of the single launch keeps 8, 12, 16 and 16 groups
+    wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=V, K=K, w=11, B=3000, steps=4, n_tokens=120000, mean_chunk=40,
+                              launches=1)
+    assert np.array_equal(wg, wo)
+    assert np.array_equal(Wg, Wo)
+
+
+def test_dense_launch_forms(gpu):
+    from flyvec_amd import Trainer, _lib, synthetic
+    V, K, w, B = 300, 64, 7, 128
+    tokens, offsets = small_corpus(20000, V)
+    W0 = synthetic.synapses(K, V)
+    got = {}
+    for launches in (1, 2):
+        t, _ = make_trainer(tokens, offsets, V, K, w, B, W0, launches=launches)
+        assert t.dense_launches == launches
+        for s in range(5):
+            t.step(s * B, B, 1e-3)
+        got[launches] = (t.get_weights(), t.step_stats()[1])
+        t.close()
+    assert np.array_equal(got[1][0], got[2][0]) and got[1][1] == got[2][1]
+    # a matrix beyond the registers of the device: two launches, and one cannot be forced
+    big = Trainer(400000, 64, 5, 32)
+    assert big.dense_launches == 2
+    with pytest.raises(_lib.FlyvecError) as e:
+        big.set_dense_launches(1)
+    assert e.value.code == _lib.FV_ERR_INVALID
+    big.close()
+    with pytest.raises(_lib.FlyvecError):
+        Trainer(V, K, w, B).set_dense_launches(3)
+
+
+def test_single_dense_launch_gives_up_cleanly(gpu, oracle_lib):
+    """The wait between the two passes of the single launch is bounded. With a limit of zero rounds every block
+    gives up at once (all kernels still run to their end): the step leaves W alone, the next synchronisation
+    reports it, and the trainer carries on with two launches."""
+    from flyvec_amd import _lib, synthetic
+    to = oracle_lib
+    V, K, w, B = 300, 64, 7, 128
+    tokens, offsets = small_corpus(20000, V)
+    W0 = synthetic.synapses(K, V)
+    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, launches=1)
+    t._set_wait_limit(0)
+    t.step(0, B, 1e-3)
+    with pytest.raises(_lib.FlyvecError) as e:
+        t.sync()
+    assert e.value.code == _lib.FV_ERR_STATE
+    assert t.dense_launches == 2
+    t.sync()                                   # reported once
+    assert np.array_equal(t.get_weights(), W0)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    for launches in (2, 1):                    # usable afterwards, in either form
+        t._set_wait_limit(1 << 14)
+        t.set_dense_launches(launches)
+        t.set_weights(W0)
+        for s in range(3):
+            t.step(s * B, B, 1e-3)
+        Wo = W0.copy()
+        to.train_steps(Wo, tokens, starts, perm, 0, B, 3, w, invf, 1e-3)
+        assert np.array_equal(t.get_weights(), Wo)
+    t.close()
 
 
 @pytest.mark.parametrize("tie", [0, 1])
