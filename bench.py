@@ -57,8 +57,9 @@ MEASURED_TRAFFIC = {
 }
 
 
-# the two passes over W of a step as one launch: W stays in registers between them, so the launch
-# moves 8*K*N bytes while the byte model of the step counts the two passes' 12*K*N
+# the two passes over W of a step (and the sparse elements' update) as one launch: W stays in
+# registers between them, so the launch moves 8*K*N bytes of W while the byte model of the step
+# counts the two passes' 12*K*N
 DENSE_ONE = "dense_max_update"
 
 
@@ -81,11 +82,12 @@ def hash_bytes_per_window(K, w):
     return 4 * w * K + 4 * w + 8 * ((K + 63) // 64)
 
 
-def bench_train(steps, warmup, cpu_seconds, c=TRAIN):
+def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0):
     from flyvec_amd import Trainer, synthetic
     tokens, offsets = synthetic.corpus(c["n_tokens"], c["V"], s=c["zipf_s"], mean_chunk=c["mean_chunk"])
     W0 = synthetic.synapses(c["K"], c["V"], seed=5)
     t = Trainer(c["V"], c["K"], c["w"], c["B"], initial_learning_rate=c["lr0"], prec=c["prec"])
+    t.set_dense_launches(dense_launches)
     t.set_corpus(tokens, offsets)
     nwin = t.num_windows
     perm = np.random.default_rng(6).permutation(nwin).astype(np.uint64)
@@ -118,9 +120,11 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN):
     N = 2 * c["V"]
     step_bytes, per_kernel = train_bytes(c["K"], N, c["w"], c["B"])
     if launches == 1:
-        # max|ds| and the update ran as one launch (timed under the first name; the second is empty)
-        kern_ms[DENSE_ONE] = kern_ms.pop("absmax_ds") + kern_ms.pop("update")
-        per_kernel[DENSE_ONE] = per_kernel.pop("absmax_ds") + per_kernel.pop("update")
+        # max|ds|, the update and the slot update ran as one launch (timed under the first name;
+        # the others are empty)
+        parts = ("absmax_ds", "update", "slot_update")
+        kern_ms[DENSE_ONE] = sum(kern_ms.pop(k) for k in parts)
+        per_kernel[DENSE_ONE] = sum(per_kernel.pop(k) for k in parts)
     dom = max(kern_ms, key=kern_ms.get)
     achieved = per_kernel[dom] / (kern_ms[dom] * 1e-3)
     ms_per_step = wall / steps * 1e3
@@ -141,7 +145,7 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN):
 
     if dom == DENSE_ONE:
         # what the launch has to move (W read once, written once) and the rate on that count
-        moved = 8 * c["K"] * N
+        moved = 8 * c["K"] * N + 8 * c["B"] * c["w"]
         out["roofline"]["moved_bytes"] = moved
         out["roofline"]["frac_of_moved"] = moved / (kern_ms[dom] * 1e-3) / HBM_PEAK
 
@@ -255,6 +259,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample length (0 = skip)")
     ap.add_argument("--no-hash", action="store_true")
+    ap.add_argument("--dense-launches", type=int, choices=[0, 1, 2], default=0,
+                    help="the passes over W of a step as one launch (1), two (2), or as the library chooses (0)")
     ap.add_argument("--workload", choices=["step", "large-step", "epoch"], default="step",
                     help="step: the headline minibatch step (default); large-step: K=1000, V=50000, w=15, "
                          "B=50000 (400 MB matrix); epoch: one full epoch over 100 M tokens with shuffle and "
@@ -283,7 +289,7 @@ def main():
     c = LARGE if args.workload == "large-step" else TRAIN
     if args.workload == "large-step":
         args.steps, args.warmup, args.no_hash = min(args.steps, 50), min(args.warmup, 5), True
-    tr = bench_train(args.steps, args.warmup, args.cpu_seconds, c)
+    tr = bench_train(args.steps, args.warmup, args.cpu_seconds, c, args.dense_launches)
     line = {
         "metric": f"train windows/s at K={c['K']},Nvoc={c['V'] // 1000}k",
         "value": tr["value"], "unit": "windows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -298,6 +304,7 @@ def main():
         "step_algorithmic_bytes": tr["step_algorithmic_bytes"],
         "event_ms_per_step": tr["event_ms_per_step"],
         "kernel_ms": tr["kernel_ms"],
+        "dense_launches": tr["dense_launches"],
     }
     if "cpu_baseline" in tr:
         line["cpu_baseline"] = tr["cpu_baseline"]

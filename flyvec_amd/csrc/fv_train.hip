@@ -797,22 +797,35 @@ struct fv_dense_args {
 
 __device__ __forceinline__ bool fv_is_sentinel(float w) { return __float_as_uint(w) == FV_SENTINEL; }
 
-__device__ __forceinline__ float fv_dense_ds(float x, float w) {
-  return (x != 0.0f && !fv_is_sentinel(w)) ? __fmul_rn(-x, w) : 0.0f;
+// ds of a dense element is -xx[h] * W (flyvec/src/cuda_funcs.cu:657-672 without the sparse term). No
+// test for a sentinel or for xx == 0 is needed in the two passes: a sentinel is a NaN and so are
+// its products, which neither replace a maximum nor pass the update's comparison, and a row with
+// xx == 0 has ds = 0, which changes nothing either.
+__device__ __forceinline__ float fv_absmax_four(float m, const float4 x, const float4 w) {
+  // |x * w| = |-x * w| bit for bit; fmaxf returns the other operand when one is a NaN
+  m = fmaxf(m, fabsf(__fmul_rn(x.x, w.x)));
+  m = fmaxf(m, fabsf(__fmul_rn(x.y, w.y)));
+  m = fmaxf(m, fabsf(__fmul_rn(x.z, w.z)));
+  return fmaxf(m, fabsf(__fmul_rn(x.w, w.w)));
 }
 
-// W += s * ds on four consecutive dense elements (flyvec/src/cuda_funcs.cu:1800-1803): an element
-// changes only where |s * ds| exceeds the cut; sentinel positions belong to the slot kernel.
-__device__ __forceinline__ void fv_update_four(const fv_dense_args &a, uint32_t p4, float4 w, const float4 x,
-                                               const float s) {
+// W += s * ds on four consecutive elements (flyvec/src/cuda_funcs.cu:1800-1803): an element changes
+// only where |s * ds| exceeds the cut. Returns whether any did.
+__device__ __forceinline__ bool fv_apply_four(float4 &w, const float4 x, const float s, const float cut) {
   bool changed = false;
   float d;
-  d = __fmul_rn(s, fv_dense_ds(x.x, w.x)); if (fabsf(d) > a.update_cut) { w.x = __fadd_rn(w.x, d); changed = true; }
-  d = __fmul_rn(s, fv_dense_ds(x.y, w.y)); if (fabsf(d) > a.update_cut) { w.y = __fadd_rn(w.y, d); changed = true; }
-  d = __fmul_rn(s, fv_dense_ds(x.z, w.z)); if (fabsf(d) > a.update_cut) { w.z = __fadd_rn(w.z, d); changed = true; }
-  d = __fmul_rn(s, fv_dense_ds(x.w, w.w)); if (fabsf(d) > a.update_cut) { w.w = __fadd_rn(w.w, d); changed = true; }
-  // A sentinel has ds = 0 here and goes back as it came: the slot kernel, a later launch, replaces it.
-  if (changed) a.Wt4[p4] = w;
+  d = __fmul_rn(s, __fmul_rn(-x.x, w.x)); if (fabsf(d) > cut) { w.x = __fadd_rn(w.x, d); changed = true; }
+  d = __fmul_rn(s, __fmul_rn(-x.y, w.y)); if (fabsf(d) > cut) { w.y = __fadd_rn(w.y, d); changed = true; }
+  d = __fmul_rn(s, __fmul_rn(-x.z, w.z)); if (fabsf(d) > cut) { w.z = __fadd_rn(w.z, d); changed = true; }
+  d = __fmul_rn(s, __fmul_rn(-x.w, w.w)); if (fabsf(d) > cut) { w.w = __fadd_rn(w.w, d); changed = true; }
+  return changed;
+}
+
+// The update of the two-launch form: a sentinel goes back as it came, the slot kernel, a later
+// launch, replaces it.
+__device__ __forceinline__ void fv_update_four(const fv_dense_args &a, uint32_t p4, float4 w, const float4 x,
+                                               const float s) {
+  if (fv_apply_four(w, x, s, a.update_cut)) a.Wt4[p4] = w;
 }
 
 // 16-byte loads a thread of a dense pass has in flight, and the blocks per compute unit of its launch
@@ -829,12 +842,14 @@ __device__ __forceinline__ void fv_update_four(const fv_dense_args &a, uint32_t 
 #define FV_UPDATE_BLOCKS_PER_CU 8
 #endif
 
-// Batch u of a thread's elements: 16-byte group p4 + u * stride, clamped so that the load is
-// unconditional; a group past the end is loaded but not used.
+// Batch u of a thread's elements: 16-byte group p4 + u * stride. Every load is unconditional; one
+// past the end reads the thread's first group again and is not used (one common address for all
+// of them would queue thousands of wavefronts on a single cache line).
 template <int U>
 __device__ __forceinline__ void fv_dense_load(const fv_dense_args &a, uint32_t p4, uint32_t stride, float4 (&w)[U]) {
+  const uint32_t inside = min(p4, a.total4 - 1);
 #pragma unroll
-  for (int u = 0; u < U; ++u) w[u] = a.Wt4[min(p4 + u * stride, a.total4 - 1)];
+  for (int u = 0; u < U; ++u) w[u] = a.Wt4[p4 + u * stride < a.total4 ? p4 + u * stride : inside];
 }
 
 // Kernel 4: block maxima of |ds| over the dense elements. A thread's first loads of W
@@ -855,11 +870,7 @@ __global__ __launch_bounds__(256) void fv_absmax_kernel(fv_dense_args a) {
 #pragma unroll
     for (int u = 0; u < FV_ABSMAX_UNROLL; ++u) {
       if (p4 + u * stride < a.total4) {
-        const float4 x = xs4[q];
-        m = fv_absmax_keep(m, fv_dense_ds(x.x, w[u].x));
-        m = fv_absmax_keep(m, fv_dense_ds(x.y, w[u].y));
-        m = fv_absmax_keep(m, fv_dense_ds(x.z, w[u].z));
-        m = fv_absmax_keep(m, fv_dense_ds(x.w, w[u].w));
+        m = fv_absmax_four(m, xs4[q], w[u]);
       }
       q += dq;
       if (q >= a.ldk4) q -= a.ldk4;
@@ -916,15 +927,19 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
   }
 }
 
-// Kernels 4 and 5 as ONE launch, for a matrix that fits the register file of the machine: one block
-// per compute unit, every thread keeps its U 16-byte groups of W in registers from the maximum pass
-// to the update, so W is read once and written once in a step. Between the passes every block
-// publishes its maximum of |ds| as (launch number, value) in one 64-bit word and one wave of it
-// reads the words of all blocks until each carries this launch's number; the values it read are the
-// maxima, no second look-up follows. The wait is bounded: a block that does not see the others
-// within spin_limit rounds (they are not resident together: the launch was given fewer compute
-// units than it was sized for) marks its word as abandoned, so that blocks arriving later give up
-// as well, sets the status word and leaves its part of W as it is.
+// Kernels 4, 5 and 6 as ONE launch, for a matrix that fits the register file of the machine: one
+// block per compute unit, every thread keeps its U 16-byte groups of W in registers from the
+// maximum pass to the update, so W is read once and written once in a step. Between the passes
+// every block publishes its maximum of |ds| as (launch number, value) in one 64-bit word and one
+// wave of it reads the words of all blocks until each carries this launch's number; the values it
+// read are the maxima, no second look-up follows. The wait is bounded: a block that does not see
+// the others within spin_limit rounds (they are not resident together: the launch was given fewer
+// compute units than it was sized for) marks its word as abandoned, so that blocks arriving later
+// give up as well, sets the status word and leaves its part of W as it is.
+// No thread reads W after the wait, so the sparse elements are finished here as well: the slot
+// records are dealt evenly over the blocks, a thread fetches its record and forms ds while W is
+// in flight and during the wait, and afterwards writes the element; a dense thread never writes a
+// sentinel's position.
 #ifndef FV_ONEPASS_THREADS
 #define FV_ONEPASS_THREADS 1024
 #endif
@@ -933,35 +948,114 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
 #define FV_ONEPASS_SPIN_LIMIT (1u << 14)  // rounds of a few microseconds each: tens of milliseconds
 #define FV_ONEPASS_ABANDONED 0xffffffffu  // in place of a block's maximum (no maximum is a NaN): it gave up
 
-template <int U>
+// The record number r of the step -> its place in the slot regions and its neuron. seg_end holds the
+// running totals of the record counts of the sparse launch's blocks (block g = neuron g / 4, class g % 4),
+// first_window the first window position of every neuron's part of a slot region.
+__device__ __forceinline__ uint64_t fv_slot_locate(const fv_dense_args &a, const uint32_t *seg_end, uint32_t n_seg,
+                                                   const uint32_t *first_window, uint32_t r, uint32_t *h_out) {
+  uint32_t lo = 0, hi = n_seg - 1;  // the smallest g with seg_end[g] > r
+  while (lo < hi) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (seg_end[mid] > r) hi = mid; else lo = mid + 1;
+  }
+  const uint32_t h = lo >> FV_NB_CLASS_SHIFT, q = lo & (FV_NB_CLASSES - 1);
+  *h_out = h;
+  return (uint64_t)q * a.slot_stride + (uint64_t)first_window[h] * a.w + (r - (lo ? seg_end[lo - 1] : 0u));
+}
+
+// The update of the single launch: a sentinel's position is never written, another thread of the
+// same launch puts the finished sparse element there. A sentinel is a NaN, and no NaN is ever
+// changed by the update, so NaN positions are simply left out of the store.
+__device__ __forceinline__ void fv_update_four_around(const fv_dense_args &a, uint32_t p4, float4 w, const float4 x,
+                                                      const float s) {
+  if (!fv_apply_four(w, x, s, a.update_cut)) return;
+  if (!(__builtin_isunordered(w.x, w.y) || __builtin_isunordered(w.z, w.w))) {
+    a.Wt4[p4] = w;
+    return;
+  }
+  float *e = (float *)&a.Wt4[p4];
+  if (w.x == w.x) e[0] = w.x;
+  if (w.y == w.y) e[1] = w.y;
+  if (w.z == w.z) e[2] = w.z;
+  if (w.w == w.w) e[3] = w.w;
+}
+
+// P: counts of the sparse launch's blocks a thread sums (FV_NB_CLASSES * K <= P * FV_ONEPASS_THREADS)
+template <int U, int P, bool DELTA>
 __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv_dense_args a) {
+  constexpr uint32_t T = FV_ONEPASS_THREADS;
+  // xx (a 16-byte word per thread, ldk floats used), the first window of every neuron's slot
+  // records (two words per thread), the running totals of the record counts
   extern __shared__ float4 xs4[];
+  uint32_t *first_window = (uint32_t *)(xs4 + T);
+  uint32_t *seg_end = first_window + 2 * T;
   __shared__ float smem16[16];
+  __shared__ uint32_t red[17];
   __shared__ float sh_s;
   __shared__ uint32_t sh_ok;
-  constexpr uint32_t T = FV_ONEPASS_THREADS;
+  const uint32_t n_seg = a.K * FV_NB_CLASSES;
   const uint32_t stride = gridDim.x * T;
   const uint32_t p4 = blockIdx.x * T + threadIdx.x;
   const uint32_t dq = stride % a.ldk4;
   const uint32_t q0 = p4 % a.ldk4;
-  float4 w[U];
-  fv_dense_load(a, p4, stride, w);
+  // The small loads first, every one unconditional, then all of this thread's W: loads return in
+  // the order of issue, so what is issued here is used while W is in flight, and nothing that is
+  // issued after W is needed before W has arrived.
+  uint32_t segc[P];
+  float sparse_max[P];  // the sparse launch's block maxima, dealt over the blocks of this one
+#pragma unroll
+  for (int j = 0; j < P; ++j) {
+    segc[j] = a.slot_count[min(threadIdx.x * P + j, n_seg - 1)];
+    sparse_max[j] = a.bmax[a.dense_blocks + min(blockIdx.x + gridDim.x * (threadIdx.x + T * j), n_seg - 1)];
+  }
+  const float4 x_stage = ((const float4 *)a.xx)[min(threadIdx.x, a.ldk4 - 1)];
+  uint32_t fw[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t h = min(threadIdx.x + T * j, a.K - 1);
+    fw[j] = a.group_base[h] + (DELTA ? a.group_base2[h] : 0u);
+  }
   // after one launch has given up, the launches already enqueued behind it do not wait at all
   const uint32_t limit = a.scalars[1] != 0.0f ? 0u : a.spin_limit;
-  for (uint32_t i = threadIdx.x; i < a.ldk4; i += T) xs4[i] = ((const float4 *)a.xx)[i];
-  // the sparse launch has finished: its block maxima go into this block's value
+  float4 w[U];
+  __builtin_amdgcn_sched_barrier(0);  // nothing that uses a small load moves up between the loads of W
+  fv_dense_load(a, p4, stride, w);
+  __builtin_amdgcn_sched_barrier(0);
+
+  xs4[threadIdx.x] = x_stage;
+  first_window[threadIdx.x] = fw[0];
+  first_window[threadIdx.x + T] = fw[1];
+  uint32_t mine = 0;
   float m = 0.0f;
-  for (uint32_t i = a.dense_blocks + threadIdx.x; i < a.n_bmax; i += T) m = fmaxf(m, a.bmax[i]);
+#pragma unroll
+  for (int j = 0; j < P; ++j) {
+    if (threadIdx.x * P + j >= n_seg) segc[j] = 0;
+    mine += segc[j];
+    m = fmaxf(m, sparse_max[j]);  // an index past the end repeats the last maximum
+  }
+  uint32_t n_records;
+  uint32_t run = fv_block_scan_total(mine, red, &n_records);
+#pragma unroll
+  for (int j = 0; j < P; ++j) {
+    run += segc[j];
+    if (threadIdx.x * P + j < n_seg) seg_end[threadIdx.x * P + j] = run;
+  }
   __syncthreads();
+  // this block's share of the records; a thread's first one is fetched now, behind W
+  const uint32_t r_lo = (uint32_t)((uint64_t)n_records * blockIdx.x / gridDim.x);
+  const uint32_t r_hi = (uint32_t)((uint64_t)n_records * (blockIdx.x + 1) / gridDim.x);
+  const uint32_t r0 = r_lo + threadIdx.x;
+  const bool live0 = r0 < r_hi;
+  uint32_t h0 = 0;
+  uint64_t at0 = 0;  // a thread without a record reads the first one of the buffer and does not use it
+  if (live0) at0 = fv_slot_locate(a, seg_end, n_seg, first_window, r0, &h0);
+  const fv_slot sl0 = a.slots[at0];
+  const uint32_t n20 = DELTA ? a.slot_n2[at0] : 0u;
   uint32_t q = q0;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (p4 + u * stride < a.total4) {
-      const float4 x = xs4[q];
-      m = fv_absmax_keep(m, fv_dense_ds(x.x, w[u].x));
-      m = fv_absmax_keep(m, fv_dense_ds(x.y, w[u].y));
-      m = fv_absmax_keep(m, fv_dense_ds(x.z, w[u].z));
-      m = fv_absmax_keep(m, fv_dense_ds(x.w, w[u].w));
+      m = fv_absmax_four(m, xs4[q], w[u]);
     }
     q += dq;
     if (q >= a.ldk4) q -= a.ldk4;
@@ -996,39 +1090,74 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
         __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | FV_ONEPASS_ABANDONED,
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         *a.status = 1u;
-        a.scalars[0] = __uint_as_float(0x7fc00000u);  // tells the slot kernel to put the saved weights back
+        a.scalars[0] = __uint_as_float(0x7fc00000u);
         a.scalars[1] = 1.0f;
       } else if (blockIdx.x == 0) {
         a.scalars[0] = nc;
       }
     }
   }
+  // ds of the first record does not depend on the scale: formed while the first wave waits
+  // (every thread takes this path, with no additions where it has no record: the fetch is then
+  // complete in every thread before the stores below)
+  const float *xs = (const float *)xs4;
+  const float x0 = xs[h0];
+  const bool update0 = live0 && x0 != 0.0f;
+  const float ds0 = DELTA ? fv_sparse_ds2(x0, sl0.wv, sl0.f, update0 ? sl0.n : 0u, a.delta, update0 ? n20 : 0u)
+                          : fv_sparse_ds(x0, sl0.wv, sl0.f, update0 ? sl0.n : 0u);
   __syncthreads();
-  if (!sh_ok) return;
+  const bool ok = sh_ok != 0;
   const float s = sh_s;
-  q = q0;
+  if (ok) {
+    q = q0;
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    if (p4 + u * stride < a.total4) fv_update_four(a, p4 + u * stride, w[u], xs4[q], s);
-    q += dq;
-    if (q >= a.ldk4) q -= a.ldk4;
+    for (int u = 0; u < U; ++u) {
+      if (p4 + u * stride < a.total4) fv_update_four_around(a, p4 + u * stride, w[u], xs4[q], s);
+      q += dq;
+      if (q >= a.ldk4) q -= a.ldk4;
+    }
+  }
+  // the sparse elements: the saved weight goes back where the row is not updated (xx == 0) or the
+  // launch gave up, else the updated one
+  if (live0) {
+    float out = sl0.wv;
+    if (ok && x0 != 0.0f) {
+      const float d = __fmul_rn(s, ds0);
+      if (fabsf(d) > a.update_cut) out = __fadd_rn(sl0.wv, d);
+    }
+    ((float *)a.Wt4)[sl0.p] = out;
+  }
+  for (uint32_t r = r0 + T; r < r_hi; r += T) {  // more records than threads: fetched only now
+    uint32_t h;
+    const uint64_t at = fv_slot_locate(a, seg_end, n_seg, first_window, r, &h);
+    const fv_slot sl = a.slots[at];
+    float out = sl.wv;
+    if (ok && xs[h] != 0.0f) {
+      const float ds = DELTA ? fv_sparse_ds2(xs[h], sl.wv, sl.f, sl.n, a.delta, a.slot_n2[at])
+                             : fv_sparse_ds(xs[h], sl.wv, sl.f, sl.n);
+      const float d = __fmul_rn(s, ds);
+      if (fabsf(d) > a.update_cut) out = __fadd_rn(sl.wv, d);
+    }
+    ((float *)a.Wt4)[sl.p] = out;
   }
 }
 
-template <int U>
+template <int U, int P, bool DELTA>
 static void fv_launch_onepass(const fv_dense_args &d, unsigned blocks, size_t smem, hipStream_t stream) {
-  hipLaunchKernelGGL(fv_dense_onepass_kernel<U>, dim3(blocks), dim3(FV_ONEPASS_THREADS), smem, stream, d);
+  hipLaunchKernelGGL((fv_dense_onepass_kernel<U, P, DELTA>), dim3(blocks), dim3(FV_ONEPASS_THREADS), smem, stream, d);
 }
 
-template <int U>
+template <int U, int P>
 static int fv_onepass_fits(size_t smem) {
-  int nb = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fv_dense_onepass_kernel<U>, FV_ONEPASS_THREADS, smem) !=
-      hipSuccess) {
+  int nb = 0, nb2 = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fv_dense_onepass_kernel<U, P, false>, FV_ONEPASS_THREADS,
+                                                   smem) != hipSuccess ||
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb2, fv_dense_onepass_kernel<U, P, true>, FV_ONEPASS_THREADS,
+                                                   smem) != hipSuccess) {
     (void)hipGetLastError();
     return 0;
   }
-  return nb >= FV_ONEPASS_BLOCKS_PER_CU;
+  return nb >= FV_ONEPASS_BLOCKS_PER_CU && nb2 >= FV_ONEPASS_BLOCKS_PER_CU;
 }
 
 // Kernel 6: the final value of every sparse element goes over its sentinel. Runs after the dense
@@ -1057,7 +1186,7 @@ __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
     for (int u = 0; u < 4; ++u) {
       if (eb + u * 256 >= count) break;
       float out = sl[u].wv;  // a row with xx == 0 is not updated: the saved weight goes back
-      if (x != 0.0f && nc == nc) {  // nc is a NaN after a dense pass that gave up: nothing is updated
+      if (x != 0.0f) {
         const float ds = DELTA ? fv_sparse_ds2(x, sl[u].wv, sl[u].f, sl[u].n, a.delta, n2[u])
                                : fv_sparse_ds(x, sl[u].wv, sl[u].f, sl[u].n);
         const float d = __fmul_rn(s, ds);
@@ -1202,6 +1331,12 @@ static int fv_trainer_alloc(fv_trainer *t) {
 
 // One launch for both dense passes when every compute unit can hold a block whose threads keep the
 // whole matrix in registers between them; otherwise (onepass_unroll = 0) the two launches.
+// a 16-byte word and two 4-byte words per thread, then one running total per block of the sparse launch
+static size_t fv_onepass_smem(const fv_trainer *t) {
+  return (size_t)FV_ONEPASS_THREADS * (sizeof(float4) + 2 * sizeof(uint32_t)) +
+         (size_t)t->K * FV_NB_CLASSES * sizeof(uint32_t);
+}
+
 static void fv_choose_onepass(fv_trainer *t, uint64_t cu) {
   t->onepass_blocks = t->onepass_unroll = 0;
   t->onepass_spin_limit = FV_ONEPASS_SPIN_LIMIT;
@@ -1209,10 +1344,11 @@ static void fv_choose_onepass(fv_trainer *t, uint64_t cu) {
   if (blocks > cu * FV_ONEPASS_BLOCKS_PER_CU) blocks = cu * FV_ONEPASS_BLOCKS_PER_CU;
   const uint64_t need = ((uint64_t)t->total4 + blocks * FV_ONEPASS_THREADS - 1) / (blocks * FV_ONEPASS_THREADS);
   if (need > FV_ONEPASS_MAX_UNROLL) return;
-  const unsigned unroll = need <= 4 ? 4 : need <= 8 ? 8 : need <= 12 ? 12 : 16;
-  const size_t smem = (size_t)t->ldk * sizeof(float);
-  const int fits = unroll == 4 ? fv_onepass_fits<4>(smem) : unroll == 8 ? fv_onepass_fits<8>(smem)
-                 : unroll == 12 ? fv_onepass_fits<12>(smem) : fv_onepass_fits<16>(smem);
+  const unsigned unroll = need <= 8 ? 8 : 16;
+  const size_t smem = fv_onepass_smem(t);
+  const bool narrow = (uint64_t)t->K * FV_NB_CLASSES <= 2 * FV_ONEPASS_THREADS;
+  const int fits = unroll == 8 ? (narrow ? fv_onepass_fits<8, 2>(smem) : fv_onepass_fits<8, 8>(smem))
+                               : (narrow ? fv_onepass_fits<16, 2>(smem) : fv_onepass_fits<16, 8>(smem));
   if (!fits) return;
   t->onepass_blocks = (unsigned)blocks;
   t->onepass_unroll = unroll;
@@ -1602,12 +1738,17 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
       d.status = t->onepass_status;
       d.epoch = t->onepass_epoch;
       d.spin_limit = t->onepass_spin_limit;
-      switch (t->onepass_unroll) {
-        case 4: fv_launch_onepass<4>(d, t->onepass_blocks, smem, t->stream); break;
-        case 8: fv_launch_onepass<8>(d, t->onepass_blocks, smem, t->stream); break;
-        case 12: fv_launch_onepass<12>(d, t->onepass_blocks, smem, t->stream); break;
-        default: fv_launch_onepass<16>(d, t->onepass_blocks, smem, t->stream); break;
+      const bool narrow = (uint64_t)t->K * FV_NB_CLASSES <= 2 * FV_ONEPASS_THREADS;
+      const size_t smem1 = fv_onepass_smem(t);
+#define FV_CASE(U, P)                                                                     \
+  if (anti) fv_launch_onepass<U, P, true>(d, t->onepass_blocks, smem1, t->stream);        \
+  else fv_launch_onepass<U, P, false>(d, t->onepass_blocks, smem1, t->stream);
+      if (t->onepass_unroll == 8) {
+        if (narrow) { FV_CASE(8, 2) } else { FV_CASE(8, 8) }
+      } else {
+        if (narrow) { FV_CASE(16, 2) } else { FV_CASE(16, 8) }
       }
+#undef FV_CASE
     }
     if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
   } else {
@@ -1617,7 +1758,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
     if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
   }
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
-  if (which & 32u) {
+  if ((which & 32u) && !t->onepass) {  // the single launch has finished the sparse elements as well
     if (anti)
       hipLaunchKernelGGL(fv_slot_update_kernel<true>, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, d);
     else

@@ -206,16 +206,21 @@ def test_minibatch_larger_than_the_match_masks(gpu, oracle_lib):
     assert np.array_equal(Wg, Wo)
 
 
-def test_timing_hooks(gpu):
+@pytest.mark.parametrize("launches", [1, 2])
+def test_timing_hooks(gpu, launches):
     from flyvec_amd import _lib, synthetic
     V, K, w, B = 300, 64, 11, 256
     tokens, offsets = small_corpus(20000, V)
-    t, _ = make_trainer(tokens, offsets, V, K, w, B, synthetic.synapses(K, V, sigma=0.02))
+    t, _ = make_trainer(tokens, offsets, V, K, w, B, synthetic.synapses(K, V, sigma=0.02), launches=launches)
     t.step(0, B, 1e-3)
+    # as one launch the max pass, the update and the slot update are timed under the first of their names
+    empty = {"update", "slot_update"} if launches == 1 else set()
     total, per = t.time_steps(B, 3, 1e-3)
-    assert total > 0 and set(per) == set(_lib.TRAIN_KERNEL_NAMES) and all(v > 0 for v in per.values())
+    assert total > 0 and set(per) == set(_lib.TRAIN_KERNEL_NAMES)
+    assert all(v > 0 for k, v in per.items() if k not in empty) and all(v >= 0 for v in per.values())
     single = t.time_kernels(reps=3)
-    assert set(single) == set(_lib.TRAIN_KERNEL_NAMES) and all(v > 0 for v in single.values())
+    assert set(single) == set(_lib.TRAIN_KERNEL_NAMES)
+    assert all(v > 0 for k, v in single.items() if k not in empty) and all(v >= 0 for v in single.values())
     assert _lib.calibration_copy(1 << 20, 3) > 0
     t.close()
 
