@@ -186,7 +186,9 @@ int fv_trainer_row_norms(fv_trainer *t, uint32_t n_rows, double *out_norms);
  * events on the trainer's stream. out_total_ms covers all steps; out_kernel_ms[FV_TRAIN_KERNELS]
  * (nullable) receives the mean duration of each kernel of the step, measured in a second,
  * separately instrumented run of the same steps. */
-#define FV_TRAIN_KERNELS 6 /* gather+winner, group by winner + xx, sparse owners, max|ds|, update, sparse update */
+#define FV_TRAIN_KERNELS 6 /* gather+winner, group by winner + xx, sparse owners, max|ds|, update, sparse update;
+                              as a single dense launch (fv_trainer_set_dense_launches) the last three are
+                              one kernel, timed under the first of them, and the other two read ~0 */
 int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint32_t n_steps, float eps,
                           float *out_total_ms, float *out_kernel_ms);
 
