@@ -945,6 +945,11 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
 #endif
 #define FV_ONEPASS_BLOCKS_PER_CU (1024 / FV_ONEPASS_THREADS)
 #define FV_ONEPASS_MAX_UNROLL 16
+// 16-byte loads of W a thread has in flight at a time: with all 16 issued at once the first pass
+// took 2 us longer (10 or 12 in flight measured best; 8 and 14 lie between)
+#ifndef FV_ONEPASS_DEPTH
+#define FV_ONEPASS_DEPTH 12
+#endif
 #define FV_ONEPASS_SPIN_LIMIT (1u << 14)  // rounds of a few microseconds each: tens of milliseconds
 #define FV_ONEPASS_ABANDONED 0xffffffffu  // in place of a block's maximum (no maximum is a NaN): it gave up
 
@@ -1019,7 +1024,10 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   const uint32_t limit = a.scalars[1] != 0.0f ? 0u : a.spin_limit;
   float4 w[U];
   __builtin_amdgcn_sched_barrier(0);  // nothing that uses a small load moves up between the loads of W
-  fv_dense_load(a, p4, stride, w);
+  const uint32_t inside = min(p4, a.total4 - 1);  // read again, and not used, by a load past the end
+#pragma unroll
+  for (int u = 0; u < (FV_ONEPASS_DEPTH < U ? FV_ONEPASS_DEPTH : U); ++u)
+    w[u] = a.Wt4[p4 + u * stride < a.total4 ? p4 + u * stride : inside];
   __builtin_amdgcn_sched_barrier(0);
 
   xs4[threadIdx.x] = x_stage;
@@ -1056,6 +1064,10 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   for (int u = 0; u < U; ++u) {
     if (p4 + u * stride < a.total4) {
       m = fv_absmax_four(m, xs4[q], w[u]);
+    }
+    if (u + FV_ONEPASS_DEPTH < U) {  // the next load takes the place of the one just used
+      const uint32_t p = p4 + (u + FV_ONEPASS_DEPTH) * stride;
+      w[u + FV_ONEPASS_DEPTH] = a.Wt4[p < a.total4 ? p : inside];
     }
     q += dq;
     if (q >= a.ldk4) q -= a.ldk4;
