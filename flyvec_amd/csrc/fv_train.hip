@@ -1072,10 +1072,19 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
     q += dq;
     if (q >= a.ldk4) q -= a.ldk4;
   }
-  const float bm = fv_block_max_nonneg(m, smem16);
-  if (threadIdx.x == 0)
-    __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | __float_as_uint(bm),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // the block's maximum, needed by its first wave only: one barrier
+  {
+    const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
+    if ((threadIdx.x & 63) == 0) smem16[threadIdx.x >> 6] = __uint_as_float(wm);
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    float bm = threadIdx.x < T / 64 ? smem16[threadIdx.x] : 0.0f;
+    bm = __uint_as_float(fv_wave_max_u32(__float_as_uint(bm)));
+    if (threadIdx.x == 0)
+      __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | __float_as_uint(bm),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   if (threadIdx.x < 64) {
     uint32_t mx = 0;
     bool done = false, abandoned = false;
