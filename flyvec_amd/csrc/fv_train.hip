@@ -62,6 +62,13 @@ struct fv_trainer {
   uint64_t n_windows;
   float *invf;
   int32_t *idx;     // B x w column indices of the current minibatch
+  // the single dense launch samples the column indices of the minibatch expected next (the windows
+  // that follow, a full batch or what is left) into idx_ahead while it waits between its passes;
+  // a step that finds its own windows there swaps the buffers and skips the sampler's look-ups
+  int32_t *idx_ahead;
+  bool ahead_valid;
+  uint64_t ahead_first;
+  uint32_t ahead_n;
   int32_t *win;     // B winners
   uint16_t *win16;  // the same, 16 bits each (padded by 64)
   // anti-Hebbian form (delta != 0), allocated with the first such step: the second neuron of every
@@ -117,6 +124,7 @@ struct fv_gather_args {
   float *sc2;
   uint64_t first;
   uint32_t n, K, ldk, w, V, tie_rule;
+  uint32_t sampled;  // idx already holds this minibatch
 };
 
 // FV_GATHER_WINDOWS windows per wavefront, one after the other: the grid then fits the machine in
@@ -128,6 +136,12 @@ struct fv_gather_args {
 
 template <int NV, bool DELTA>
 __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, uint32_t r, int32_t idx, int lane);
+
+// Column index of position c of a window from its token: a masked token stays -1, the centre token
+// addresses the target block (flyvec/src/cuda_funcs.cu:915-936).
+__device__ __forceinline__ int32_t fv_column_index(int32_t tok, uint32_t c, uint32_t w, uint32_t V) {
+  return tok < 0 ? -1 : (c == w / 2 ? tok + (int32_t)V : tok);
+}
 
 // DELTA: also the window's second neuron (flyvec/src/cuda_funcs.cu:495-548 with num_m = 2), which
 // receives the anti-Hebbian terms.
@@ -145,10 +159,13 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
     const uint32_t r = g + k * per;
     idx[k] = -1;
     if (lane < (int)a.w && r < a.n) {
-      const uint64_t s = a.pstart[a.first + r];
-      const int32_t tok = a.corpus[s + lane];
-      idx[k] = tok < 0 ? -1 : (lane == (int)(a.w / 2) ? tok + (int32_t)a.V : tok);
-      a.idx[(uint64_t)r * a.w + lane] = idx[k];
+      if (a.sampled) {
+        idx[k] = a.idx[(uint64_t)r * a.w + lane];
+      } else {
+        const uint64_t s = a.pstart[a.first + r];
+        idx[k] = fv_column_index(a.corpus[s + lane], (uint32_t)lane, a.w, a.V);
+        a.idx[(uint64_t)r * a.w + lane] = idx[k];
+      }
     }
   }
 #pragma unroll
@@ -793,6 +810,12 @@ struct fv_dense_args {
   unsigned long long *arrive;
   uint32_t *status;
   uint32_t epoch, spin_limit;
+  // the minibatch sampled ahead (ahead_n = 0: none)
+  const int32_t *corpus;
+  const uint64_t *pstart;
+  int32_t *idx_ahead;
+  uint64_t ahead_first;
+  uint32_t ahead_n;
 };
 
 __device__ __forceinline__ bool fv_is_sentinel(float w) { return __float_as_uint(w) == FV_SENTINEL; }
@@ -1059,6 +1082,13 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   if (live0) at0 = fv_slot_locate(a, seg_end, n_seg, first_window, r0, &h0);
   const fv_slot sl0 = a.slots[at0];
   const uint32_t n20 = DELTA ? a.slot_n2[at0] : 0u;
+  // the next minibatch's column indices, by all waves but the first: the window's start now
+  constexpr uint32_t TS = T - 64;
+  const uint32_t ahead_entries = a.ahead_n * a.w;
+  const uint32_t e0 = blockIdx.x * TS + (threadIdx.x - 64);
+  const bool samples0 = threadIdx.x >= 64 && e0 < ahead_entries;
+  const uint32_t er0 = samples0 ? e0 / a.w : 0u;
+  const uint64_t start0 = a.ahead_n ? a.pstart[a.ahead_first + er0] : 0ull;
   uint32_t q = q0;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -1118,6 +1148,17 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
       }
     }
   }
+  // the token of the sampled position while the first wave waits; then, for a minibatch with more
+  // positions than the launch has sampling threads, the rest
+  if (samples0) {
+    const uint32_t c = e0 - er0 * a.w;
+    a.idx_ahead[e0] = fv_column_index(a.corpus[start0 + c], c, a.w, a.V);
+  }
+  if (threadIdx.x >= 64)
+    for (uint32_t e = e0 + gridDim.x * TS; e < ahead_entries; e += gridDim.x * TS) {
+      const uint32_t r = e / a.w, c = e - r * a.w;
+      a.idx_ahead[e] = fv_column_index(a.corpus[a.pstart[a.ahead_first + r] + c], c, a.w, a.V);
+    }
   // ds of the first record does not depend on the scale: formed while the first wave waits
   // (every thread takes this path, with no additions where it has no record: the fetch is then
   // complete in every thread before the stores below)
@@ -1278,6 +1319,7 @@ static void fv_trainer_free_corpus(fv_trainer *t) {
   t->invf = nullptr;
   t->n_tokens = t->n_windows = 0;
   t->have_corpus = false;
+  t->ahead_valid = false;
 }
 
 // Waits for the trainer's stream; reports a single-launch dense pass that gave up waiting for its
@@ -1299,6 +1341,7 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   fv_trainer_free_corpus(t);
   (void)hipFree(t->Wt);
   (void)hipFree(t->idx);
+  (void)hipFree(t->idx_ahead);
   (void)hipFree(t->slots);
   (void)hipFree(t->slot_count);
   (void)hipFree(t->order);
@@ -1324,6 +1367,10 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMalloc((void **)&t->Wt, elems * sizeof(float)));
   FV_HIP(hipMalloc((void **)&t->idx, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t)));
   FV_HIP(hipMemsetAsync(t->idx, 0xff, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t), t->stream));
+  if (t->onepass_unroll) {
+    FV_HIP(hipMalloc((void **)&t->idx_ahead, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t)));
+    FV_HIP(hipMemsetAsync(t->idx_ahead, 0xff, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t), t->stream));
+  }
   FV_HIP(hipMalloc((void **)&t->win, ((size_t)t->B + 16) * sizeof(int32_t)));  // read in 16-byte pieces
   FV_HIP(hipMalloc((void **)&t->sc, (size_t)t->B * sizeof(float)));
   FV_HIP(hipMalloc((void **)&t->order, (size_t)t->B * sizeof(uint32_t)));
@@ -1546,6 +1593,7 @@ extern "C" int fv_trainer_shuffle(fv_trainer *t, uint64_t seed) {
   hipLaunchKernelGGL(fv_shuffle_kernel, dim3(fv_perm_blocks(n)), dim3(256), 0, t->stream, t->perm, t->perm_alt, n, f);
   FV_HIP(hipGetLastError());
   std::swap(t->perm, t->perm_alt);
+  t->ahead_valid = false;  // sampled in the old order
   hipLaunchKernelGGL(fv_order_starts_kernel, dim3(fv_perm_blocks(n)), dim3(256), 0, t->stream, t->perm, t->starts,
                      t->pstart, n);
   FV_HIP(hipGetLastError());
@@ -1565,6 +1613,7 @@ extern "C" int fv_trainer_set_permutation(fv_trainer *t, const uint64_t *perm, u
                (unsigned long long)i, (unsigned long long)perm[i]);
   FV_HIP(hipStreamSynchronize(t->stream));
   FV_HIP(hipMemcpy(t->perm, perm, n * sizeof(uint64_t), hipMemcpyHostToDevice));
+  t->ahead_valid = false;  // sampled in the old order
   hipLaunchKernelGGL(fv_order_starts_kernel, dim3(fv_perm_blocks(n)), dim3(256), 0, t->stream, t->perm, t->starts,
                      t->pstart, n);
   FV_HIP(hipGetLastError());
@@ -1651,6 +1700,17 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.w = t->w;
   g.V = (uint32_t)t->V;
   g.tie_rule = t->cfg.tie_rule;
+  // a whole step whose windows the previous one has sampled ahead takes that buffer
+  const bool whole = which == 0x3f;
+  g.sampled = 0;
+  if (whole) {
+    if (t->ahead_valid && t->ahead_first == first && t->ahead_n == n) {
+      std::swap(t->idx, t->idx_ahead);
+      g.idx = t->idx;
+      g.sampled = 1;
+    }
+    t->ahead_valid = false;
+  }
   if (ev) FV_HIP(hipEventRecord(ev[0], t->stream));
   if (which & 1u) switch ((t->K + 63) / 64) {
 #define FV_CASE(NV) case NV: fv_launch_gather<NV>(g, anti, t->stream); break;
@@ -1737,6 +1797,11 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.arrive = nullptr;
   d.status = nullptr;
   d.epoch = d.spin_limit = 0;
+  d.corpus = t->corpus;
+  d.pstart = t->pstart;
+  d.idx_ahead = nullptr;
+  d.ahead_first = 0;
+  d.ahead_n = 0;
   d.slot_stride = (uint64_t)t->B * t->w * (anti ? 2 : 1);
   d.bmax = t->bmax;
   d.scalars = t->scalars;
@@ -1759,6 +1824,16 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
       d.status = t->onepass_status;
       d.epoch = t->onepass_epoch;
       d.spin_limit = t->onepass_spin_limit;
+      // the windows that follow this step's, a full batch or what is left of the order
+      const uint64_t next_first = first + n;
+      if (whole && next_first < t->n_windows) {
+        d.ahead_first = next_first;
+        d.ahead_n = (uint32_t)(t->n_windows - next_first < t->B ? t->n_windows - next_first : t->B);
+        d.idx_ahead = t->idx_ahead;
+        t->ahead_valid = true;
+        t->ahead_first = next_first;
+        t->ahead_n = d.ahead_n;
+      }
       const bool narrow = (uint64_t)t->K * FV_NB_CLASSES <= 2 * FV_ONEPASS_THREADS;
       const size_t smem1 = fv_onepass_smem(t);
 #define FV_CASE(U, P)                                                                     \

@@ -290,6 +290,50 @@ def test_repeatable_and_permutation_round_trip(gpu):
     assert np.array_equal(outs[0], outs[1])
 
 
+@pytest.mark.parametrize("launches", [1, 2])
+def test_steps_in_any_order_and_across_order_changes(gpu, oracle_lib, launches):
+    """The single dense launch samples the column indices of the windows that follow its step; the next
+    step uses them only if it takes exactly those windows in an unchanged order.  Sequential steps, jumps,
+    partial batches, a new permutation, a device reshuffle and a new corpus in between: always the oracle's W."""
+    from flyvec_amd import synthetic
+    to = oracle_lib
+    V, K, w, B = 300, 64, 7, 128
+    tokens, offsets = small_corpus(20000, V)
+    W0 = synthetic.synapses(K, V)
+    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, launches=launches)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    nwin = t.num_windows
+    Wo = W0.copy()
+
+    def both(first, n, corpus=tokens, st=starts, f=invf):
+        t.step(first, n, 1e-3)
+        wo = to.train_steps(Wo, corpus, st, perm, first, n, 1, w, f, 1e-3)
+        assert np.array_equal(t.winners(n), wo), (first, n)
+
+    both(0, B); both(B, B); both(2 * B, B)        # the windows that follow: sampled ahead
+    both(7 * B, B)                                  # a jump
+    both(8 * B, 100)                                # fewer windows than were sampled ahead
+    both(8 * B + 100, B); both(9 * B + 100, B)      # following a partial batch
+    both(0, B)                                      # backwards
+    both(nwin - B - 40, B); both(nwin - 40, 40)     # the last, partial batch of the order (sampled ahead as such)
+    assert np.array_equal(t.get_weights(), Wo)
+    both(B, B)
+    perm = np.random.default_rng(9).permutation(nwin).astype(np.uint64)
+    t.set_permutation(perm)                         # the windows that follow are other windows now
+    both(2 * B, B); both(3 * B, B)
+    t.shuffle(5)
+    perm = t.get_permutation()
+    both(4 * B, B); both(5 * B, B)
+    assert np.array_equal(t.get_weights(), Wo)
+    tokens2, offsets2 = small_corpus(15000, V, seed=3)
+    t.set_corpus(tokens2, offsets2)                 # identity order over another corpus
+    starts2, invf2 = oracle_inputs(to, tokens2, offsets2, V, w)
+    perm = np.arange(t.num_windows, dtype=np.uint64)
+    both(6 * B, B, tokens2, starts2, invf2); both(7 * B, B, tokens2, starts2, invf2)
+    assert np.array_equal(t.get_weights(), Wo)
+    t.close()
+
+
 def test_device_shuffle_is_a_cumulative_bijection(gpu):
     from flyvec_amd import Trainer
     V, w = 300, 11
