@@ -29,6 +29,7 @@
 #include <math.h>
 #include <string.h>
 
+#include <atomic>
 #include <utility>
 #include <vector>
 
@@ -1322,6 +1323,11 @@ static void fv_trainer_free_corpus(fv_trainer *t) {
   t->ahead_valid = false;
 }
 
+// Trainers alive in this process. The single dense launch needs every compute unit for itself: two
+// of them in flight at once, from two trainers' streams, could each hold half the machine and wait
+// for the other half, so the form is only used while one trainer exists.
+static std::atomic<int> fv_trainers_alive{0};
+
 // Waits for the trainer's stream; reports a single-launch dense pass that gave up waiting for its
 // other blocks (the step it belonged to did not update the matrix).
 static int fv_trainer_wait(fv_trainer *t) {
@@ -1357,6 +1363,7 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   (void)hipFree(t->arrive);
   if (t->onepass_status) (void)hipHostFree(t->onepass_status);
   if (t->stream) (void)hipStreamDestroy(t->stream);
+  fv_trainers_alive.fetch_sub(1);
   delete t;
   return FV_OK;
 }
@@ -1448,6 +1455,7 @@ extern "C" int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_tr
              "batch x window = %llu is out of range", (unsigned long long)cfg->batch * cfg->window);
   fv_trainer *t = new fv_trainer();
   memset(t, 0, sizeof *t);
+  fv_trainers_alive.fetch_add(1);
   t->cfg = *cfg;
   t->K = cfg->hid;
   t->ldk = ldk;
@@ -1816,7 +1824,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.prec = t->cfg.prec;
   d.update_cut = t->update_cut;
   const size_t smem = (size_t)t->ldk * sizeof(float);
-  if (t->onepass) {
+  const bool onepass = t->onepass && fv_trainers_alive.load() == 1;
+  if (onepass) {
     // both dense passes in the launch that takes the place of the first one
     if (which & 8u) {
       if (++t->onepass_epoch == 0) t->onepass_epoch = 1;
@@ -1854,7 +1863,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
     if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
   }
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
-  if ((which & 32u) && !t->onepass) {  // the single launch has finished the sparse elements as well
+  if ((which & 32u) && !onepass) {  // the single launch has finished the sparse elements as well
     if (anti)
       hipLaunchKernelGGL(fv_slot_update_kernel<true>, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, d);
     else
@@ -1944,7 +1953,7 @@ extern "C" int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches) {
 
 extern "C" int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches) {
   FV_REQUIRE(t && out_launches, FV_ERR_INVALID, "null argument");
-  *out_launches = t->onepass ? 1u : 2u;
+  *out_launches = t->onepass && fv_trainers_alive.load() == 1 ? 1u : 2u;
   return FV_OK;
 }
 

@@ -165,9 +165,11 @@ int fv_trainer_sync(fv_trainer *t);
  * the update, flyvec/src/cuda_funcs.cu:1787-1806) run as ONE launch that keeps the matrix in
  * registers between them when it fits the device (64 MiB on 256 compute units), else as two.
  * launches = 1 or 2 forces the form (1 fails with FV_ERR_INVALID when the matrix does not fit),
- * 0 returns to the choice made at creation. Results are bit-identical either way. */
+ * 0 returns to the choice made at creation. Results are bit-identical either way. The single
+ * launch needs the whole device for itself, so while a process holds more than one trainer every
+ * step takes two launches whatever is set here. */
 int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches);
-int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches); /* 1 or 2: the form in use */
+int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches); /* 1 or 2: the form the next step takes */
 /* Test hook: between its two passes a single-launch dense pass waits for all its blocks, at most
  * `rounds` polling rounds (2^14 by default, tens of milliseconds); 0 makes every block give up at once, which
  * is how the error path of fv_trainer_sync is exercised. No counterpart in the reference. */

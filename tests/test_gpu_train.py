@@ -334,6 +334,36 @@ def test_steps_in_any_order_and_across_order_changes(gpu, oracle_lib, launches):
     t.close()
 
 
+def test_two_trainers_side_by_side(gpu, oracle_lib):
+    """The single dense launch wants every compute unit, so two trainers in one process both take two launches
+    (steps of both are enqueued without a synchronisation in between here); alone again, a trainer returns to one."""
+    from flyvec_amd import synthetic
+    to = oracle_lib
+    V, K, w, B = 300, 64, 7, 128
+    tokens, offsets = small_corpus(20000, V)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    Wa, Wb = synthetic.synapses(K, V, seed=1), synthetic.synapses(K, V, seed=2)
+    a, perm_a = make_trainer(tokens, offsets, V, K, w, B, Wa, perm_seed=6)
+    assert a.dense_launches == 1
+    b, perm_b = make_trainer(tokens, offsets, V, K, w, B, Wb, perm_seed=7)
+    assert a.dense_launches == 2 and b.dense_launches == 2
+    for s in range(6):
+        a.step(s * B, B, 1e-3)
+        b.step(s * B, B, 1e-3)
+    b.sync()
+    Wo = Wb.copy()
+    to.train_steps(Wo, tokens, starts, perm_b, 0, B, 6, w, invf, 1e-3)
+    assert np.array_equal(b.get_weights(), Wo)
+    b.close()
+    assert a.dense_launches == 1
+    for s in range(6, 9):
+        a.step(s * B, B, 1e-3)
+    Wo = Wa.copy()
+    to.train_steps(Wo, tokens, starts, perm_a, 0, B, 9, w, invf, 1e-3)
+    assert np.array_equal(a.get_weights(), Wo)
+    a.close()
+
+
 def test_device_shuffle_is_a_cumulative_bijection(gpu):
     from flyvec_amd import Trainer
     V, w = 300, 11
