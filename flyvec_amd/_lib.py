@@ -35,7 +35,9 @@ class TrainConfig(C.Structure):
         ("initial_learning_rate", C.c_float),
         ("delta", C.c_float),
         ("prec", C.c_float),
-        ("reserved", C.c_uint32),
+        ("lmid", C.c_float),
+        ("lbase", C.c_float),
+        ("prune_duplicates", C.c_uint32),
     ]
 
 
@@ -58,6 +60,7 @@ SIGNATURES = {
     "fv_build_window_starts": [_vp, _u64, _u64, _vp, _u64],
     "fv_inverse_frequency": [_vp, _u64, _u64, _vp],
     "fv_mask_tokens": [_vp, _u64, _vp, _u64, _u64],
+    "fv_prune_windows": [_vp, _u64, _u64],
     "fv_trainer_create": [C.POINTER(TrainConfig), _pp],
     "fv_trainer_destroy": [_vp],
     "fv_trainer_set_corpus": [_vp, _vp, _u64, _vp, _u64],

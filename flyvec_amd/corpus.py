@@ -100,6 +100,16 @@ def mask_tokens(tokens, remove_ids, vocab=None):
     return tokens
 
 
+def prune_windows(windows):
+    """In place: in every row of an int32 (rows, cols) window matrix a value that an earlier column holds
+    becomes -1; the centre column takes no part and keeps its value (flyvec/src/prune_input.cpp:14
+    prune_input_data, a tool the reference exports but never calls)."""
+    if windows.dtype != np.int32 or windows.ndim != 2 or not windows.flags.c_contiguous or not windows.flags.writeable:
+        raise ValueError("windows must be a writable C-contiguous int32 matrix")
+    check(_lib.load().fv_prune_windows(ptr(windows), windows.shape[0], windows.shape[1]))
+    return windows
+
+
 def merge_directory(shard_dir, out_dir, stop_ids=None):
     """Shards of the reference's encoder -> encodings.npy + offsets.npy for ``flyvec_train``."""
     pairs = shard_pairs(shard_dir)

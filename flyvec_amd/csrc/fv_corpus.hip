@@ -386,3 +386,49 @@ extern "C" int fv_mask_tokens(int32_t *tokens, uint64_t n_tokens, const int32_t 
   if (e != hipSuccess) return fv_fail(FV_ERR_HIP, "fv_mask_tokens failed: %s", hipGetErrorString(e));
   return FV_OK;
 }
+
+// ---- in-window duplicate pruning of a window matrix (an off-line tool of the reference) ---------------
+
+// One wavefront per row, lane c holds the value of column c. flyvec/src/prune_input.cpp:14-60 scans a
+// row left to right and replaces a value already kept at an earlier position by -1; the centre column
+// takes no part (it counts as -1 during the scan) and keeps its value. A first occurrence is always
+// kept, so: a column other than the centre loses its value if an earlier column other than the centre
+// holds the same one.
+__global__ __launch_bounds__(256) void fv_prune_windows_kernel(int32_t *__restrict__ data, uint64_t rows,
+                                                               uint32_t cols) {
+  const int lane = threadIdx.x & 63;
+  const int mid = (int)(cols / 2);
+  for (uint64_t r = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6); r < rows; r += (uint64_t)gridDim.x * 4) {
+    const int32_t val = lane < (int)cols ? data[r * cols + lane] : -1;
+    bool dup = false;
+    for (int j = 0; j + 1 < (int)cols; ++j) {
+      const int32_t earlier = (int32_t)fv_readlane((uint32_t)val, j);
+      dup = dup || (lane > j && j != mid && earlier == val);
+    }
+    if (lane < (int)cols && lane != mid && dup) data[r * cols + lane] = -1;
+  }
+}
+
+#define FV_PRUNE_PART (1ull << 26)  // matrix entries per trip through the device
+
+extern "C" int fv_prune_windows(int32_t *data, uint64_t rows, uint64_t cols) {
+  FV_REQUIRE(data || rows == 0 || cols == 0, FV_ERR_INVALID, "fv_prune_windows: null matrix");
+  FV_REQUIRE(cols <= FV_MAX_WINDOW, FV_ERR_INVALID, "fv_prune_windows: %llu columns, at most %d are supported",
+             (unsigned long long)cols, FV_MAX_WINDOW);
+  if (rows == 0 || cols <= 1) return FV_OK;
+  const uint64_t part_rows = FV_PRUNE_PART / cols < rows ? FV_PRUNE_PART / cols : rows;
+  int32_t *buf = nullptr;
+  hipError_t e = hipMalloc((void **)&buf, part_rows * cols * sizeof(int32_t));
+  for (uint64_t first = 0; e == hipSuccess && first < rows; first += part_rows) {
+    const uint64_t n = rows - first < part_rows ? rows - first : part_rows;
+    e = hipMemcpy(buf, data + first * cols, n * cols * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (e != hipSuccess) break;
+    const unsigned blocks = (unsigned)((n + 3) / 4 < 16384 ? (n + 3) / 4 : 16384);
+    hipLaunchKernelGGL(fv_prune_windows_kernel, dim3(blocks), dim3(256), 0, 0, buf, n, (uint32_t)cols);
+    e = hipGetLastError();
+    if (e == hipSuccess) e = hipMemcpy(data + first * cols, buf, n * cols * sizeof(int32_t), hipMemcpyDeviceToHost);
+  }
+  (void)hipFree(buf);
+  if (e != hipSuccess) return fv_fail(FV_ERR_HIP, "fv_prune_windows failed: %s", hipGetErrorString(e));
+  return FV_OK;
+}

@@ -142,16 +142,22 @@ __device__ __forceinline__ uint32_t fv_wave_min_u32(uint32_t v) { return ~fv_wav
 // Every load is unconditional -- rows of skipped positions read row 0, lanes past K re-read
 // element K - 1, both replaced by 0 afterwards -- so a batch of RB rows is RB * NV independent
 // loads in flight per lane with no branch between them.
-template <int NV, int RB, typename Acc>
+// WEIGHTED: every weight is first multiplied, in fp32, by the weight of its window position --
+// l_mid for the centre, whose column lies in the second half of the columns, l_base for the others
+// (flyvec/src/cuda_funcs.cu:266-286).
+template <int NV, int RB, typename Acc, bool WEIGHTED = false>
 __device__ __forceinline__ void fv_gather_batch(const float *__restrict__ Wt, uint32_t ldk, uint32_t n_cols,
                                                 const uint32_t (&off)[NV], bool last_valid, int c0,
-                                                int32_t idx_lane, Acc (&acc)[NV]) {
+                                                int32_t idx_lane, Acc (&acc)[NV], float l_mid = 1.0f,
+                                                float l_base = 1.0f) {
   float v[RB][NV];
   bool ok[RB];
+  float l[RB];
 #pragma unroll
   for (int b = 0; b < RB; ++b) {
     const int32_t i = (int32_t)fv_readlane((uint32_t)idx_lane, c0 + b);
     ok[b] = (uint32_t)i < n_cols;
+    l[b] = (uint32_t)i >= n_cols / 2 ? l_mid : l_base;
     const float *row = Wt + (uint64_t)(ok[b] ? (uint32_t)i : 0u) * ldk;
 #pragma unroll
     for (int j = 0; j < NV; ++j) v[b][j] = row[off[j]];
@@ -161,23 +167,26 @@ __device__ __forceinline__ void fv_gather_batch(const float *__restrict__ Wt, ui
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const bool use = ok[b] && (j < NV - 1 || last_valid);
-      acc[j] = acc[j] + (Acc)(use ? v[b][j] : 0.0f);
+      const float t = WEIGHTED ? __fmul_rn(v[b][j], l[b]) : v[b][j];
+      acc[j] = acc[j] + (Acc)(use ? t : 0.0f);
     }
   }
 }
 
-template <int NV, int RB, typename Acc>
+template <int NV, int RB, typename Acc, bool WEIGHTED = false>
 __device__ __forceinline__ void fv_gather_accumulate(const float *__restrict__ Wt, uint32_t ldk, uint32_t K,
                                                      uint32_t n_cols, int lane, int w, int32_t idx_lane,
-                                                     Acc (&acc)[NV]) {
+                                                     Acc (&acc)[NV], float l_mid = 1.0f, float l_base = 1.0f) {
   uint32_t off[NV];
 #pragma unroll
   for (int j = 0; j < NV; ++j) off[j] = (uint32_t)lane + 64u * j;
   const bool last_valid = off[NV - 1] < K;
   if (!last_valid) off[NV - 1] = K - 1;
   int c0 = 0;
-  for (; c0 + RB <= w; c0 += RB) fv_gather_batch<NV, RB, Acc>(Wt, ldk, n_cols, off, last_valid, c0, idx_lane, acc);
-  for (; c0 < w; ++c0) fv_gather_batch<NV, 1, Acc>(Wt, ldk, n_cols, off, last_valid, c0, idx_lane, acc);
+  for (; c0 + RB <= w; c0 += RB)
+    fv_gather_batch<NV, RB, Acc, WEIGHTED>(Wt, ldk, n_cols, off, last_valid, c0, idx_lane, acc, l_mid, l_base);
+  for (; c0 < w; ++c0)
+    fv_gather_batch<NV, 1, Acc, WEIGHTED>(Wt, ldk, n_cols, off, last_valid, c0, idx_lane, acc, l_mid, l_base);
 }
 
 template <int NV>

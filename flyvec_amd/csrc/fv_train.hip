@@ -126,6 +126,8 @@ struct fv_gather_args {
   uint64_t first;
   uint32_t n, K, ldk, w, V, tie_rule;
   uint32_t sampled;  // idx already holds this minibatch
+  uint32_t prune;    // in-window duplicate pruning while sampling
+  float lmid, lbase; // weight of a window's centre position and of the others (WEIGHTED kernels)
 };
 
 // FV_GATHER_WINDOWS windows per wavefront, one after the other: the grid then fits the machine in
@@ -135,8 +137,22 @@ struct fv_gather_args {
 #define FV_GATHER_WINDOWS 1
 #endif
 
-template <int NV, bool DELTA>
+template <int NV, bool DELTA, bool WEIGHTED>
 __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, uint32_t r, int32_t idx, int lane);
+
+// In-window duplicate pruning of the reference's switched-off sampler variant
+// (flyvec/src/cuda_funcs.cu:938-979): for i = 1 .. w-1 every position >= i holding the current value
+// of position i-1 becomes -1, then the centre gets its token back. A first occurrence is never
+// pruned, so that is: a position other than the centre loses its token if an earlier position holds
+// the same one. Lane c holds the token of position c; called by the lanes below w together.
+__device__ __forceinline__ int32_t fv_prune_token(int32_t tok, int lane, int w) {
+  bool dup = false;
+  for (int j = 0; j + 1 < w; ++j) {
+    const int32_t earlier = (int32_t)fv_readlane((uint32_t)tok, j);
+    dup = dup || (lane > j && earlier == tok);
+  }
+  return (dup && lane != w / 2) ? -1 : tok;
+}
 
 // Column index of position c of a window from its token: a masked token stays -1, the centre token
 // addresses the target block (flyvec/src/cuda_funcs.cu:915-936).
@@ -145,8 +161,8 @@ __device__ __forceinline__ int32_t fv_column_index(int32_t tok, uint32_t c, uint
 }
 
 // DELTA: also the window's second neuron (flyvec/src/cuda_funcs.cu:495-548 with num_m = 2), which
-// receives the anti-Hebbian terms.
-template <int NV, bool DELTA>
+// receives the anti-Hebbian terms. WEIGHTED: position weights other than 1 (:266-286, :307-327).
+template <int NV, bool DELTA, bool WEIGHTED>
 __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a) {
   const int lane = threadIdx.x & 63;
   const uint32_t g = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -164,7 +180,9 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
         idx[k] = a.idx[(uint64_t)r * a.w + lane];
       } else {
         const uint64_t s = a.pstart[a.first + r];
-        idx[k] = fv_column_index(a.corpus[s + lane], (uint32_t)lane, a.w, a.V);
+        int32_t tok = a.corpus[s + lane];
+        if (a.prune) tok = fv_prune_token(tok, lane, (int)a.w);
+        idx[k] = fv_column_index(tok, (uint32_t)lane, a.w, a.V);
         a.idx[(uint64_t)r * a.w + lane] = idx[k];
       }
     }
@@ -172,7 +190,7 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
 #pragma unroll
   for (int k = 0; k < FV_GATHER_WINDOWS; ++k) {
     const uint32_t r = g + k * per;
-    if (r < a.n) fv_gather_one_window<NV, DELTA>(a, r, idx[k], lane);
+    if (r < a.n) fv_gather_one_window<NV, DELTA, WEIGHTED>(a, r, idx[k], lane);
   }
 }
 
@@ -206,11 +224,13 @@ __device__ __forceinline__ uint32_t fv_wave_argmax(const double (&acc)[NV], uint
 
 // Frequency-scaled activation of neuron h for the window whose column index c sits in lane c:
 // fp32 products, double sum in window order, one rounding (flyvec/src/cuda_funcs.cu:289-305).
+template <bool WEIGHTED>
 __device__ __forceinline__ float fv_scaled_activation(const fv_gather_args &a, int32_t idx, uint32_t h) {
   double pd = 0.0;
   if ((uint32_t)idx < 2 * a.V) {
-    const float wv = a.Wt[(uint64_t)idx * a.ldk + h];
+    float wv = a.Wt[(uint64_t)idx * a.ldk + h];
     const float f = a.invf[(uint32_t)idx >= a.V ? (uint32_t)idx - a.V : (uint32_t)idx];
+    if (WEIGHTED) wv = __fmul_rn(wv, (uint32_t)idx >= a.V ? a.lmid : a.lbase);  // (W * L) * 1/f, :307-327
     pd = (double)__fmul_rn(wv, f);
   }
   double s = 0.0;
@@ -223,16 +243,16 @@ __device__ __forceinline__ float fv_scaled_activation(const fv_gather_args &a, i
   return (float)s;
 }
 
-template <int NV, bool DELTA>
+template <int NV, bool DELTA, bool WEIGHTED>
 __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, uint32_t r, int32_t idx, int lane) {
   double acc[NV];
 #pragma unroll
   for (int j = 0; j < NV; ++j) acc[j] = 0.0;
-  fv_gather_accumulate<NV, fv_rows_per_batch<NV>::value, double>(a.Wt, a.ldk, a.K, 2 * a.V, lane,
-                                                                 (int)a.w, idx, acc);
+  fv_gather_accumulate<NV, fv_rows_per_batch<NV>::value, double, WEIGHTED>(a.Wt, a.ldk, a.K, 2 * a.V, lane,
+                                                                           (int)a.w, idx, acc, a.lmid, a.lbase);
   const uint32_t hstar = fv_wave_argmax<NV>(acc, a.K, a.tie_rule, lane, 0xffffffffu);
   // the scaled activation is only ever read at the chosen neurons (flyvec/src/cuda_funcs.cu:731)
-  const float s = fv_scaled_activation(a, idx, hstar);
+  const float s = fv_scaled_activation<WEIGHTED>(a, idx, hstar);
   if (lane == 0) {
     a.win[r] = (int32_t)hstar;
     a.win16[r] = (uint16_t)hstar;
@@ -240,7 +260,7 @@ __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, ui
   }
   if (DELTA) {
     const uint32_t second = fv_wave_argmax<NV>(acc, a.K, a.tie_rule, lane, hstar);
-    const float s2 = fv_scaled_activation(a, idx, second);
+    const float s2 = fv_scaled_activation<WEIGHTED>(a, idx, second);
     if (lane == 0) {
       a.win2[r] = (int32_t)second;
       a.win2_16[r] = (uint16_t)second;
@@ -286,9 +306,11 @@ struct fv_group_args {
   uint32_t accumulate;  // add the total to xx[h] instead of storing it
 };
 
-// ds of one sparse element: the dense term, then n sequential additions of 1/f.
-__device__ __forceinline__ float fv_sparse_ds(float xx, float wv, float f, uint32_t n) {
-  return fv_add_repeat(__fmul_rn(-xx, wv), f, n);
+// ds of one sparse element: the dense term, then n sequential additions of l * 1/f, l the weight of
+// the element's window position (flyvec/src/cuda_funcs.cu:675-697: a double product of two floats
+// rounded once is their fp32 product; l = 1 leaves 1/f as it is).
+__device__ __forceinline__ float fv_sparse_ds(float xx, float wv, float f, uint32_t n, float l) {
+  return fv_add_repeat(__fmul_rn(-xx, wv), __fmul_rn(l, f), n);
 }
 
 __device__ __forceinline__ float fv_absmax_keep(float m, float v) {
@@ -296,10 +318,12 @@ __device__ __forceinline__ float fv_absmax_keep(float m, float v) {
   return a > m ? a : m;  // a NaN never replaces m, as in the reference's comparison
 }
 
-// ds of one sparse element with the anti-Hebbian term: after the n additions of 1/f, n2 additions
-// of -delta * 1/f (flyvec/src/cuda_funcs.cu:667-668; this order of the additions is the checker's).
-__device__ __forceinline__ float fv_sparse_ds2(float xx, float wv, float f, uint32_t n, float delta, uint32_t n2) {
-  return fv_add_repeat(fv_sparse_ds(xx, wv, f, n), __fmul_rn(-delta, f), n2);
+// ds of one sparse element with the anti-Hebbian term: after the n additions of l * 1/f, n2 additions
+// of (-delta * l) * 1/f (flyvec/src/cuda_funcs.cu:667-668, 689, 693; this order of the additions is
+// the checker's).
+__device__ __forceinline__ float fv_sparse_ds2(float xx, float wv, float f, uint32_t n, float delta, uint32_t n2,
+                                               float l) {
+  return fv_add_repeat(fv_sparse_ds(xx, wv, f, n, l), __fmul_rn(__fmul_rn(-delta, l), f), n2);
 }
 
 // Block-wide maximum of non-negative floats (blocks of up to 16 waves; smem holds one float per wave).
@@ -543,6 +567,7 @@ struct fv_sparse_args {
   const uint32_t *group_count2;
   uint32_t *slot_n2;
   float delta;
+  float lmid, lbase;  // weight of a window's centre position (columns >= V) and of the others
 };
 
 // Barrier for data exchanged through LDS only: waits for the wave's LDS operations, not for its
@@ -738,7 +763,7 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
       // xx == 0 has ds == 0)
       for (uint32_t eb = tid; eb < take; eb += 4 * T) {
         uint32_t pe[4], ne[4], n2e[4];
-        float wv[4], fe[4];
+        float wv[4], fe[4], le[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           const uint32_t k = list[min(eb + u * T, take - 1)];
@@ -753,6 +778,7 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
           pe[u] = col * a.ldk + h;
           wv[u] = a.Wt[pe[u]];
           fe[u] = a.invf[col >= a.V ? col - a.V : col];
+          le[u] = col >= a.V ? a.lmid : a.lbase;
           if (eb + u * T < take) {
             if (narrow) {
               atomicAnd(&cnt[k >> 1], 0xffff0000u >> (16 * (k & 1)));
@@ -775,8 +801,8 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
             if (DELTA) a.slot_n2[slot_first + emitted + eb + u * T] = n2e[u];
             a.Wt[pe[u]] = __uint_as_float(FV_SENTINEL);
             if (x_h != 0.0f)
-              ds_max = fv_absmax_keep(ds_max, DELTA ? fv_sparse_ds2(x_h, wv[u], fe[u], ne[u], a.delta, n2e[u])
-                                                    : fv_sparse_ds(x_h, wv[u], fe[u], ne[u]));
+              ds_max = fv_absmax_keep(ds_max, DELTA ? fv_sparse_ds2(x_h, wv[u], fe[u], ne[u], a.delta, n2e[u], le[u])
+                                                    : fv_sparse_ds(x_h, wv[u], fe[u], ne[u], le[u]));
           }
       }
       emitted += take;
@@ -811,6 +837,7 @@ struct fv_dense_args {
   unsigned long long *arrive;
   uint32_t *status;
   uint32_t epoch, spin_limit;
+  float lmid, lbase;  // weight of a window's centre position (elements p >= V * ldk) and of the others
   // the minibatch sampled ahead (ahead_n = 0: none)
   const int32_t *corpus;
   const uint64_t *pstart;
@@ -1166,8 +1193,9 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   const float *xs = (const float *)xs4;
   const float x0 = xs[h0];
   const bool update0 = live0 && x0 != 0.0f;
-  const float ds0 = DELTA ? fv_sparse_ds2(x0, sl0.wv, sl0.f, update0 ? sl0.n : 0u, a.delta, update0 ? n20 : 0u)
-                          : fv_sparse_ds(x0, sl0.wv, sl0.f, update0 ? sl0.n : 0u);
+  const float l0 = sl0.p >= a.V * a.ldk ? a.lmid : a.lbase;
+  const float ds0 = DELTA ? fv_sparse_ds2(x0, sl0.wv, sl0.f, update0 ? sl0.n : 0u, a.delta, update0 ? n20 : 0u, l0)
+                          : fv_sparse_ds(x0, sl0.wv, sl0.f, update0 ? sl0.n : 0u, l0);
   __syncthreads();
   const bool ok = sh_ok != 0;
   const float s = sh_s;
@@ -1196,8 +1224,9 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
     const fv_slot sl = a.slots[at];
     float out = sl.wv;
     if (ok && xs[h] != 0.0f) {
-      const float ds = DELTA ? fv_sparse_ds2(xs[h], sl.wv, sl.f, sl.n, a.delta, a.slot_n2[at])
-                             : fv_sparse_ds(xs[h], sl.wv, sl.f, sl.n);
+      const float l = sl.p >= a.V * a.ldk ? a.lmid : a.lbase;
+      const float ds = DELTA ? fv_sparse_ds2(xs[h], sl.wv, sl.f, sl.n, a.delta, a.slot_n2[at], l)
+                             : fv_sparse_ds(xs[h], sl.wv, sl.f, sl.n, l);
       const float d = __fmul_rn(s, ds);
       if (fabsf(d) > a.update_cut) out = __fadd_rn(sl.wv, d);
     }
@@ -1250,8 +1279,9 @@ __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
       if (eb + u * 256 >= count) break;
       float out = sl[u].wv;  // a row with xx == 0 is not updated: the saved weight goes back
       if (x != 0.0f) {
-        const float ds = DELTA ? fv_sparse_ds2(x, sl[u].wv, sl[u].f, sl[u].n, a.delta, n2[u])
-                               : fv_sparse_ds(x, sl[u].wv, sl[u].f, sl[u].n);
+        const float l = sl[u].p >= a.V * a.ldk ? a.lmid : a.lbase;
+        const float ds = DELTA ? fv_sparse_ds2(x, sl[u].wv, sl[u].f, sl[u].n, a.delta, n2[u], l)
+                               : fv_sparse_ds(x, sl[u].wv, sl[u].f, sl[u].n, l);
         const float d = __fmul_rn(s, ds);
         if (fabsf(d) > a.update_cut) out = __fadd_rn(sl[u].wv, d);
       }
@@ -1442,6 +1472,10 @@ extern "C" int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_tr
   FV_REQUIRE(cfg->vocab >= 1 && cfg->vocab < (1ull << 30), FV_ERR_INVALID,
              "vocab = %llu is out of range", (unsigned long long)cfg->vocab);
   FV_REQUIRE(cfg->tie_rule <= 1, FV_ERR_INVALID, "tie_rule must be 0 or 1");
+  FV_REQUIRE(cfg->prune_duplicates <= 1, FV_ERR_INVALID, "prune_duplicates must be 0 or 1");
+  FV_REQUIRE(fabsf(cfg->lmid) <= 1.0e6f && fabsf(cfg->lbase) <= 1.0e6f, FV_ERR_INVALID,
+             "Lmid = %g, Lbase = %g: out of range (1 and 1 are the reference's values)", (double)cfg->lmid,
+             (double)cfg->lbase);
   FV_REQUIRE(cfg->delta == cfg->delta && fabsf(cfg->delta) <= 1.0e6f, FV_ERR_INVALID, "delta = %g is out of range",
              (double)cfg->delta);
   // the slot regions of a step with delta != 0 hold twice as many records
@@ -1642,12 +1676,20 @@ extern "C" int fv_trainer_get_permutation(fv_trainer *t, uint64_t *out_perm, uin
 
 
 template <int NV>
-static void fv_launch_gather(const fv_gather_args &a, bool with_second, hipStream_t stream) {
+static void fv_launch_gather(const fv_gather_args &a, bool with_second, bool weighted, hipStream_t stream) {
   const uint32_t waves = (a.n + FV_GATHER_WINDOWS - 1) / FV_GATHER_WINDOWS;
-  if (with_second)
-    hipLaunchKernelGGL((fv_gather_winner_kernel<NV, true>), dim3((waves + 3) / 4), dim3(256), 0, stream, a);
-  else
-    hipLaunchKernelGGL((fv_gather_winner_kernel<NV, false>), dim3((waves + 3) / 4), dim3(256), 0, stream, a);
+  const dim3 grid((waves + 3) / 4), block(256);
+  if (weighted) {
+    if (with_second)
+      hipLaunchKernelGGL((fv_gather_winner_kernel<NV, true, true>), grid, block, 0, stream, a);
+    else
+      hipLaunchKernelGGL((fv_gather_winner_kernel<NV, false, true>), grid, block, 0, stream, a);
+  } else {
+    if (with_second)
+      hipLaunchKernelGGL((fv_gather_winner_kernel<NV, true, false>), grid, block, 0, stream, a);
+    else
+      hipLaunchKernelGGL((fv_gather_winner_kernel<NV, false, false>), grid, block, 0, stream, a);
+  }
 }
 
 // Enqueues the kernels of one step (those whose bit is set in `which`); ev (nullable) receives
@@ -1708,6 +1750,10 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.w = t->w;
   g.V = (uint32_t)t->V;
   g.tie_rule = t->cfg.tie_rule;
+  g.prune = t->cfg.prune_duplicates;
+  g.lmid = t->cfg.lmid;
+  g.lbase = t->cfg.lbase;
+  const bool weighted = t->cfg.lmid != 1.0f || t->cfg.lbase != 1.0f;
   // a whole step whose windows the previous one has sampled ahead takes that buffer
   const bool whole = which == 0x3f;
   g.sampled = 0;
@@ -1721,7 +1767,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   }
   if (ev) FV_HIP(hipEventRecord(ev[0], t->stream));
   if (which & 1u) switch ((t->K + 63) / 64) {
-#define FV_CASE(NV) case NV: fv_launch_gather<NV>(g, anti, t->stream); break;
+#define FV_CASE(NV) case NV: fv_launch_gather<NV>(g, anti, weighted, t->stream); break;
     FV_CASE(1) FV_CASE(2) FV_CASE(3) FV_CASE(4) FV_CASE(5) FV_CASE(6) FV_CASE(7) FV_CASE(8)
     FV_CASE(9) FV_CASE(10) FV_CASE(11) FV_CASE(12) FV_CASE(13) FV_CASE(14) FV_CASE(15) FV_CASE(16)
     FV_CASE(17) FV_CASE(18) FV_CASE(19) FV_CASE(20) FV_CASE(21) FV_CASE(22) FV_CASE(23) FV_CASE(24)
@@ -1776,6 +1822,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.group_count2 = t->group_count2;
   sp.slot_n2 = t->slot_n2;
   sp.delta = delta;
+  sp.lmid = t->cfg.lmid;
+  sp.lbase = t->cfg.lbase;
   sp.xx = t->xx;
   sp.invf = t->invf;
   sp.bmax_sparse = t->bmax + t->dense_blocks;
@@ -1805,6 +1853,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.arrive = nullptr;
   d.status = nullptr;
   d.epoch = d.spin_limit = 0;
+  d.lmid = t->cfg.lmid;
+  d.lbase = t->cfg.lbase;
   d.corpus = t->corpus;
   d.pstart = t->pstart;
   d.idx_ahead = nullptr;
@@ -1835,7 +1885,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
       d.spin_limit = t->onepass_spin_limit;
       // the windows that follow this step's, a full batch or what is left of the order
       const uint64_t next_first = first + n;
-      if (whole && next_first < t->n_windows) {
+      if (whole && next_first < t->n_windows && !t->cfg.prune_duplicates) {  // the ahead sampler does not prune
         d.ahead_first = next_first;
         d.ahead_n = (uint32_t)(t->n_windows - next_first < t->B ? t->n_windows - next_first : t->B);
         d.idx_ahead = t->idx_ahead;

@@ -40,12 +40,13 @@ class Trainer:
     """Owns the synapse matrix, the corpus and the window table in HBM."""
 
     def __init__(self, vocab, hid=400, window=11, batch=10000, initial_learning_rate=0.002,
-                 delta=0.0, prec=1.0e-30, tie_rule=0):
+                 delta=0.0, prec=1.0e-30, tie_rule=0, lmid=1.0, lbase=1.0, prune_duplicates=False):
         self.lib = _lib.load()
         self.vocab, self.hid, self.window, self.batch = int(vocab), int(hid), int(window), int(batch)
         cfg = _lib.TrainConfig(vocab=self.vocab, hid=self.hid, window=self.window, batch=self.batch,
                                tie_rule=int(tie_rule), initial_learning_rate=initial_learning_rate,
-                               delta=delta, prec=prec, reserved=0)
+                               delta=delta, prec=prec, lmid=lmid, lbase=lbase,
+                               prune_duplicates=int(bool(prune_duplicates)))
         h = C.c_void_p()
         check(self.lib.fv_trainer_create(C.byref(cfg), C.byref(h)))
         self.handle = h

@@ -42,6 +42,9 @@ def build_parser():
     p.add_argument("--hid", default=400, type=int, help="Number of hidden units (neurons)")
     p.add_argument("--initial_learning_rate", default=0.002, type=float, help="Initial learning rate")
     p.add_argument("--delta", default=0.0, type=float, help="Anti-Hebbian strength on the second neuron of a window (flyvec/src/cuda_funcs.cu:1230 schedules it over the epochs)")
+    p.add_argument("--Lmid", default=1.0, type=float, help="Weight of a window's centre position (the reference holds 1.0 and has no flag for it; flyvec/src/cuda_funcs.cu:266-327, 675-697)")
+    p.add_argument("--Lbase", default=1.0, type=float, help="Weight of the other window positions (likewise)")
+    p.add_argument("--prune_duplicates", action="store_true", help="Drop a token that an earlier position of its window holds (the sampler variant the reference has switched off, flyvec/src/cuda_funcs.cu:938-979)")
     p.add_argument("--mu", default=0.0, type=float, help="Mean of the random normal initialisation")
     p.add_argument("--sigma", default=0.02, type=float, help="Stdev of the random normal initialisation")
     p.add_argument("--Nep", default=15, type=int, help="Maximum number of epochs, fewer if starting from a checkpoint")
@@ -76,7 +79,8 @@ def train(args, log=print):
 
     trainer = Trainer(vocab=vocabulary_size, hid=args.hid, window=args.W, batch=args.batch_size,
                       initial_learning_rate=args.initial_learning_rate, delta=args.delta, prec=args.prec,
-                      tie_rule=1 if args.tie_rule == "reference" else 0)
+                      tie_rule=1 if args.tie_rule == "reference" else 0, lmid=args.Lmid, lbase=args.Lbase,
+                      prune_duplicates=args.prune_duplicates)
     log("Copying input...")
     trainer.set_corpus(tokens, offsets)
     log(f"Number of phrases:  {trainer.num_windows}")

@@ -86,6 +86,12 @@ int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, uint64_t voca
 int fv_mask_tokens(int32_t *tokens, uint64_t n_tokens, const int32_t *remove_ids, uint64_t n_remove,
                    uint64_t vocab);
 
+/* flyvec/src/prune_input.cpp:14 prune_input_data (exported by the reference, bound at
+ * flyvec/train_flyvec.py:79, never called): in every row of a rows x cols int32 window matrix a value
+ * that an earlier column holds becomes -1; the centre column (cols / 2) takes no part and keeps its
+ * value. In place, one pass on the device; cols <= 64. */
+int fv_prune_windows(int32_t *data, uint64_t rows, uint64_t cols);
+
 /* ---- trainer ------------------------------------------------------------------ */
 
 typedef struct fv_trainer fv_trainer;
@@ -102,7 +108,12 @@ typedef struct fv_train_config {
   float initial_learning_rate; /* "initial_learning_rate" */
   float delta;                 /* "delta": strength of the anti-Hebbian term on the second neuron (0 = none) */
   float prec;                  /* "prec" */
-  uint32_t reserved;           /* 0 */
+  float lmid;                  /* "Lmid": weight of a window's centre position (flyvec/src/cuda_funcs.cu:266-327,
+                                  675-697); 1 is all the reference's command line reaches */
+  float lbase;                 /* "Lbase": weight of the other positions; 1 likewise */
+  uint32_t prune_duplicates;   /* 1: the sampler drops a token that an earlier position of its window holds
+                                  (not the centre's): flyvec/src/cuda_funcs.cu:938-979, switched off in the
+                                  reference (:1681); 0 is the reference's behaviour */
 } fv_train_config;
 
 /* flyvec/src/model_descriptor.cu:18 model_create_descriptor + flyvec/src/model_arrays.cu:15,22

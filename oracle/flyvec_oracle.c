@@ -17,6 +17,12 @@
  *       invariance to a global rescale of 1/frequency by a power of two,
  *       max|dW| == eps), a from-scratch brute force in Python floats on tiny
  *       shapes, and numpy restatements of each stage.
+ *   fvo_train_step_weighted (position weights Lmid / Lbase) : the brute force
+ *       with weights, and closed forms (a weight of 0 is a masked position; a
+ *       common power of two changes no bit of the update; weights under which
+ *       centre and context elect different winners).
+ *   fvo_prune_windows : the reference's own prune_input_data (oracle/_ref).
+ *   fvo_inflate_prune : a set-based first-occurrence formulation in Python.
  *
  * Order-dependent fp32 sums (the reference uses atomics whose order is not
  * defined) are given a fixed order here.  The sparse term of ds: increasing
@@ -92,6 +98,54 @@ void fvo_inflate(const int32_t *corpus, const uint64_t *starts, const uint64_t *
       idx[r * (uint64_t)w + c] = (val == -1) ? -1 : (c == mid ? (int32_t)(val + (int64_t)V) : val);
     }
   }
+}
+
+/* flyvec/src/cuda_funcs.cu:938-979 (inflate_from_M_kernel_4_and_prune, switched off in the reference
+ * at :1681): for i = 1 .. w-1 every position c >= i that holds the CURRENT value of position i-1
+ * becomes -1; afterwards the centre gets its original token back; then the indices are formed as in
+ * fvo_inflate. */
+void fvo_inflate_prune(const int32_t *corpus, const uint64_t *starts, const uint64_t *perm,
+                       uint64_t first, uint64_t n, int w, uint64_t V, int32_t *idx) {
+  const int mid = w / 2;
+  int32_t tmp[256];
+  for (uint64_t r = 0; r < n; ++r) {
+    const int32_t *src = corpus + starts[perm[first + r]];
+    for (int c = 0; c < w; ++c) tmp[c] = src[c];
+    for (int i = 1; i < w; ++i) {
+      int32_t val = tmp[i - 1];
+      for (int c = i; c < w; ++c)
+        if (tmp[c] == val) tmp[c] = -1;
+    }
+    tmp[mid] = src[mid];
+    for (int c = 0; c < w; ++c)
+      idx[r * (uint64_t)w + c] = (tmp[c] == -1) ? -1 : (c == mid ? (int32_t)(tmp[c] + (int64_t)V) : tmp[c]);
+  }
+}
+
+/* flyvec/src/prune_input.cpp:14-60 (prune_input_data, exported by the reference but never called):
+ * rows x cols window matrix in place; scanning a row left to right, a value already kept at an
+ * earlier position becomes -1; the centre column takes no part (it counts as -1 while the row is
+ * scanned) and keeps its value. */
+void fvo_prune_windows(int32_t *data, uint64_t rows, uint64_t cols) {
+  const uint64_t mid = cols / 2;
+  int32_t *tmp = (int32_t *)malloc(sizeof(int32_t) * (cols ? cols : 1));
+  for (uint64_t r = 0; r < rows; ++r) {
+    int32_t *row = data + r * cols;
+    if (cols == 0) continue;
+    tmp[0] = row[0];
+    for (uint64_t c = 1; c < cols; ++c) {
+      if (c == mid) {
+        tmp[c] = -1;
+        continue;
+      }
+      int dup = 0;
+      for (uint64_t cc = 0; cc < c && !dup; ++cc) dup = tmp[cc] == row[c];
+      tmp[c] = dup ? -1 : row[c];
+    }
+    tmp[mid] = row[mid];
+    for (uint64_t c = 0; c < cols; ++c) row[c] = tmp[c];
+  }
+  free(tmp);
 }
 
 /* flyvec/src/cuda_funcs.cu:248-263 (raw) and :289-305 (scaled by 1/frequency):
@@ -219,10 +273,11 @@ void fvo_xx_sums(const int32_t *win, const float *sc, uint64_t n, int K, int ord
  * Outputs (any may be NULL): winners[n], sc_at_winner[n], xx[K], *nc_out.
  * ds_scratch must hold K*N floats.
  */
-void fvo_train_step_delta(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx, uint64_t n, int w,
-                          const float *invf, float eps, float prec, int tie_rule, float delta, float *ds_scratch,
-                          int32_t *winners, float *sc_at_winner, int32_t *seconds, float *sc_at_second,
-                          float *xx_out, float *nc_out) {
+void fvo_train_step_weighted(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx, uint64_t n, int w,
+                             const float *invf, float eps, float prec, int tie_rule, float delta, float lmid,
+                             float lbase, float *ds_scratch, int32_t *winners, float *sc_at_winner,
+                             int32_t *seconds, float *sc_at_second, float *xx_out, float *nc_out) {
+  const int mid = w / 2;
   int32_t *win = (int32_t *)malloc(sizeof(int32_t) * (n ? n : 1));
   float *scw = (float *)malloc(sizeof(float) * (n ? n : 1));
   int32_t *win2 = (int32_t *)malloc(sizeof(int32_t) * (n ? n : 1));
@@ -240,7 +295,11 @@ void fvo_train_step_delta(float *W, int K, uint64_t N, uint64_t V, const int32_t
         const float *row = W + (uint64_t)h * N;
         double sr = 0.0;
         for (int c = 0; c < w; ++c)
-          if (ix[c] != -1) sr += (double)row[ix[c]];
+          if (ix[c] != -1) {
+            /* flyvec/src/cuda_funcs.cu:266-286: the fp32 product with the position's weight is what is summed */
+            float wl = row[ix[c]] * (c == mid ? lmid : lbase);
+            sr += (double)wl;
+          }
         raw[h] = (float)sr;
       }
       int best = tie_rule ? fvo_argmax_reference(raw, K) : fvo_argmax_lowest(raw, K);
@@ -248,7 +307,9 @@ void fvo_train_step_delta(float *W, int K, uint64_t N, uint64_t V, const int32_t
       double ss = 0.0;
       for (int c = 0; c < w; ++c)
         if (ix[c] != -1) {
-          float prod = row[ix[c]] * invf[(uint64_t)ix[c] % V];
+          /* flyvec/src/cuda_funcs.cu:307-327: (W * L) * 1/f, both products in fp32 */
+          float wl = row[ix[c]] * (c == mid ? lmid : lbase);
+          float prod = wl * invf[(uint64_t)ix[c] % V];
           ss += (double)prod;
         }
       win[r] = best;
@@ -264,7 +325,8 @@ void fvo_train_step_delta(float *W, int K, uint64_t N, uint64_t V, const int32_t
         double s2 = 0.0;
         for (int c = 0; c < w; ++c)
           if (ix[c] != -1) {
-            float prod = row2[ix[c]] * invf[(uint64_t)ix[c] % V];
+            float wl = row2[ix[c]] * (c == mid ? lmid : lbase);
+            float prod = wl * invf[(uint64_t)ix[c] % V];
             s2 += (double)prod;
           }
         win2[r] = second;
@@ -306,7 +368,11 @@ void fvo_train_step_delta(float *W, int K, uint64_t N, uint64_t V, const int32_t
     float *d = ds + (uint64_t)win[r] * N;
     const int32_t *ix = idx + r * (uint64_t)w;
     for (int c = 0; c < w; ++c)
-      if (ix[c] != -1) d[ix[c]] = d[ix[c]] + invf[(uint64_t)ix[c] % V];
+      if (ix[c] != -1) {
+        /* flyvec/src/cuda_funcs.cu:675-697: 1.0 * L * 1/f is a double product, rounded to fp32 by the add */
+        float add = (float)((double)(c == mid ? lmid : lbase) * (double)invf[(uint64_t)ix[c] % V]);
+        d[ix[c]] = d[ix[c]] + add;
+      }
   }
   if (delta != 0) {
     /* flyvec/src/cuda_funcs.cu:668: ds[second][idx] += -delta * 1/f. Fixed order: after every
@@ -316,7 +382,9 @@ void fvo_train_step_delta(float *W, int K, uint64_t N, uint64_t V, const int32_t
       const int32_t *ix = idx + r * (uint64_t)w;
       for (int c = 0; c < w; ++c)
         if (ix[c] != -1) {
-          float g = -delta * invf[(uint64_t)ix[c] % V];
+          /* (-delta * L) * 1/f, both products in fp32 (flyvec/src/cuda_funcs.cu:689, 693) */
+          float dl = -delta * (c == mid ? lmid : lbase);
+          float g = dl * invf[(uint64_t)ix[c] % V];
           d[ix[c]] = d[ix[c]] + g;
         }
     }
@@ -365,6 +433,15 @@ void fvo_train_step_delta(float *W, int K, uint64_t N, uint64_t V, const int32_t
   free(xx);
 }
 
+/* The step with unit position weights (Lmid = Lbase = 1, all the reference's command line reaches). */
+void fvo_train_step_delta(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx, uint64_t n, int w,
+                          const float *invf, float eps, float prec, int tie_rule, float delta, float *ds_scratch,
+                          int32_t *winners, float *sc_at_winner, int32_t *seconds, float *sc_at_second,
+                          float *xx_out, float *nc_out) {
+  fvo_train_step_weighted(W, K, N, V, idx, n, w, invf, eps, prec, tie_rule, delta, 1.0f, 1.0f, ds_scratch, winners,
+                          sc_at_winner, seconds, sc_at_second, xx_out, nc_out);
+}
+
 /* The step without the anti-Hebbian term (delta = 0, the trainer's default). */
 void fvo_train_step(float *W, int K, uint64_t N, uint64_t V, const int32_t *idx, uint64_t n, int w,
                     const float *invf, float eps, float prec, int tie_rule, float *ds_scratch,
@@ -386,10 +463,11 @@ float fvo_epoch_delta(float delta, uint64_t epoch, uint64_t n_epochs) {
  * remainder only).  winners (if given) receives the winners of every step
  * back to back.  Returns the number of windows processed.
  */
-uint64_t fvo_train_steps_delta(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
-                               const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
-                               uint64_t n_steps, int w, const float *invf, float eps, float prec,
-                               int tie_rule, float delta, int32_t *winners) {
+uint64_t fvo_train_steps_weighted(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
+                                  const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
+                                  uint64_t n_steps, int w, const float *invf, float eps, float prec,
+                                  int tie_rule, float delta, float lmid, float lbase, int prune,
+                                  int32_t *winners) {
   const uint64_t N = 2 * V;
   float *ds = (float *)malloc(sizeof(float) * (size_t)K * N);
   int32_t *idx = (int32_t *)malloc(sizeof(int32_t) * B * (uint64_t)w);
@@ -398,14 +476,25 @@ uint64_t fvo_train_steps_delta(float *W, int K, uint64_t V, const int32_t *corpu
     uint64_t k0 = first + j * B;
     if (k0 >= n_windows) break;
     uint64_t n = (k0 + B <= n_windows) ? B : n_windows - k0;
-    fvo_inflate(corpus, starts, perm, k0, n, w, V, idx);
-    fvo_train_step_delta(W, K, N, V, idx, n, w, invf, eps, prec, tie_rule, delta, ds,
-                         winners ? winners + done : NULL, NULL, NULL, NULL, NULL, NULL);
+    if (prune)
+      fvo_inflate_prune(corpus, starts, perm, k0, n, w, V, idx);
+    else
+      fvo_inflate(corpus, starts, perm, k0, n, w, V, idx);
+    fvo_train_step_weighted(W, K, N, V, idx, n, w, invf, eps, prec, tie_rule, delta, lmid, lbase, ds,
+                            winners ? winners + done : NULL, NULL, NULL, NULL, NULL, NULL);
     done += n;
   }
   free(ds);
   free(idx);
   return done;
+}
+
+uint64_t fvo_train_steps_delta(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
+                               const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
+                               uint64_t n_steps, int w, const float *invf, float eps, float prec,
+                               int tie_rule, float delta, int32_t *winners) {
+  return fvo_train_steps_weighted(W, K, V, corpus, starts, perm, n_windows, first, B, n_steps, w, invf, eps, prec,
+                                  tie_rule, delta, 1.0f, 1.0f, 0, winners);
 }
 
 uint64_t fvo_train_steps(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,

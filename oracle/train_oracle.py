@@ -68,6 +68,20 @@ def lib():
                                            C.c_int, C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_float,
                                            C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                            C.c_void_p, C.c_void_p]
+        L.fvo_train_step_weighted.restype = None
+        L.fvo_train_step_weighted.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, C.c_void_p, C.c_uint64,
+                                              C.c_int, C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_float,
+                                              C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
+                                              C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.fvo_train_steps_weighted.restype = C.c_uint64
+        L.fvo_train_steps_weighted.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                               C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_void_p,
+                                               C.c_float, C.c_float, C.c_int, C.c_float, C.c_float, C.c_float,
+                                               C.c_int, C.c_void_p]
+        L.fvo_inflate_prune.restype = None
+        L.fvo_inflate_prune.argtypes = L.fvo_inflate.argtypes
+        L.fvo_prune_windows.restype = None
+        L.fvo_prune_windows.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64]
         L.fvo_train_steps_delta.restype = C.c_uint64
         L.fvo_train_steps_delta.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p,
                                             C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_void_p,
@@ -89,6 +103,8 @@ def ref_lib():
         R.getnum_samples.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64]
         R.compute_offset_phrases.restype = None
         R.compute_offset_phrases.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64]
+        R.prune_input_data.restype = None
+        R.prune_input_data.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64]
         _ref = R
     return _ref
 
@@ -155,6 +171,32 @@ def inflate(corpus, starts, perm, first, n, w, V):
     return out
 
 
+def inflate_prune(corpus, starts, perm, first, n, w, V):
+    """inflate() with the in-window duplicate pruning of the reference's (switched-off) device kernel."""
+    corpus = np.ascontiguousarray(corpus, dtype=np.int32)
+    starts = np.ascontiguousarray(starts, dtype=np.uint64)
+    perm = np.ascontiguousarray(perm, dtype=np.uint64)
+    out = np.empty((n, w), dtype=np.int32)
+    lib().fvo_inflate_prune(_p(corpus), _p(starts), _p(perm), first, n, w, V, _p(out))
+    return out
+
+
+def prune_windows(data):
+    """The reference's host tool prune_input_data on a copy of an int32 (rows, cols) window matrix."""
+    out = np.array(data, dtype=np.int32, order="C", copy=True)
+    rows, cols = out.shape
+    lib().fvo_prune_windows(_p(out), rows, cols)
+    return out
+
+
+def ref_prune_windows(data):
+    """The same through the reference's own prune_input.cpp (oracle/_ref)."""
+    out = np.array(data, dtype=np.int32, order="C", copy=True)
+    rows, cols = out.shape
+    ref_lib().prune_input_data(_p(out), rows, cols)
+    return out
+
+
 def activations(W, idx, invf):
     W = np.ascontiguousarray(W, dtype=np.float32)
     idx = np.ascontiguousarray(idx, dtype=np.int32)
@@ -195,9 +237,10 @@ def epoch_delta(delta, epoch, n_epochs):
     return float(lib().fvo_epoch_delta(delta, epoch, n_epochs))
 
 
-def train_step(W, idx, invf, eps, prec=1e-30, tie_rule=0, delta=0.0):
+def train_step(W, idx, invf, eps, prec=1e-30, tie_rule=0, delta=0.0, lmid=1.0, lbase=1.0):
     """In-place step on W (K, 2V) fp32 C-order.  Returns dict(winners, sc, seconds, sc2, xx, nc, ds);
-    delta is the anti-Hebbian strength of the step (0 = none)."""
+    delta is the anti-Hebbian strength of the step (0 = none), lmid / lbase weigh the centre and the
+    context positions of a window (1 = the reference's command line)."""
     assert W.dtype == np.float32 and W.flags.c_contiguous
     idx = np.ascontiguousarray(idx, dtype=np.int32)
     invf = np.ascontiguousarray(invf, dtype=np.float32)
@@ -210,12 +253,13 @@ def train_step(W, idx, invf, eps, prec=1e-30, tie_rule=0, delta=0.0):
     nc = np.zeros(1, dtype=np.float32)
     win2 = np.empty(n, dtype=np.int32)
     sc2 = np.empty(n, dtype=np.float32)
-    lib().fvo_train_step_delta(_p(W), K, N, len(invf), _p(idx), n, w, _p(invf), eps, prec, tie_rule, delta,
-                               _p(ds), _p(win), _p(sc), _p(win2), _p(sc2), _p(xx), _p(nc))
+    lib().fvo_train_step_weighted(_p(W), K, N, len(invf), _p(idx), n, w, _p(invf), eps, prec, tie_rule, delta,
+                                  lmid, lbase, _p(ds), _p(win), _p(sc), _p(win2), _p(sc2), _p(xx), _p(nc))
     return dict(winners=win, sc=sc, seconds=win2, sc2=sc2, xx=xx, nc=float(nc[0]), ds=ds)
 
 
-def train_steps(W, corpus, starts, perm, first, B, n_steps, w, invf, eps, prec=1e-30, tie_rule=0, delta=0.0):
+def train_steps(W, corpus, starts, perm, first, B, n_steps, w, invf, eps, prec=1e-30, tie_rule=0, delta=0.0,
+                lmid=1.0, lbase=1.0, prune=False):
     """In-place n_steps minibatches; returns the winners of all processed windows."""
     assert W.dtype == np.float32 and W.flags.c_contiguous
     corpus = np.ascontiguousarray(corpus, dtype=np.int32)
@@ -227,6 +271,7 @@ def train_steps(W, corpus, starts, perm, first, B, n_steps, w, invf, eps, prec=1
     nwin = len(perm)
     cap = max(0, min(n_steps * B, nwin - first))
     win = np.empty(cap, dtype=np.int32)
-    done = lib().fvo_train_steps_delta(_p(W), K, V, _p(corpus), _p(starts), _p(perm), nwin, first, B, n_steps,
-                                       w, _p(invf), eps, prec, tie_rule, delta, _p(win))
+    done = lib().fvo_train_steps_weighted(_p(W), K, V, _p(corpus), _p(starts), _p(perm), nwin, first, B, n_steps,
+                                          w, _p(invf), eps, prec, tie_rule, delta, lmid, lbase, int(bool(prune)),
+                                          _p(win))
     return win[:done]

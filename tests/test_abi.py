@@ -42,9 +42,10 @@ def test_python_binding_covers_the_header():
 
 def test_struct_layout_matches_the_header():
     from flyvec_amd._lib import TrainConfig
-    # uint64 + 4 x uint32 + 3 x float + uint32 = 40 bytes, no padding
-    assert C.sizeof(TrainConfig) == 40
+    # uint64 + 4 x uint32 + 5 x float + uint32 = 48 bytes, no padding
+    assert C.sizeof(TrainConfig) == 48
     assert TrainConfig.vocab.offset == 0 and TrainConfig.hid.offset == 8 and TrainConfig.prec.offset == 32
+    assert TrainConfig.lmid.offset == 36 and TrainConfig.lbase.offset == 40 and TrainConfig.prune_duplicates.offset == 44
 
 
 def test_argument_errors_need_no_device():
@@ -54,12 +55,18 @@ def test_argument_errors_need_no_device():
     assert lib.fv_trainer_create(None, C.byref(out)) == _lib.FV_ERR_INVALID
     assert b"null" in lib.fv_last_error()
     cfg = _lib.TrainConfig(vocab=10, hid=4000, window=11, batch=10, tie_rule=0, initial_learning_rate=1e-3,
-                           delta=0.0, prec=1e-30, reserved=0)
+                           delta=0.0, prec=1e-30, lmid=1.0, lbase=1.0, prune_duplicates=0)
     assert lib.fv_trainer_create(C.byref(cfg), C.byref(out)) == _lib.FV_ERR_INVALID
     assert b"hid" in lib.fv_last_error()
     cfg.hid, cfg.delta = 400, float("nan")
     assert lib.fv_trainer_create(C.byref(cfg), C.byref(out)) == _lib.FV_ERR_INVALID
     assert b"delta" in lib.fv_last_error()
+    cfg.delta, cfg.lmid = 0.0, float("nan")
+    assert lib.fv_trainer_create(C.byref(cfg), C.byref(out)) == _lib.FV_ERR_INVALID
+    assert b"Lmid" in lib.fv_last_error()
+    cfg.lmid, cfg.prune_duplicates = 1.0, 2
+    assert lib.fv_trainer_create(C.byref(cfg), C.byref(out)) == _lib.FV_ERR_INVALID
+    assert b"prune_duplicates" in lib.fv_last_error()
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -60,3 +60,27 @@ def test_shards_to_checkpoint(gpu, tmp_path):
     assert W.shape == (32, 2 * V) and np.isfinite(W).all()
     # masked ids never enter a window: their context and target columns keep their initial spread
     assert np.abs(W[:, stop]).max() < 0.2
+
+
+def test_prune_windows_equals_the_checker_and_the_reference_tool(gpu, oracle_lib):
+    """fv_prune_windows against the CPU restatement, which tests/test_oracle_train.py holds against the
+    reference's own prune_input_data; here also directly against that build where it travelled."""
+    from flyvec_amd import _lib, corpus
+    to = oracle_lib
+    rng = np.random.default_rng(0)
+    for rows, cols, hi in [(1, 1, 3), (7, 2, 2), (1000, 3, 4), (5000, 11, 8), (300, 16, 5), (257, 64, 30), (4, 11, 1)]:
+        data = rng.integers(-1, hi, size=(rows, cols)).astype(np.int32)
+        want = to.prune_windows(data)
+        got = corpus.prune_windows(data.copy())
+        assert np.array_equal(got, want), (rows, cols)
+        if to.ref_lib() is not None:
+            assert np.array_equal(got, to.ref_prune_windows(data)), (rows, cols)
+        assert np.array_equal(corpus.prune_windows(got.copy()), got)          # idempotent
+        assert np.array_equal(got[:, cols // 2], data[:, cols // 2])           # the centre is never touched
+    empty = np.zeros((0, 11), dtype=np.int32)
+    assert corpus.prune_windows(empty).shape == (0, 11)
+    with pytest.raises(_lib.FlyvecError) as e:
+        corpus.prune_windows(np.zeros((2, 65), dtype=np.int32))
+    assert e.value.code == _lib.FV_ERR_INVALID
+    with pytest.raises(ValueError):
+        corpus.prune_windows(np.zeros((2, 3), dtype=np.int64))

@@ -568,3 +568,95 @@ def test_delta_epoch_schedule_and_driver(gpu, oracle_lib):
     with pytest.raises(Exception):
         t.second_winners(B)                  # and has no second neurons to show
     t.close()
+
+
+# ---- position weights (Lmid, Lbase) and in-window duplicate pruning --------------------------------------
+
+def run_both_variant(to, V, K, w, B, steps, delta=0.0, lmid=1.0, lbase=1.0, prune=False, tie=0, launches=0,
+                     n_tokens=60000, sigma=0.02, seed=0, vocab_for_tokens=None):
+    """Steps with the rule's dormant variants switched on, against the checker step by step."""
+    from flyvec_amd import Trainer, synthetic
+    # pruning only matters when tokens repeat inside a window: draw them from a small vocabulary then
+    tokens, offsets = small_corpus(n_tokens, vocab_for_tokens or V, seed=seed)
+    tokens[-1] = V - 1
+    W0 = synthetic.synapses(K, V, seed=5 + seed, sigma=sigma)
+    t = Trainer(V, K, w, B, initial_learning_rate=2e-4, tie_rule=tie, lmid=lmid, lbase=lbase, prune_duplicates=prune)
+    t.set_dense_launches(launches)
+    t.set_corpus(tokens, offsets)
+    perm = np.random.default_rng(6).permutation(t.num_windows).astype(np.uint64)
+    t.set_permutation(perm)
+    t.set_weights(W0)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    eps = t.epoch_eps(0, 15)
+    steps = min(steps, t.num_windows // B)
+    Wo = W0.copy()
+    inflate = to.inflate_prune if prune else to.inflate
+    for s in range(steps):
+        t.step(s * B, B, eps, delta=delta)
+        idx = inflate(tokens, starts, perm, s * B, B, w, V)
+        ref = to.train_step(Wo, idx, invf, eps, tie_rule=tie, delta=delta, lmid=lmid, lbase=lbase)
+        assert np.array_equal(t.winners(B), ref["winners"]), f"winners, step {s}"
+        if delta:
+            assert np.array_equal(t.second_winners(B), ref["seconds"]), f"second neurons, step {s}"
+        xx, nc = t.step_stats()
+        assert np.array_equal(xx, ref["xx"]) and nc == ref["nc"], f"xx / max|ds|, step {s}"
+    Wg = t.get_weights()
+    t.close()
+    return Wg, Wo
+
+
+@pytest.mark.parametrize("launches", [1, 2])
+@pytest.mark.parametrize("lmid,lbase,delta", [(2.5, 0.75, 0.0), (0.3, 1.0, 0.0), (1.0, 3.0, 0.4), (0.0, 1.0, 0.0),
+                                              (1.0, 0.0, 0.4), (-1.5, 0.5, 0.0)])
+def test_position_weights_bit_exact(gpu, oracle_lib, lmid, lbase, delta, launches):
+    Wg, Wo = run_both_variant(oracle_lib, V=500, K=400, w=11, B=512, steps=6, delta=delta, lmid=lmid, lbase=lbase,
+                              launches=launches)
+    assert np.array_equal(Wg, Wo)
+
+
+@pytest.mark.parametrize("K,w,V,B,tie", [(1, 1, 5, 1, 0), (3, 2, 7, 3, 1), (65, 15, 200, 256, 0), (130, 64, 300, 64, 1),
+                                         (1000, 4, 300, 512, 0), (30, 11, 30000, 700, 0)])
+def test_position_weights_shapes(gpu, oracle_lib, K, w, V, B, tie):
+    n_tokens = 40000 if V < 20000 else 120000
+    Wg, Wo = run_both_variant(oracle_lib, V=V, K=K, w=w, B=B, steps=4, delta=0.25, lmid=1.75, lbase=0.6, tie=tie,
+                              n_tokens=n_tokens)
+    assert np.array_equal(Wg, Wo)
+
+
+def test_unit_weights_take_the_unweighted_kernels(gpu, oracle_lib):
+    # Lmid = Lbase = 1 is the default path: same bits as a trainer created without the fields
+    Wa, Wo = run_both_variant(oracle_lib, V=300, K=64, w=7, B=128, steps=5)
+    Wb = run_both(gpu, oracle_lib, V=300, K=64, w=7, B=128, steps=5, n_tokens=60000)[2]
+    assert np.array_equal(Wa, Wo) and np.array_equal(Wa, Wb)
+
+
+@pytest.mark.parametrize("launches", [1, 2])
+@pytest.mark.parametrize("w,small_vocab", [(11, 12), (7, 5), (64, 40), (2, 3), (1, 4)])
+def test_duplicate_pruning_bit_exact(gpu, oracle_lib, w, small_vocab, launches):
+    # tokens drawn from a handful of ids, so most windows hold repeats; V stays larger (unused columns)
+    Wg, Wo = run_both_variant(oracle_lib, V=300, K=96, w=w, B=256, steps=6, prune=True, vocab_for_tokens=small_vocab,
+                              launches=launches, delta=0.2 if w == 7 else 0.0)
+    assert np.array_equal(Wg, Wo)
+
+
+def test_duplicate_pruning_with_weights_and_epoch_driver(gpu, oracle_lib):
+    """Everything at once through run_epoch: pruning, weights, the anti-Hebbian schedule, a partial last batch."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    V, K, w, B = 200, 96, 11, 300
+    tokens, offsets = small_corpus(9000, 25, n_masked=10)
+    tokens[-1] = V - 1
+    W0 = synthetic.synapses(K, V, sigma=0.02)
+    t = Trainer(V, K, w, B, initial_learning_rate=2e-4, delta=0.3, lmid=1.5, lbase=0.8, prune_duplicates=True)
+    t.set_corpus(tokens, offsets)
+    perm = np.random.default_rng(6).permutation(t.num_windows).astype(np.uint64)
+    t.set_permutation(perm)
+    t.set_weights(W0)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    t.run_epoch(3, 15)
+    eps, delta = t.epoch_eps(3, 15), t.epoch_delta(3, 15)
+    Wo = W0.copy()
+    n_steps = (t.num_windows + B - 1) // B
+    to.train_steps(Wo, tokens, starts, perm, 0, B, n_steps, w, invf, eps, delta=delta, lmid=1.5, lbase=0.8, prune=True)
+    assert np.array_equal(t.get_weights(), Wo)
+    t.close()

@@ -27,23 +27,25 @@ def brute_argmax_lowest(raw):
     return best
 
 
-def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest, delta=0.0):
+def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest, delta=0.0, lmid=1.0, lbase=1.0):
     """flyvec/src/cuda_funcs.cu:1662-1803 (sparse, frequency scaling) in Python scalars. With
     delta != 0 the second neuron of every window (the search repeated with the winner's activation
     overwritten by -9999.9999, :495-548) receives the anti-Hebbian terms (:668, :726-734); their
-    place in the order of additions: after the Hebbian ones."""
+    place in the order of additions: after the Hebbian ones. lmid / lbase weigh the centre position and
+    the others (:266-286, :307-327, :675-697)."""
     W = W.copy()
     K, N = W.shape
     V = N // 2
     n, w = idx.shape
     delta = f32(delta)
+    L = [f32(lmid) if c == w // 2 else f32(lbase) for c in range(w)]
 
     def scaled(h, r):
         ss = 0.0
         for c in range(w):
             i = idx[r, c]
             if i != -1:
-                ss += float(f32(W[h, i] * invf[i % V]))  # fp32 product, double sum
+                ss += float(f32(f32(W[h, i] * L[c]) * invf[i % V]))  # fp32 products, double sum
         return f32(ss)
 
     win, sc, win2, sc2 = [], [], [], []
@@ -54,7 +56,7 @@ def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest, delta=0.0):
             for c in range(w):
                 i = idx[r, c]
                 if i != -1:
-                    s += float(W[h, i])
+                    s += float(f32(W[h, i] * L[c]))
             raw.append(f32(s))
         b = argmax(raw)
         win.append(b)
@@ -81,13 +83,13 @@ def brute_step(W, idx, invf, eps, prec, argmax=brute_argmax_lowest, delta=0.0):
         for c in range(w):
             i = idx[r, c]
             if i != -1:
-                ds[win[r], i] = f32(ds[win[r], i] + invf[i % V])
+                ds[win[r], i] = f32(ds[win[r], i] + f32(float(L[c]) * float(invf[i % V])))  # double product
     if delta != 0:
         for r in range(n):
             for c in range(w):
                 i = idx[r, c]
                 if i != -1:
-                    ds[win2[r], i] = f32(ds[win2[r], i] + f32(-delta * invf[i % V]))
+                    ds[win2[r], i] = f32(ds[win2[r], i] + f32(f32(-delta * L[c]) * invf[i % V]))
     nc = f32(0)
     for h in range(K):
         if xx[h] != 0:
@@ -448,3 +450,148 @@ def test_epoch_delta_schedule():
     for delta, ep, nep in [(0.4, 0, 15), (0.4, 7, 15), (0.4, 14, 15), (1.0, 100, 200), (0.0, 3, 15)]:
         want = f32(float(f32(delta)) * 0.5 * (1.0 + math.tanh((float(f32(ep)) - 0.125 * nep) / 10.0)))
         assert to.epoch_delta(delta, ep, nep) == want
+
+
+# ---- position weights Lmid / Lbase -------------------------------------------------------------------
+
+@pytest.mark.parametrize("seed", range(8))
+def test_weighted_step_against_brute_force(seed):
+    rng = np.random.default_rng(300 + seed)
+    K, V, w, n = int(rng.integers(1, 5)), int(rng.integers(3, 7)), int(rng.choice([1, 3, 4])), int(rng.integers(1, 9))
+    W = rng.standard_normal((K, 2 * V)).astype(f32)
+    idx = rng.integers(0, V, size=(n, w)).astype(np.int32)
+    idx[:, w // 2] += V
+    idx[rng.random((n, w)) < 0.15] = -1
+    invf = (1.0 / rng.integers(1, 50, size=V)).astype(f32)
+    delta = 0.0 if seed % 2 == 0 else 0.3
+    lmid, lbase = float(f32(rng.uniform(0.2, 3.0))), float(f32(rng.uniform(0.2, 3.0)))
+    want = brute_step(W, idx, invf, 2e-2, 1e-30, delta=delta, lmid=lmid, lbase=lbase)
+    got_W = W.copy()
+    res = to.train_step(got_W, idx, invf, 2e-2, 1e-30, tie_rule=0, delta=delta, lmid=lmid, lbase=lbase)
+    assert np.array_equal(res["winners"], want[1])
+    assert np.array_equal(res["xx"], want[2]) and res["nc"] == want[3]
+    assert np.array_equal(got_W, want[0])
+    if delta:
+        assert np.array_equal(res["seconds"], want[4])
+
+
+def test_unit_weights_are_the_plain_step_and_a_power_of_two_changes_nothing():
+    W, idx, invf = setup_small(3)
+    Wa, Wb, Wc = W.copy(), W.copy(), W.copy()
+    ra = to.train_step(Wa, idx, invf, 1e-3, delta=0.2)
+    rb = to.train_step(Wb, idx, invf, 1e-3, delta=0.2, lmid=1.0, lbase=1.0)
+    assert np.array_equal(Wa, Wb) and np.array_equal(ra["xx"], rb["xx"])
+    # Lmid = Lbase = 4: activations, xx and ds are all 4x (exactly: a power of two), max|ds| is 4x, the
+    # scale eps / max|ds| is a quarter: the same update bit for bit
+    rc = to.train_step(Wc, idx, invf, 1e-3, delta=0.2, lmid=4.0, lbase=4.0)
+    assert np.array_equal(rc["winners"], ra["winners"]) and np.array_equal(rc["seconds"], ra["seconds"])
+    assert np.array_equal(rc["xx"], ra["xx"] * f32(4)) and rc["nc"] == ra["nc"] * 4
+    assert np.array_equal(Wc, Wa)
+
+
+def test_a_zero_weight_is_a_masked_position():
+    """Lmid = 0 removes the centre from both activations and adds 0 to ds there: the step on the same
+    windows with the centre masked (-1).  Lbase = 0: the step with every context position masked."""
+    W, idx, invf = setup_small(7, n=6)
+    w = idx.shape[1]
+    mid = w // 2
+    for lmid, lbase in [(0.0, 1.0), (1.0, 0.0)]:
+        masked = idx.copy()
+        if lmid == 0.0:
+            masked[:, mid] = -1
+        else:
+            keep = masked[:, mid].copy()
+            masked[:] = -1
+            masked[:, mid] = keep
+        Wa, Wb = W.copy(), W.copy()
+        ra = to.train_step(Wa, idx, invf, 1e-3, lmid=lmid, lbase=lbase)
+        rb = to.train_step(Wb, masked, invf, 1e-3)
+        assert np.array_equal(ra["winners"], rb["winners"])
+        assert np.array_equal(ra["xx"], rb["xx"]) and ra["nc"] == rb["nc"]
+        assert np.array_equal(Wa, Wb)
+
+
+def test_weights_reach_the_centre_and_the_context_separately():
+    """One window: the winner is the argmax of Lmid * W[:, centre] + Lbase * sum of W[:, context];
+    weights chosen so that the winner differs between (Lmid, Lbase) = (8, 1) and (1, 8)."""
+    K, V = 2, 4
+    W = np.zeros((K, 2 * V), dtype=f32)
+    idx = np.array([[0, V + 1, 2]], dtype=np.int32)       # context 0, centre 1 (target block), context 2
+    W[0, V + 1] = 1.0                                     # neuron 0 likes the centre token
+    W[1, 0] = 0.75; W[1, 2] = 0.75                        # neuron 1 likes the context
+    invf = np.full(V, 0.5, dtype=f32)
+    for lmid, lbase, want in [(8.0, 1.0, 0), (1.0, 8.0, 1), (1.0, 1.0, 1)]:
+        Wc = W.copy()
+        res = to.train_step(Wc, idx, invf, 1e-3, lmid=lmid, lbase=lbase)
+        assert int(res["winners"][0]) == want
+        raw = lmid * W[:, V + 1] + lbase * (W[:, 0] + W[:, 2])
+        assert want == int(np.argmax(raw))
+        # the sparse term of the winner's row: L * 1/f per position, on top of -xx * W
+        h = want
+        ds = f32(-res["xx"][h]) * W[h]
+        for c, i in enumerate(idx[0]):
+            ds[i] = f32(ds[i] + f32((lmid if c == 1 else lbase) * 0.5))
+        assert np.array_equal(res["ds"][h], ds)
+
+
+# ---- in-window duplicate pruning ---------------------------------------------------------------------
+
+def first_occurrence_mask(tokens_row, include_centre, mid):
+    """True where a position holds a token that no EARLIER position holds (the centre counted among the
+    earlier ones or not), written with sets, not with the reference's nested scan."""
+    seen, keep = set(), []
+    for c, t in enumerate(tokens_row):
+        keep.append(t not in seen)
+        if c != mid or include_centre:
+            seen.add(t)
+    return keep
+
+
+def test_prune_windows_matches_the_reference_tool():
+    """fvo_prune_windows against the reference's own prune_input_data (compiled into oracle/_ref)."""
+    if to.ref_lib() is None:
+        pytest.skip("oracle/_ref not built")
+    rng = np.random.default_rng(0)
+    for cols in (1, 2, 3, 4, 11, 16):
+        data = rng.integers(-1, 6, size=(200, cols)).astype(np.int32)
+        assert np.array_equal(to.prune_windows(data), to.ref_prune_windows(data)), cols
+    data = rng.integers(0, 3, size=(50, 11)).astype(np.int32)     # many duplicates
+    assert np.array_equal(to.prune_windows(data), to.ref_prune_windows(data))
+
+
+def test_prune_windows_keeps_first_occurrences():
+    rng = np.random.default_rng(1)
+    for cols in (1, 5, 11):
+        data = rng.integers(0, 7, size=(100, cols)).astype(np.int32)
+        out = to.prune_windows(data)
+        mid = cols // 2
+        for row, got in zip(data, out):
+            keep = first_occurrence_mask(row.tolist(), False, mid)
+            want = [t if (k or c == mid) else -1 for c, (t, k) in enumerate(zip(row.tolist(), keep))]
+            assert got.tolist() == want
+
+
+def test_inflate_prune_keeps_first_occurrences_and_the_centre():
+    rng = np.random.default_rng(2)
+    V, w = 6, 7
+    corpus = rng.integers(0, V, size=400).astype(np.int32)
+    corpus[rng.random(400) < 0.1] = -1
+    starts = np.arange(0, 400 - w, dtype=np.uint64)
+    perm = rng.permutation(len(starts)).astype(np.uint64)
+    got = to.inflate_prune(corpus, starts, perm, 3, 200, w, V)
+    plain = to.inflate(corpus, starts, perm, 3, 200, w, V)
+    mid = w // 2
+    for r in range(200):
+        row = corpus[int(starts[perm[3 + r]]):][:w].tolist()
+        keep = first_occurrence_mask(row, True, mid)
+        for c in range(w):
+            if c == mid:
+                assert got[r, c] == plain[r, c]                   # the centre always survives
+            elif row[c] != -1 and keep[c]:
+                assert got[r, c] == plain[r, c]
+            else:
+                assert got[r, c] == -1
+    # a window without repeated tokens is untouched
+    corpus2 = np.arange(50, dtype=np.int32) % 40
+    st2 = np.arange(0, 30, dtype=np.uint64)
+    assert np.array_equal(to.inflate_prune(corpus2, st2, st2, 0, 30, w, 40), to.inflate(corpus2, st2, st2, 0, 30, w, 40))
