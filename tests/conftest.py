@@ -30,6 +30,15 @@ def gpu():
     return _lib
 
 
+@pytest.fixture(autouse=True)
+def _no_trainer_left_over():
+    """A trainer that an earlier test left to the garbage collector (inside an exception's traceback, say)
+    still counts as alive in the library, and a second live trainer switches the single dense launch off."""
+    import gc
+    gc.collect()
+    yield
+
+
 @pytest.fixture(scope="session")
 def oracle_lib():
     from oracle import train_oracle
