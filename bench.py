@@ -47,15 +47,15 @@ HASH = dict(K=400, V=20000, w=11, k=32, n=1 << 20)
 # WRITE_SIZE reads them all: x1.0). Traffic below the algorithmic bytes means the rest was served
 # by the L2 caches.
 MEASURED_TRAFFIC = {
-    "dense_max_update": (33332.5 * 2.0 + 65230.9) * 1024,
-    "gather_winner": (26344.4 * 2.0 + 492.9) * 1024,
-    "sparse_owners": (4573.3 * 2.0 + 2483.8) * 1024,
-    "group_xx": (307.0 * 2.0 + 87.2) * 1024,
-    "hash": (2245564.2 * 2.0 + 78866.2) * 1024,
+    "dense_max_update": (33304.9 * 2.0 + 65234.4) * 1024,
+    "gather_winner": (26321.3 * 2.0 + 498.2) * 1024,
+    "sparse_owners": (4568.2 * 2.0 + 2483.7) * 1024,
+    "group_xx": (305.5 * 2.0 + 87.2) * 1024,
+    "hash": (2245027.6 * 2.0 + 79242.7) * 1024,
     # the passes over W as two launches and the slot launch (--dense-launches 2)
-    "update": (32326.6 * 2.0 + 62498.2) * 1024,
-    "absmax_ds": (31275.5 * 2.0 + 64.0) * 1024,
-    "slot_update": (621.0 * 2.0 + 1501.2) * 1024,
+    "update": (32354.2 * 2.0 + 62498.2) * 1024,
+    "absmax_ds": (31270.0 * 2.0 + 64.0) * 1024,
+    "slot_update": (622.6 * 2.0 + 1501.2) * 1024,
 }
 
 

@@ -1,27 +1,28 @@
 // The FlyVec training minibatch step on one MI355X.
 //
 // Replaces the kernel chain of flyvec/src/cuda_funcs.cu:1662-1803 (sparse input, frequency
-// scaling, Lmid = Lbase = 1, delta = 0, p = 2).  The reference materialises ds (K x N) and
-// walks it five times per step; here ds is never stored and nothing uses global atomics:
+// scaling, p = 2; delta, Lmid / Lbase and the pruning sampler included).  The reference
+// materialises ds (K x N) and walks it five times per step; here ds is never stored and nothing
+// uses global atomics:
 //
 //   1. gather+winner   one wavefront per window: sampler (cuda_funcs.cu:915-936), raw
 //                      activation = sum of ~w token rows of the token-major matrix with the K
 //                      neurons spread over lanes (:248-263, double accumulators, one rounding),
 //                      argmax by a wave reduction (:488-561) and the winner's frequency-scaled
 //                      activation (:289-305; it is only ever read at the winner, :731).
-//   2. neuron owners   one block per neuron h: the ordered list of windows h won; xx[h] = sum of
-//                      their scaled activations in window order (:722-744 -- the reference's
-//                      atomic order is undefined, this one is fixed, so a step is reproducible
-//                      bit for bit); then the sparse Hebbian term of row h (:657-672): the block
-//                      alone owns elements (h, token), so it counts repeated tokens in LDS, and
-//                      for each distinct token saves the true weight and the count in a slot
-//                      record, evaluates ds there, and plants a sentinel in W.
-//   3. max|ds|         dense pass: ds = -xx[h] * W (:394-406), sentinel elements skipped; block
-//                      maxima (cu_special_reduction.cu:26-99, 153-189).
-//   4. update          W += s * ds where |s * ds| > 1e-10, s = eps / max(prec, max|ds|), rows
-//                      with xx == 0 untouched (cuda_funcs.cu:1797-1799,
-//                      cu_special_reduction.cu:316-354); dense blocks leave sentinels alone,
-//                      slot blocks of the same launch write the final value over each sentinel.
+//   2. group + xx      one block per neuron h: the ordered list of the windows h won and xx[h], the
+//                      sum of their scaled activations (:722-744 -- the reference's atomic order
+//                      is undefined, this one is fixed, so a step is reproducible bit for bit).
+//   3. sparse owners   four blocks per neuron, one per column class: the sparse Hebbian term of
+//                      row h (:657-672). A block alone owns its elements (h, column), so it counts
+//                      repeated columns in LDS and for each distinct one saves the true weight and
+//                      the count in a slot record, evaluates ds there, and plants a sentinel in W.
+//   4. dense passes    max|ds| with ds = -xx[h] * W (:394-406; cu_special_reduction.cu:26-99,
+//                      153-189), then W += s * ds where |s * ds| > 1e-10, s = eps / max(prec,
+//                      max|ds|) (cuda_funcs.cu:1797-1803, cu_special_reduction.cu:316-354), then the
+//                      final value of every sparse element over its sentinel. One launch that keeps
+//                      W in registers between the passes when the matrix fits the register file of
+//                      the machine, otherwise three launches (4a max, 5 update, 6 slot update).
 //
 // Every one of the n additions of 1/f onto ds[h][i] adds the same value, so the reference's
 // result for that element depends only on n; replaying n sequential fp32 adds reproduces it
@@ -816,7 +817,7 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
   }
 }
 
-// ---- kernels 3 and 4: dense passes over the matrix ------------------------------------------------
+// ---- kernel 4: dense passes over the matrix (one launch, or 4a + 5 + 6) ---------------------------
 
 struct fv_dense_args {
   float4 *Wt4;
@@ -903,7 +904,7 @@ __device__ __forceinline__ void fv_dense_load(const fv_dense_args &a, uint32_t p
   for (int u = 0; u < U; ++u) w[u] = a.Wt4[p4 + u * stride < a.total4 ? p4 + u * stride : inside];
 }
 
-// Kernel 4: block maxima of |ds| over the dense elements. A thread's first loads of W
+// Kernel 4a: block maxima of |ds| over the dense elements. A thread's first loads of W
 // are issued before the block stages xx in LDS.
 __global__ __launch_bounds__(256) void fv_absmax_kernel(fv_dense_args a) {
   extern __shared__ float4 xs4[];  // xx, ldk4 float4
