@@ -1037,6 +1037,9 @@ __device__ __forceinline__ void fv_update_four_around(const fv_dense_args &a, ui
   if (w.w == w.w) e[3] = w.w;
 }
 
+static_assert(FV_MAX_HID <= 2 * FV_ONEPASS_THREADS, "two first-window words per thread cover every neuron");
+static_assert(FV_MAX_HID * FV_NB_CLASSES <= 8 * FV_ONEPASS_THREADS, "eight record counts per thread cover every block");
+
 // P: counts of the sparse launch's blocks a thread sums (FV_NB_CLASSES * K <= P * FV_ONEPASS_THREADS)
 template <int U, int P, bool DELTA>
 __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv_dense_args a) {
