@@ -58,6 +58,15 @@ MEASURED_TRAFFIC = {
     "slot_update": (622.6 * 2.0 + 1501.2) * 1024,
 }
 
+# the same for --workload large-step (profiles/train_step_K1000_V50000_B50000.txt)
+MEASURED_TRAFFIC_LARGE = {
+    "gather_winner": (742880.9 * 2.0 + 4485.2) * 1024,
+    "group_xx": (1244.3 * 2.0 + 316.0) * 1024,
+    "sparse_owners": (32999.4 * 2.0 + 18011.6) * 1024,
+    "absmax_ds": (195342.3 * 2.0 + 67.9) * 1024,
+    "update": (195628.1 * 2.0 + 390612.5) * 1024,
+    "slot_update": (3551.4 * 2.0 + 11373.0) * 1024,
+}
 
 # the two passes over W of a step (and the sparse elements' update) as one launch: W stays in
 # registers between them, so the launch moves 8*K*N bytes of W while the byte model of the step
@@ -137,7 +146,7 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0):
         "kernel_ms": kern_ms,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK,
-                     "traffic": MEASURED_TRAFFIC.get(dom) if c is TRAIN else None,
+                     "traffic": (MEASURED_TRAFFIC if c is TRAIN else MEASURED_TRAFFIC_LARGE).get(dom),
                      "algorithmic_bytes": per_kernel[dom]},
         "dense_launches": launches,
         "step_roofline_frac": (step_bytes / HBM_PEAK) / (ms_per_step * 1e-3),
