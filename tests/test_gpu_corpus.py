@@ -84,3 +84,12 @@ def test_prune_windows_equals_the_checker_and_the_reference_tool(gpu, oracle_lib
     assert e.value.code == _lib.FV_ERR_INVALID
     with pytest.raises(ValueError):
         corpus.prune_windows(np.zeros((2, 3), dtype=np.int64))
+
+
+def test_prune_windows_golden_fixture(gpu):
+    """The reference's own prune_input_data output (tests/golden/prune_windows.npz) through the C ABI."""
+    import os
+    from flyvec_amd import corpus
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "prune_windows.npz"))
+    for k in range(int(z["n_cases"])):
+        assert np.array_equal(corpus.prune_windows(z[f"in_{k}"].copy()), z[f"out_{k}"]), k

@@ -559,6 +559,16 @@ def test_prune_windows_matches_the_reference_tool():
     assert np.array_equal(to.prune_windows(data), to.ref_prune_windows(data))
 
 
+def test_prune_windows_golden_fixture_from_reference_build():
+    """tests/golden/prune_windows.npz was written by tests/golden/make_prune_windows.py from the reference's own
+    prune_input_data; it travels to machines where neither the reference nor its build is present."""
+    import os
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "prune_windows.npz"))
+    for k in range(int(z["n_cases"])):
+        assert np.array_equal(to.prune_windows(z[f"in_{k}"]), z[f"out_{k}"]), k
+    assert z["out_7"].tolist() == [[7, -1, 7, -1, -1], [1, 2, 1, -1, -1], [-1, 3, -1, -1, -1], [4, 5, 6, -1, -1]]
+
+
 def test_prune_windows_keeps_first_occurrences():
     rng = np.random.default_rng(1)
     for cols in (1, 5, 11):
