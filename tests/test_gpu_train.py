@@ -660,3 +660,26 @@ def test_duplicate_pruning_with_weights_and_epoch_driver(gpu, oracle_lib):
     to.train_steps(Wo, tokens, starts, perm, 0, B, n_steps, w, invf, eps, delta=delta, lmid=1.5, lbase=0.8, prune=True)
     assert np.array_equal(t.get_weights(), Wo)
     t.close()
+
+
+def test_dense_launch_forms_agree_over_an_epoch_of_the_headline_shape(gpu):
+    """K = 400, V = 20000, w = 11, B = 10000: 1200 steps through run_epoch as one dense launch per step and as
+    three; every block exchange, slot record and ahead-sampled minibatch of the single launch has to
+    come out right for the two matrices to be equal bit for bit."""
+    from flyvec_amd import Trainer, synthetic
+    V, K, w, B = 20000, 400, 11, 10000
+    tokens, offsets = synthetic.corpus(18_000_000, V)
+    W0 = synthetic.synapses(K, V, seed=5)
+    got = {}
+    for launches in (1, 2):
+        t = Trainer(V, K, w, B, initial_learning_rate=2e-4)
+        t.set_dense_launches(launches)
+        t.set_corpus(tokens, offsets)
+        assert t.num_windows // B >= 1100
+        t.set_weights(W0)
+        t.shuffle(11)
+        t.run_epoch(0, 15)
+        got[launches] = t.get_weights()
+        t.close()
+    assert np.isfinite(got[1]).all() and not np.array_equal(got[1], W0)
+    assert np.array_equal(got[1], got[2])
