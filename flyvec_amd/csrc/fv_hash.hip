@@ -178,7 +178,10 @@ extern "C" int fv_hasher_create(const float *W, uint32_t hid, uint64_t n_columns
   hipError_t e = hipSuccess;
   if (rc == FV_OK) {
     e = hipStreamCreate(&h->stream);
-    if (e == hipSuccess) e = hipMalloc((void **)&h->Wt, (size_t)h->N * h->ldk * sizeof(float));
+    // the rows behind the matrix that the gather reads for masked positions and past K: zeros
+    if (e == hipSuccess) e = hipMalloc((void **)&h->Wt, (size_t)(h->N + FV_PAD_ROWS) * h->ldk * sizeof(float));
+    if (e == hipSuccess)
+      e = hipMemsetAsync(h->Wt + (size_t)h->N * h->ldk, 0, (size_t)FV_PAD_ROWS * h->ldk * sizeof(float), h->stream);
     if (e == hipSuccess) e = hipMalloc((void **)&h->err, sizeof(uint32_t));
     if (e == hipSuccess) e = hipMemsetAsync(h->err, 0, sizeof(uint32_t), h->stream);
     if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "hasher allocation failed: %s", hipGetErrorString(e));

@@ -137,39 +137,36 @@ __device__ __forceinline__ uint32_t fv_wave_min_u32(uint32_t v) { return ~fv_wav
 
 // ---- gather-sum of one window, shared by the training and the hashing kernel ----------------
 // Lane l holds neurons l, l + 64, ... of the window's activation. acc[j] += W[idx_c][l + 64 j]
-// for every window position c in order (idx_c is held by lane c of idx_lane; positions whose
-// index is outside [0, n_cols) add +0, which leaves a sum that started at +0 unchanged).
-// Every load is unconditional -- rows of skipped positions read row 0, lanes past K re-read
-// element K - 1, both replaced by 0 afterwards -- so a batch of RB rows is RB * NV independent
-// loads in flight per lane with no branch between them.
+// for every window position c in order (idx_c is held by lane c of idx_lane). The matrix carries
+// FV_PAD_ROWS rows behind its n_cols real ones: row n_cols is all zeros and is what a position
+// whose index is outside [0, n_cols) reads (adding +0 leaves a sum that started at +0 unchanged),
+// and lanes past K read on into the following row (the last one is never written) and accumulate
+// values nobody uses. So every load is unconditional and no value is selected afterwards: a
+// batch of RB rows is RB * NV independent loads in flight per lane with no branch between them,
+// and one conversion and one addition per element.
 // WEIGHTED: every weight is first multiplied, in fp32, by the weight of its window position --
 // l_mid for the centre, whose column lies in the second half of the columns, l_base for the others
 // (flyvec/src/cuda_funcs.cu:266-286).
+#define FV_PAD_ROWS 2
+
 template <int NV, int RB, typename Acc, bool WEIGHTED = false>
-__device__ __forceinline__ void fv_gather_batch(const float *__restrict__ Wt, uint32_t ldk, uint32_t n_cols,
-                                                const uint32_t (&off)[NV], bool last_valid, int c0,
-                                                int32_t idx_lane, Acc (&acc)[NV], float l_mid = 1.0f,
+__device__ __forceinline__ void fv_gather_batch(const float *__restrict__ Wt, uint32_t ldk, uint32_t n_cols, int lane,
+                                                int c0, int32_t idx_lane, Acc (&acc)[NV], float l_mid = 1.0f,
                                                 float l_base = 1.0f) {
   float v[RB][NV];
-  bool ok[RB];
   float l[RB];
 #pragma unroll
   for (int b = 0; b < RB; ++b) {
-    const int32_t i = (int32_t)fv_readlane((uint32_t)idx_lane, c0 + b);
-    ok[b] = (uint32_t)i < n_cols;
-    l[b] = (uint32_t)i >= n_cols / 2 ? l_mid : l_base;
-    const float *row = Wt + (uint64_t)(ok[b] ? (uint32_t)i : 0u) * ldk;
+    const uint32_t i = fv_readlane((uint32_t)idx_lane, c0 + b);
+    l[b] = i >= n_cols / 2 ? l_mid : l_base;
+    const float *row = Wt + (uint64_t)(i < n_cols ? i : n_cols) * ldk;  // the same in every lane
 #pragma unroll
-    for (int j = 0; j < NV; ++j) v[b][j] = row[off[j]];
+    for (int j = 0; j < NV; ++j) v[b][j] = row[lane + 64 * j];
   }
 #pragma unroll
   for (int b = 0; b < RB; ++b) {
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const bool use = ok[b] && (j < NV - 1 || last_valid);
-      const float t = WEIGHTED ? __fmul_rn(v[b][j], l[b]) : v[b][j];
-      acc[j] = acc[j] + (Acc)(use ? t : 0.0f);
-    }
+    for (int j = 0; j < NV; ++j) acc[j] = acc[j] + (Acc)(WEIGHTED ? __fmul_rn(v[b][j], l[b]) : v[b][j]);
   }
 }
 
@@ -177,16 +174,12 @@ template <int NV, int RB, typename Acc, bool WEIGHTED = false>
 __device__ __forceinline__ void fv_gather_accumulate(const float *__restrict__ Wt, uint32_t ldk, uint32_t K,
                                                      uint32_t n_cols, int lane, int w, int32_t idx_lane,
                                                      Acc (&acc)[NV], float l_mid = 1.0f, float l_base = 1.0f) {
-  uint32_t off[NV];
-#pragma unroll
-  for (int j = 0; j < NV; ++j) off[j] = (uint32_t)lane + 64u * j;
-  const bool last_valid = off[NV - 1] < K;
-  if (!last_valid) off[NV - 1] = K - 1;
+  (void)K;
   int c0 = 0;
   for (; c0 + RB <= w; c0 += RB)
-    fv_gather_batch<NV, RB, Acc, WEIGHTED>(Wt, ldk, n_cols, off, last_valid, c0, idx_lane, acc, l_mid, l_base);
+    fv_gather_batch<NV, RB, Acc, WEIGHTED>(Wt, ldk, n_cols, lane, c0, idx_lane, acc, l_mid, l_base);
   for (; c0 < w; ++c0)
-    fv_gather_batch<NV, 1, Acc, WEIGHTED>(Wt, ldk, n_cols, off, last_valid, c0, idx_lane, acc, l_mid, l_base);
+    fv_gather_batch<NV, 1, Acc, WEIGHTED>(Wt, ldk, n_cols, lane, c0, idx_lane, acc, l_mid, l_base);
 }
 
 template <int NV>

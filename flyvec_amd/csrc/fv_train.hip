@@ -1403,7 +1403,8 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
 }
 
 static int fv_trainer_alloc(fv_trainer *t) {
-  const size_t elems = (size_t)t->N * t->ldk;
+  // FV_PAD_ROWS rows of zeros behind the matrix: what the gather reads for masked positions and past K
+  const size_t elems = (size_t)(t->N + FV_PAD_ROWS) * t->ldk;
   FV_HIP(hipStreamCreate(&t->stream));
   FV_HIP(hipMalloc((void **)&t->Wt, elems * sizeof(float)));
   FV_HIP(hipMalloc((void **)&t->idx, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t)));
