@@ -195,32 +195,37 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
   }
 }
 
-// Argmax over the wave's K values (neuron h = lane + 64 j in acc[j]); the entry of neuron `replaced`
-// (none if >= K) counts as -9999.9999. Ties: the smaller tie key wins. Key = neuron index (lowest
-// index wins), or the position of the neuron in the reference's reduction order: its 64 threads
-// each scan a stride-64 class (= this lane's values, ascending), warp 0 beats warp 1, and inside a
-// warp the shuffle-down tree prefers lanes in bit-reversed order.
+// Argmax over the wave's K values, given as order-preserving keys (neuron h = lane + 64 j in key[j];
+// entries past K hold 0 and are never chosen). The largest key is found first (one 32-bit maximum
+// per register, one wave reduction); among the neurons that hold it the smaller tie key wins. Tie
+// key = neuron index (lowest index wins: the first set bit of a ballot per register), or the position
+// of the neuron in the reference's reduction order: its 64 threads each scan a stride-64 class (= this
+// lane's values, ascending), warp 0 beats warp 1, and inside a warp the shuffle-down tree prefers
+// lanes in bit-reversed order (flyvec/src/cuda_funcs.cu:488-561).
 template <int NV>
-__device__ __forceinline__ uint32_t fv_wave_argmax(const double (&acc)[NV], uint32_t K, uint32_t tie_rule, int lane,
-                                                   uint32_t replaced) {
-  const uint32_t lane_rank = ((uint32_t)lane & 32u) | (__brev((uint32_t)lane & 31u) >> 27);
-  uint64_t best = 0;
+__device__ __forceinline__ uint32_t fv_wave_argmax(const uint32_t (&key)[NV], uint32_t K, uint32_t tie_rule, int lane) {
+  uint32_t m = key[0];
 #pragma unroll
-  for (int j = 0; j < NV; ++j) {
-    const uint32_t h = lane + 64 * j;
-    const bool valid = (j < NV - 1) || h < K;
-    const uint32_t key = tie_rule ? ((lane_rank << 16) | (uint32_t)j) : h;
-    const float v = h == replaced ? (float)-9999.9999 : (float)acc[j];
-    const uint64_t pk = ((uint64_t)fv_ord_key(v) << 32) | (0xffffffffu - key);
-    best = (valid && pk > best) ? pk : best;
+  for (int j = 1; j < NV; ++j) m = max(m, key[j]);
+  const uint32_t top = fv_wave_max_u32(m);
+  const bool last_valid = (uint32_t)lane + 64u * (NV - 1) < K;
+  if (tie_rule == 0) {
+    uint32_t best = 0xffffffffu;
+#pragma unroll
+    for (int j = NV - 1; j >= 0; --j) {
+      const uint64_t hits = __ballot(key[j] == top && (j < NV - 1 || last_valid));
+      if (hits) best = 64u * j + (uint32_t)__ffsll((long long)hits) - 1u;  // lower registers overwrite higher ones
+    }
+    return best;
   }
-  best = fv_wave_max_u64(best);
-  const uint32_t bkey = 0xffffffffu - (uint32_t)best;
-  if (tie_rule) {
-    const uint32_t rank = bkey >> 16;
-    return (bkey & 0xffffu) * 64 + ((rank & 32u) | (__brev(rank & 31u) >> 27));
-  }
-  return bkey;
+  const uint32_t lane_rank = ((uint32_t)lane & 32u) | (__brev((uint32_t)lane & 31u) >> 27);
+  uint32_t tie = 0xffffffffu;
+#pragma unroll
+  for (int j = NV - 1; j >= 0; --j)
+    if (key[j] == top && (j < NV - 1 || last_valid)) tie = (lane_rank << 16) | (uint32_t)j;
+  const uint32_t bkey = fv_wave_min_u32(tie);
+  const uint32_t rank = bkey >> 16;
+  return (bkey & 0xffffu) * 64 + ((rank & 32u) | (__brev(rank & 31u) >> 27));
 }
 
 // Frequency-scaled activation of neuron h for the window whose column index c sits in lane c:
@@ -251,7 +256,12 @@ __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, ui
   for (int j = 0; j < NV; ++j) acc[j] = 0.0;
   fv_gather_accumulate<NV, fv_rows_per_batch<NV>::value, double, WEIGHTED>(a.Wt, a.ldk, a.K, 2 * a.V, lane,
                                                                            (int)a.w, idx, acc, a.lmid, a.lbase);
-  const uint32_t hstar = fv_wave_argmax<NV>(acc, a.K, a.tie_rule, lane, 0xffffffffu);
+  // the search runs on order-preserving keys of the fp32 activations; entries past K sort lowest
+  uint32_t key[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j)
+    key[j] = (j < NV - 1 || (uint32_t)lane + 64u * j < a.K) ? fv_ord_key((float)acc[j]) : 0u;
+  const uint32_t hstar = fv_wave_argmax<NV>(key, a.K, a.tie_rule, lane);
   // the scaled activation is only ever read at the chosen neurons (flyvec/src/cuda_funcs.cu:731)
   const float s = fv_scaled_activation<WEIGHTED>(a, idx, hstar);
   if (lane == 0) {
@@ -260,7 +270,12 @@ __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, ui
     a.sc[r] = s;
   }
   if (DELTA) {
-    const uint32_t second = fv_wave_argmax<NV>(acc, a.K, a.tie_rule, lane, hstar);
+    // flyvec/src/cuda_funcs.cu:495-548: the winner's activation becomes -9999.9999, the search repeats
+    const uint32_t lost = fv_ord_key((float)-9999.9999);
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      if ((uint32_t)lane + 64u * j == hstar) key[j] = lost;
+    const uint32_t second = fv_wave_argmax<NV>(key, a.K, a.tie_rule, lane);
     const float s2 = fv_scaled_activation<WEIGHTED>(a, idx, second);
     if (lane == 0) {
       a.win2[r] = (int32_t)second;
