@@ -178,8 +178,14 @@ __device__ __forceinline__ void fv_gather_accumulate(const float *__restrict__ W
   int c0 = 0;
   for (; c0 + RB <= w; c0 += RB)
     fv_gather_batch<NV, RB, Acc, WEIGHTED>(Wt, ldk, n_cols, lane, c0, idx_lane, acc, l_mid, l_base);
-  for (; c0 < w; ++c0)
-    fv_gather_batch<NV, 1, Acc, WEIGHTED>(Wt, ldk, n_cols, lane, c0, idx_lane, acc, l_mid, l_base);
+  // the rows left over, in batches of 8, 4, 2, 1 rather than one at a time: fewer dependent trips
+#define FV_TAIL(R)                                                                                    \
+  if (RB > R && (w - c0) >= R) {                                                                      \
+    fv_gather_batch<NV, (R < RB ? R : 1), Acc, WEIGHTED>(Wt, ldk, n_cols, lane, c0, idx_lane, acc, l_mid, l_base); \
+    c0 += R;                                                                                          \
+  }
+  FV_TAIL(8) FV_TAIL(4) FV_TAIL(2) FV_TAIL(1)
+#undef FV_TAIL
 }
 
 template <int NV>
