@@ -47,25 +47,25 @@ HASH = dict(K=400, V=20000, w=11, k=32, n=1 << 20)
 # WRITE_SIZE reads them all: x1.0). Traffic below the algorithmic bytes means the rest was served
 # by the L2 caches.
 MEASURED_TRAFFIC = {
-    "dense_max_update": (33304.9 * 2.0 + 65234.4) * 1024,
-    "gather_winner": (26321.3 * 2.0 + 498.2) * 1024,
-    "sparse_owners": (4568.2 * 2.0 + 2483.7) * 1024,
-    "group_xx": (305.5 * 2.0 + 87.2) * 1024,
-    "hash": (2245027.6 * 2.0 + 79242.7) * 1024,
+    "dense_max_update": (33329.0 * 2.0 + 65238.1) * 1024,
+    "gather_winner": (28500.1 * 2.0 + 511.1) * 1024,
+    "sparse_owners": (4571.8 * 2.0 + 2483.8) * 1024,
+    "group_xx": (305.0 * 2.0 + 87.2) * 1024,
+    "hash": (2477844.4 * 2.0 + 82382.9) * 1024,
     # the passes over W as two launches and the slot launch (--dense-launches 2)
-    "update": (32354.2 * 2.0 + 62498.2) * 1024,
+    "update": (32230.1 * 2.0 + 62498.2) * 1024,
     "absmax_ds": (31270.0 * 2.0 + 64.0) * 1024,
-    "slot_update": (622.6 * 2.0 + 1501.2) * 1024,
+    "slot_update": (622.7 * 2.0 + 1501.2) * 1024,
 }
 
 # the same for --workload large-step (profiles/train_step_K1000_V50000_B50000.txt)
 MEASURED_TRAFFIC_LARGE = {
-    "gather_winner": (742880.9 * 2.0 + 4485.2) * 1024,
-    "group_xx": (1244.3 * 2.0 + 316.0) * 1024,
-    "sparse_owners": (32999.4 * 2.0 + 18011.6) * 1024,
-    "absmax_ds": (195342.3 * 2.0 + 67.9) * 1024,
-    "update": (195628.1 * 2.0 + 390612.5) * 1024,
-    "slot_update": (3551.4 * 2.0 + 11373.0) * 1024,
+    "gather_winner": (759026.2 * 2.0 + 5566.8) * 1024,
+    "group_xx": (1246.9 * 2.0 + 316.0) * 1024,
+    "sparse_owners": (32998.9 * 2.0 + 18007.4) * 1024,
+    "absmax_ds": (195342.3 * 2.0 + 68.0) * 1024,
+    "update": (195628.9 * 2.0 + 390612.4) * 1024,
+    "slot_update": (3551.5 * 2.0 + 11354.9) * 1024,
 }
 
 # the two passes over W of a step (and the sparse elements' update) as one launch: W stays in
