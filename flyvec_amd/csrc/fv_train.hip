@@ -63,7 +63,8 @@ struct fv_trainer {
   uint64_t *perm_alt;  // second permutation buffer, allocated by the first shuffle
   uint64_t n_windows;
   float *invf;
-  int32_t *idx;     // B x w column indices of the current minibatch
+  int32_t *idx;     // B rows of idx_stride column indices of the current minibatch (w used, the rest -1)
+  uint32_t idx_stride;  // w rounded up to 4: rows are read 16 bytes at a time
   // the single dense launch samples the column indices of the minibatch expected next (the windows
   // that follow, a full batch or what is left) into idx_ahead while it waits between its passes;
   // a step that finds its own windows there swaps the buffers and skips the sampler's look-ups
@@ -126,6 +127,7 @@ struct fv_gather_args {
   float *sc2;
   uint64_t first;
   uint32_t n, K, ldk, w, V, tie_rule;
+  uint32_t stride;   // entries per row of idx: w rounded up to 4, the ones past w hold -1
   uint32_t sampled;  // idx already holds this minibatch
   uint32_t prune;    // in-window duplicate pruning while sampling
   float lmid, lbase; // weight of a window's centre position and of the others (WEIGHTED kernels)
@@ -178,15 +180,15 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
     idx[k] = -1;
     if (lane < (int)a.w && r < a.n) {
       if (a.sampled) {
-        idx[k] = a.idx[(uint64_t)r * a.w + lane];
+        idx[k] = a.idx[(uint64_t)r * a.stride + lane];
       } else {
         const uint64_t s = a.pstart[a.first + r];
         int32_t tok = a.corpus[s + lane];
         if (a.prune) tok = fv_prune_token(tok, lane, (int)a.w);
         idx[k] = fv_column_index(tok, (uint32_t)lane, a.w, a.V);
-        a.idx[(uint64_t)r * a.w + lane] = idx[k];
       }
     }
+    if (!a.sampled && lane < (int)a.stride && r < a.n) a.idx[(uint64_t)r * a.stride + lane] = idx[k];
   }
 #pragma unroll
   for (int k = 0; k < FV_GATHER_WINDOWS; ++k) {
@@ -298,15 +300,16 @@ __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, ui
 #define FV_NB_CLASSES (1 << FV_NB_CLASS_SHIFT)  // column classes per neuron (kernel 3)
 #define FV_NB_CNT_WORDS 5120    // LDS counter words per class block (20 KB)
 #define FV_SP_LIST_CAP 1024     // positions of non-zero counters collected in LDS at a time
-#define FV_SP_CHUNK 16          // window positions read by 16 neighbouring lanes
-#define FV_IDX_PAD 80            // entries of -1 behind the index matrix: a padding row plus a chunk
+#define FV_SP_CHUNK 16          // window positions read by 4 neighbouring lanes, 16 bytes each
+#define FV_IDX_PAD 80            // entries of -1 behind the index matrix: a padding row (up to 64 entries) and spare
 #define FV_SP_STAGE 2048        // window ids staged in LDS at a time
 #ifndef FV_SP_THREADS
 #define FV_SP_THREADS 256       // threads of a class block
 #endif
 #ifndef FV_SP_LOADS
-#define FV_SP_LOADS 16          // most loads a lane has in flight in the counting pass
+#define FV_SP_LOADS 8           // most 16-byte loads a lane has in flight in the counting pass
 #endif
+#define FV_SP_HEAVY 128         // a class block of a neuron with more windows than this runs at raised wave priority
 #define FV_NB_ROUND 2048        // scaled activations staged in LDS at a time
 #define FV_NB_LOADS 32          // winners a thread of the grouping kernel fetches together
 
@@ -576,6 +579,7 @@ struct fv_sparse_args {
   float *bmax_sparse;    // one maximum of |ds| per block
   uint32_t *slot_count;  // records written per block
   uint32_t ldk, w, V, pad_row;  // pad_row: the row index just behind the index matrix
+  uint32_t stride;              // entries per row of idx (a multiple of 4)
   // anti-Hebbian form only: the windows in which the neuron came second, grouped like the others;
   // the count of those occurrences of an element goes to slot_n2 beside its record
   const uint32_t *order2;
@@ -591,37 +595,48 @@ struct fv_sparse_args {
 __device__ __forceinline__ void fv_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // Counting pass of one class block over the windows whose ids are staged in LDS: ord[0 .. n_staged),
-// followed up to the next multiple of 16 * LOADS by the id of the padding row behind the index
-// matrix (all -1). Sixteen consecutive lanes read sixteen consecutive positions of one window, so a
-// wave's load touches four rows; positions past the window (the next row or the padding) are
-// loaded and dropped. A lane issues LOADS loads back to back with no branch between them (the
-// compiler waits for every load in flight at a branch target), then counts. With the class in the
-// top bits and the column of the class below, one subtraction and one comparison tell whether an
-// entry is this block's: of class q, inside [lo, lo + span), not masked, not dropped.
-#define FV_SP_WPS (FV_SP_THREADS / 16)  // windows the block takes per step
+// followed up to the next multiple of FV_SP_WPS * LOADS by the id of the padding row behind the
+// index matrix (all -1). A row of idx is `stride` entries, a multiple of 4, those past w holding -1;
+// four consecutive lanes read the sixteen positions of a chunk of one window 16 bytes each, so a
+// wave's load covers sixteen windows. A lane issues LOADS loads back to back with no branch between
+// them (the compiler waits for every load in flight at a branch target), then counts. With the
+// class in the top bits and the column of the class below, one subtraction and one comparison tell
+// whether an entry is this block's: of class q, inside [lo, lo + span), not masked, not padding.
+#define FV_SP_WPS (FV_SP_THREADS / 4)  // windows the block takes per step
+template <bool NARROW>
+__device__ __forceinline__ void fv_sparse_count_entry(uint32_t *cnt, int32_t iv, uint32_t drop, uint32_t origin,
+                                                      uint32_t span) {
+  const uint32_t t = __builtin_rotateright32((uint32_t)iv | drop, FV_NB_CLASS_SHIFT) - origin;
+  if (t < span) {
+    if (NARROW)
+      atomicAdd(&cnt[t >> 1], 1u << (16 * (t & 1)));
+    else
+      atomicAdd(&cnt[t], 1u);
+  }
+}
+
 template <bool NARROW, int LOADS>
 __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const uint32_t *ord, uint32_t n_staged,
-                                                const int32_t *__restrict__ idx, uint32_t w, uint32_t q,
+                                                const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
                                                 uint32_t lo, uint32_t span, uint32_t tid) {
-  const uint32_t c = tid & 15u, slot = tid >> 4;
+  const uint32_t c4 = 4u * (tid & 3u), slot = tid >> 2;
   const uint32_t steps = (n_staged + FV_SP_WPS - 1) / FV_SP_WPS;
   const uint32_t origin = (q << (32 - FV_NB_CLASS_SHIFT)) | lo;
-  for (uint32_t c0 = 0; c0 < w; c0 += FV_SP_CHUNK) {
-    const uint32_t cc = c0 + c;
-    const uint32_t drop = cc < w ? 0u : 0xffffffffu;
+  for (uint32_t c0 = 0; c0 < stride; c0 += FV_SP_CHUNK) {
+    const bool live = c0 + c4 < stride;  // a row shorter than the chunk: the lanes past its end read its start again
+    const uint32_t cc = live ? c0 + c4 : 0u;
+    const uint32_t drop = live ? 0u : 0xffffffffu;
     for (uint32_t s0 = 0; s0 < steps; s0 += LOADS) {
-      int32_t iv[LOADS];
+      int4 iv[LOADS];
 #pragma unroll
-      for (int b = 0; b < LOADS; ++b) iv[b] = idx[ord[(s0 + b) * FV_SP_WPS + slot] * w + cc];
+      for (int b = 0; b < LOADS; ++b)
+        iv[b] = *(const int4 *)(idx + (uint64_t)ord[(s0 + b) * FV_SP_WPS + slot] * stride + cc);
 #pragma unroll
       for (int b = 0; b < LOADS; ++b) {
-        const uint32_t t = __builtin_rotateright32((uint32_t)iv[b] | drop, FV_NB_CLASS_SHIFT) - origin;
-        if (t < span) {
-          if (NARROW)
-            atomicAdd(&cnt[t >> 1], 1u << (16 * (t & 1)));
-          else
-            atomicAdd(&cnt[t], 1u);
-        }
+        fv_sparse_count_entry<NARROW>(cnt, iv[b].x, drop, origin, span);
+        fv_sparse_count_entry<NARROW>(cnt, iv[b].y, drop, origin, span);
+        fv_sparse_count_entry<NARROW>(cnt, iv[b].z, drop, origin, span);
+        fv_sparse_count_entry<NARROW>(cnt, iv[b].w, drop, origin, span);
       }
     }
   }
@@ -630,19 +645,19 @@ __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const uint32_t *o
 // The same with the number of loads in flight fitted to the number of windows; pads ord[].
 template <bool NARROW>
 __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, uint32_t *ord, uint32_t n_staged, uint32_t pad_row,
-                                                    const int32_t *__restrict__ idx, uint32_t w, uint32_t q,
+                                                    const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
                                                     uint32_t lo, uint32_t span, uint32_t tid) {
-  static_assert(FV_SP_STAGE % (FV_SP_WPS * FV_SP_LOADS) == 0 && FV_SP_LOADS % 8 == 0, "padding of ord[] stays inside it");
-  const uint32_t per = FV_SP_WPS * (n_staged <= FV_SP_WPS * 2 ? 2 : n_staged <= FV_SP_WPS * 8 ? 8 : FV_SP_LOADS);
+  static_assert(FV_SP_STAGE % (FV_SP_WPS * FV_SP_LOADS) == 0 && FV_SP_LOADS % 4 == 0, "padding of ord[] stays inside it");
+  const uint32_t per = FV_SP_WPS * (n_staged <= FV_SP_WPS ? 1 : n_staged <= FV_SP_WPS * 4 ? 4 : FV_SP_LOADS);
   const uint32_t padded = (n_staged + per - 1) / per * per;
   for (uint32_t i = n_staged + tid; i < padded; i += FV_SP_THREADS) ord[i] = pad_row;
   fv_lds_barrier();
-  if (per == FV_SP_WPS * 2)
-    fv_sparse_count<NARROW, 2>(cnt, ord, n_staged, idx, w, q, lo, span, tid);
-  else if (per == FV_SP_WPS * 8)
-    fv_sparse_count<NARROW, 8>(cnt, ord, n_staged, idx, w, q, lo, span, tid);
+  if (per == FV_SP_WPS)
+    fv_sparse_count<NARROW, 1>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+  else if (per == FV_SP_WPS * 4)
+    fv_sparse_count<NARROW, 4>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
   else
-    fv_sparse_count<NARROW, FV_SP_LOADS>(cnt, ord, n_staged, idx, w, q, lo, span, tid);
+    fv_sparse_count<NARROW, FV_SP_LOADS>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
 }
 
 // DELTA: the neuron's elements are counted over two lists of windows, those it won and those in
@@ -668,6 +683,9 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
     }
     return;
   }
+  // The launch lasts as long as its few heaviest blocks: their waves go first wherever they share a
+  // SIMD with the waves of light blocks.
+  if (c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
   const uint32_t base = a.group_base[h];
   const uint32_t base2 = DELTA ? a.group_base2[h] : 0u;
   const float x_h = a.xx[h];
@@ -707,9 +725,9 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
           fv_lds_barrier();
         }
         if (narrow)
-          fv_sparse_count_any<true>(counters, ord, n_staged, a.pad_row, a.idx, a.w, q, lo, span, tid);
+          fv_sparse_count_any<true>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
         else
-          fv_sparse_count_any<false>(counters, ord, n_staged, a.pad_row, a.idx, a.w, q, lo, span, tid);
+          fv_sparse_count_any<false>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
       }
     }
     // Every non-zero counter is one distinct element. Their positions are collected in LDS, up to
@@ -860,6 +878,7 @@ struct fv_dense_args {
   int32_t *idx_ahead;
   uint64_t ahead_first;
   uint32_t ahead_n;
+  uint32_t idx_stride;  // entries per row of idx_ahead
 };
 
 __device__ __forceinline__ bool fv_is_sentinel(float w) { return __float_as_uint(w) == FV_SENTINEL; }
@@ -1131,10 +1150,10 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   const uint32_t n20 = DELTA ? a.slot_n2[at0] : 0u;
   // the next minibatch's column indices, by all waves but the first: the window's start now
   constexpr uint32_t TS = T - 64;
-  const uint32_t ahead_entries = a.ahead_n * a.w;
+  const uint32_t ahead_entries = a.ahead_n * a.idx_stride;  // the entries past w of a row get -1
   const uint32_t e0 = blockIdx.x * TS + (threadIdx.x - 64);
   const bool samples0 = threadIdx.x >= 64 && e0 < ahead_entries;
-  const uint32_t er0 = samples0 ? e0 / a.w : 0u;
+  const uint32_t er0 = samples0 ? e0 / a.idx_stride : 0u;
   const uint64_t start0 = a.ahead_n ? a.pstart[a.ahead_first + er0] : 0ull;
   uint32_t q = q0;
 #pragma unroll
@@ -1198,13 +1217,13 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   // the token of the sampled position while the first wave waits; then, for a minibatch with more
   // positions than the launch has sampling threads, the rest
   if (samples0) {
-    const uint32_t c = e0 - er0 * a.w;
-    a.idx_ahead[e0] = fv_column_index(a.corpus[start0 + c], c, a.w, a.V);
+    const uint32_t c = e0 - er0 * a.idx_stride;
+    a.idx_ahead[e0] = c < a.w ? fv_column_index(a.corpus[start0 + c], c, a.w, a.V) : -1;
   }
   if (threadIdx.x >= 64)
     for (uint32_t e = e0 + gridDim.x * TS; e < ahead_entries; e += gridDim.x * TS) {
-      const uint32_t r = e / a.w, c = e - r * a.w;
-      a.idx_ahead[e] = fv_column_index(a.corpus[a.pstart[a.ahead_first + r] + c], c, a.w, a.V);
+      const uint32_t r = e / a.idx_stride, c = e - r * a.idx_stride;
+      a.idx_ahead[e] = c < a.w ? fv_column_index(a.corpus[a.pstart[a.ahead_first + r] + c], c, a.w, a.V) : -1;
     }
   // ds of the first record does not depend on the scale: formed while the first wave waits
   // (every thread takes this path, with no additions where it has no record: the fetch is then
@@ -1422,11 +1441,13 @@ static int fv_trainer_alloc(fv_trainer *t) {
   const size_t elems = (size_t)(t->N + FV_PAD_ROWS) * t->ldk;
   FV_HIP(hipStreamCreate(&t->stream));
   FV_HIP(hipMalloc((void **)&t->Wt, elems * sizeof(float)));
-  FV_HIP(hipMalloc((void **)&t->idx, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t)));
-  FV_HIP(hipMemsetAsync(t->idx, 0xff, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t), t->stream));
+  t->idx_stride = (t->w + 3u) & ~3u;
+  const size_t idx_entries = (size_t)t->B * t->idx_stride + FV_IDX_PAD;
+  FV_HIP(hipMalloc((void **)&t->idx, idx_entries * sizeof(int32_t)));
+  FV_HIP(hipMemsetAsync(t->idx, 0xff, idx_entries * sizeof(int32_t), t->stream));
   if (t->onepass_unroll) {
-    FV_HIP(hipMalloc((void **)&t->idx_ahead, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t)));
-    FV_HIP(hipMemsetAsync(t->idx_ahead, 0xff, ((size_t)t->B * t->w + FV_IDX_PAD) * sizeof(int32_t), t->stream));
+    FV_HIP(hipMalloc((void **)&t->idx_ahead, idx_entries * sizeof(int32_t)));
+    FV_HIP(hipMemsetAsync(t->idx_ahead, 0xff, idx_entries * sizeof(int32_t), t->stream));
   }
   FV_HIP(hipMalloc((void **)&t->win, ((size_t)t->B + 16) * sizeof(int32_t)));  // read in 16-byte pieces
   FV_HIP(hipMalloc((void **)&t->sc, (size_t)t->B * sizeof(float)));
@@ -1757,6 +1778,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.pstart = t->pstart;
   g.invf = t->invf;
   g.idx = t->idx;
+  g.stride = t->idx_stride;
   g.win = t->win;
   g.win16 = t->win16;
   g.sc = t->sc;
@@ -1849,6 +1871,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.bmax_sparse = t->bmax + t->dense_blocks;
   sp.slot_count = t->slot_count;
   sp.pad_row = t->B;
+  sp.stride = t->idx_stride;
   sp.ldk = t->ldk;
   sp.w = t->w;
   sp.V = (uint32_t)t->V;
@@ -1878,6 +1901,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.corpus = t->corpus;
   d.pstart = t->pstart;
   d.idx_ahead = nullptr;
+  d.idx_stride = t->idx_stride;
   d.ahead_first = 0;
   d.ahead_n = 0;
   d.slot_stride = (uint64_t)t->B * t->w * (anti ? 2 : 1);
