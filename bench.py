@@ -47,15 +47,15 @@ HASH = dict(K=400, V=20000, w=11, k=32, n=1 << 20)
 # WRITE_SIZE reads them all: x1.0). Traffic below the algorithmic bytes means the rest was served
 # by the L2 caches.
 MEASURED_TRAFFIC = {
-    "dense_max_update": (33329.0 * 2.0 + 65238.1) * 1024,
-    "gather_winner": (28500.1 * 2.0 + 511.1) * 1024,
-    "sparse_owners": (4571.8 * 2.0 + 2483.8) * 1024,
-    "group_xx": (305.0 * 2.0 + 87.2) * 1024,
-    "hash": (2477844.4 * 2.0 + 82382.9) * 1024,
+    "dense_max_update": (33326.2 * 2.0 + 65231.5) * 1024,
+    "gather_winner": (28495.7 * 2.0 + 503.2) * 1024,
+    "sparse_owners": (4607.5 * 2.0 + 2483.7) * 1024,
+    "group_xx": (310.0 * 2.0 + 87.2) * 1024,
+    "hash": (2477777.6 * 2.0 + 82452.4) * 1024,
     # the passes over W as two launches and the slot launch (--dense-launches 2)
-    "update": (32230.1 * 2.0 + 62498.2) * 1024,
+    "update": (32193.9 * 2.0 + 62498.2) * 1024,
     "absmax_ds": (31270.0 * 2.0 + 64.0) * 1024,
-    "slot_update": (622.7 * 2.0 + 1501.2) * 1024,
+    "slot_update": (622.6 * 2.0 + 1501.2) * 1024,
 }
 
 # the same for --workload large-step (profiles/train_step_K1000_V50000_B50000.txt)
