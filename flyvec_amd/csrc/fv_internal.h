@@ -134,6 +134,28 @@ __device__ __forceinline__ uint32_t fv_wave_max_u32(uint32_t v) {
 
 __device__ __forceinline__ uint32_t fv_wave_min_u32(uint32_t v) { return ~fv_wave_max_u32(~v); }
 
+// Inclusive prefix sum over the 64 lanes (all must be active) in six DPP additions: shifts by 1, 2,
+// 4, 8 inside each row of 16 lanes (a lane without a source adds 0), then the last lane of row 0 / 2
+// onto rows 1 / 3, then the last lane of row 1 onto rows 2 and 3. A cross-lane shuffle costs an LDS
+// round trip per step; these are ordinary vector instructions.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t fv_dpp_or_zero(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, true);
+}
+__device__ __forceinline__ uint32_t fv_wave_inclusive_scan_u32(uint32_t v) {
+  v += fv_dpp_or_zero<0x111, 0xf>(v);  // row_shr:1
+  v += fv_dpp_or_zero<0x112, 0xf>(v);  // row_shr:2
+  v += fv_dpp_or_zero<0x114, 0xf>(v);  // row_shr:4
+  v += fv_dpp_or_zero<0x118, 0xf>(v);  // row_shr:8
+  v += fv_dpp_or_zero<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v += fv_dpp_or_zero<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+// Sum over the 64 lanes, the same in every lane.
+__device__ __forceinline__ uint32_t fv_wave_sum_u32(uint32_t v) {
+  return fv_readlane(fv_wave_inclusive_scan_u32(v), 63);
+}
+
 
 // ---- gather-sum of one window, shared by the training and the hashing kernel ----------------
 // Lane l holds neurons l, l + 64, ... of the window's activation. acc[j] += W[idx_c][l + 64 j]

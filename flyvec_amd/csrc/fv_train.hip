@@ -358,7 +358,7 @@ __device__ __forceinline__ float fv_block_max_nonneg(float m, float *smem) {
 
 // Sum over the block of one value per thread (result in every thread).
 __device__ __forceinline__ uint32_t fv_block_sum_u32(uint32_t v, uint32_t *smem /*17*/) {
-  for (int d = 32; d >= 1; d >>= 1) v += __shfl_down(v, d, 64);
+  v = fv_wave_sum_u32(v);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
   __syncthreads();
   if (lane == 0) smem[wave] = v;
@@ -371,12 +371,7 @@ __device__ __forceinline__ uint32_t fv_block_sum_u32(uint32_t v, uint32_t *smem 
 // Exclusive prefix sum of one value per thread over the block.
 __device__ __forceinline__ uint32_t fv_block_exclusive_scan(uint32_t v, uint32_t *smem /*17*/) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint32_t incl = v;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const uint32_t o = __shfl_up(incl, d, 64);
-    if (lane >= d) incl += o;
-  }
+  const uint32_t incl = fv_wave_inclusive_scan_u32(v);
   __syncthreads();
   if (lane == 63) smem[wave] = incl;
   __syncthreads();
@@ -388,12 +383,7 @@ __device__ __forceinline__ uint32_t fv_block_exclusive_scan(uint32_t v, uint32_t
 // Exclusive prefix sum and total of one value per thread over the block, in one pass.
 __device__ __forceinline__ uint32_t fv_block_scan_total(uint32_t v, uint32_t *smem /*17*/, uint32_t *total) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
-  uint32_t incl = v;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const uint32_t o = __shfl_up(incl, d, 64);
-    if (lane >= d) incl += o;
-  }
+  const uint32_t incl = fv_wave_inclusive_scan_u32(v);
   __syncthreads();
   if (lane == 63) smem[wave] = incl;
   __syncthreads();
@@ -772,15 +762,10 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
         // list positions: prefix sum inside the wave, one LDS atomic per wave
         const uint32_t my = (uint32_t)__popcll(mine);
         const int lane = tid & 63;
-        uint32_t incl = my;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-          const uint32_t o = __shfl_up(incl, d, 64);
-          if (lane >= d) incl += o;
-        }
+        const uint32_t incl = fv_wave_inclusive_scan_u32(my);
         uint32_t wave_base = 0;
         if (lane == 63 && incl) wave_base = atomicAdd(&sh_pos, incl);
-        wave_base = __shfl(wave_base, 63, 64);
+        wave_base = fv_readlane(wave_base, 63);
         uint32_t e = wave_base + incl - my;
         while (mine) {
           const uint32_t b = (uint32_t)__ffsll((long long)mine) - 1;
