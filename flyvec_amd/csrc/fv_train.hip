@@ -515,9 +515,15 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
   // windows that is the plain sum in window order.
   float part = 0.0f;
   if (staged) {
-    if (tid < 64)
-      for (uint32_t j = tid; j < c_h; j += 64) part = __fadd_rn(part, scbuf[j]);
-    __syncthreads();
+    if (tid < 64) {
+      // four values fetched together, added one after the other
+      uint32_t j = tid;
+      for (; j + 192 < c_h; j += 256) {
+        const float v0 = scbuf[j], v1 = scbuf[j + 64], v2 = scbuf[j + 128], v3 = scbuf[j + 192];
+        part = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(part, v0), v1), v2), v3);
+      }
+      for (; j < c_h; j += 64) part = __fadd_rn(part, scbuf[j]);
+    }
   } else {
     for (uint32_t j0 = 0; j0 < c_h; j0 += FV_NB_ROUND) {
       const uint32_t mr = min(c_h - j0, (uint32_t)FV_NB_ROUND);
@@ -538,14 +544,14 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
       __syncthreads();
     }
   }
-  float xx = 0.0f;
-  if (tid < 64) scbuf[tid] = part;
-  __syncthreads();
-  if (tid == 0) {
-    const uint32_t np = min(c_h, 64u);
-    for (uint32_t l = 0; l < np; ++l) xx = __fadd_rn(xx, scbuf[l]);
+  // The partial sums in lane order, read straight from the lanes of the first wave (a partial sum
+  // without values is +0, which changes nothing: the running total starts at +0 and so is never -0).
+  if (tid < 64) {
+    float xx = 0.0f;
+#pragma unroll
+    for (int l = 0; l < 64; ++l) xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), l)));
+    if (tid == 0) a.xx[h] = a.accumulate ? __fadd_rn(a.xx[h], xx) : xx;
   }
-  if (tid == 0) a.xx[h] = a.accumulate ? __fadd_rn(a.xx[h], xx) : xx;
 }
 
 // ---- kernel 3: sparse elements -----------------------------------------------------------------------
