@@ -93,12 +93,13 @@ def hash_bytes_per_window(K, w):
     return 4 * w * K + 4 * w + 8 * ((K + 63) // 64)
 
 
-def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0):
+def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0, separate_grouping=False):
     from flyvec_amd import Trainer, synthetic
     tokens, offsets = synthetic.corpus(c["n_tokens"], c["V"], s=c["zipf_s"], mean_chunk=c["mean_chunk"])
     W0 = synthetic.synapses(c["K"], c["V"], seed=5)
     t = Trainer(c["V"], c["K"], c["w"], c["B"], initial_learning_rate=c["lr0"], prec=c["prec"])
     t.set_dense_launches(dense_launches)
+    t.set_grouping_launch(separate_grouping)
     t.set_corpus(tokens, offsets)
     nwin = t.num_windows
     perm = np.random.default_rng(6).permutation(nwin).astype(np.uint64)
@@ -126,6 +127,7 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0):
     # overhead to each); this destroys W, so it comes last
     kern_ms = t.time_kernels(reps=50)
     launches = t.dense_launches
+    grouping_separate = t.grouping_launch
     t.close()
 
     N = 2 * c["V"]
@@ -136,6 +138,10 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0):
         parts = ("absmax_ds", "update", "slot_update")
         kern_ms[DENSE_ONE] = sum(kern_ms.pop(k) for k in parts)
         per_kernel[DENSE_ONE] = sum(per_kernel.pop(k) for k in parts)
+    if not grouping_separate:
+        # the sparse launch has grouped the windows by winner itself: no grouping launch ran
+        kern_ms["sparse_owners"] += kern_ms.pop("group_xx")
+        per_kernel["sparse_owners"] += per_kernel.pop("group_xx")
     dom = max(kern_ms, key=kern_ms.get)
     achieved = per_kernel[dom] / (kern_ms[dom] * 1e-3)
     ms_per_step = wall / steps * 1e3
@@ -149,6 +155,7 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0):
                      "traffic": (MEASURED_TRAFFIC if c is TRAIN else MEASURED_TRAFFIC_LARGE).get(dom),
                      "algorithmic_bytes": per_kernel[dom]},
         "dense_launches": launches,
+        "grouping_launch": "own" if grouping_separate else "in sparse_owners",
         "step_roofline_frac": (step_bytes / HBM_PEAK) / (ms_per_step * 1e-3),
         "step_algorithmic_bytes": step_bytes,
         "n_windows": nwin,
@@ -270,6 +277,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample length (0 = skip)")
     ap.add_argument("--no-hash", action="store_true")
+    ap.add_argument("--separate-grouping", action="store_true",
+                    help="group the windows by winner in a launch of its own (the default does it inside the sparse launch)")
     ap.add_argument("--dense-launches", type=int, choices=[0, 1, 2], default=0,
                     help="the passes over W of a step as one launch (1), two (2), or as the library chooses (0)")
     ap.add_argument("--workload", choices=["step", "large-step", "epoch"], default="step",
@@ -300,7 +309,7 @@ def main():
     c = LARGE if args.workload == "large-step" else TRAIN
     if args.workload == "large-step":
         args.steps, args.warmup, args.no_hash = min(args.steps, 50), min(args.warmup, 5), True
-    tr = bench_train(args.steps, args.warmup, args.cpu_seconds, c, args.dense_launches)
+    tr = bench_train(args.steps, args.warmup, args.cpu_seconds, c, args.dense_launches, args.separate_grouping)
     line = {
         "metric": f"train windows/s at K={c['K']},Nvoc={c['V'] // 1000}k",
         "value": tr["value"], "unit": "windows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -316,6 +325,7 @@ def main():
         "event_ms_per_step": tr["event_ms_per_step"],
         "kernel_ms": tr["kernel_ms"],
         "dense_launches": tr["dense_launches"],
+        "grouping_launch": tr["grouping_launch"],
     }
     if "cpu_baseline" in tr:
         line["cpu_baseline"] = tr["cpu_baseline"]

@@ -82,6 +82,8 @@ SIGNATURES = {
     "fv_trainer_set_dense_launches": [_vp, _u32],
     "fv_trainer_get_dense_launches": [_vp, C.POINTER(_u32)],
     "fv_trainer_set_wait_limit": [_vp, _u32],
+    "fv_trainer_set_grouping_launch": [_vp, _u32],
+    "fv_trainer_get_grouping_launch": [_vp, C.POINTER(_u32)],
     "fv_trainer_get_winners": [_vp, _vp, _u32],
     "fv_trainer_get_step_stats": [_vp, _vp, C.POINTER(_f32)],
     "fv_trainer_row_norms": [_vp, _u32, _vp],

@@ -31,6 +31,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -74,6 +75,12 @@ struct fv_trainer {
   uint32_t ahead_n;
   int32_t *win;     // B winners
   uint16_t *win16;  // the same, 16 bits each (padded by 64)
+  // Steps whose sparse launch groups for itself: the winner kernel sets bit r of the winner's row of
+  // won[parity]; the sparse launch reads the rows and clears the other parity's, which the next such
+  // step fills. Null when the batch is too large.
+  uint32_t *won[2];        // K rows of won_words words each
+  uint32_t won_words;      // words per row (even)
+  uint32_t won_parity;     // the pair the last such step used
   // anti-Hebbian form (delta != 0), allocated with the first such step: the second neuron of every
   // window, its scaled activation, the windows grouped by it, the second count of every slot record
   int32_t *win2;
@@ -103,6 +110,8 @@ struct fv_trainer {
   // host-visible word a block sets when it gave up waiting for the others
   unsigned onepass_blocks, onepass_unroll;
   bool onepass;  // in use (fv_trainer_set_dense_launches)
+  bool separate_grouping;  // the grouping kernel always runs as a launch of its own (fv_trainer_set_grouping_launch)
+  bool last_grouped_in_sparse;  // the form the last whole step took: a launch on its own repeats that form
   unsigned long long *arrive;
   uint32_t onepass_epoch;
   uint32_t onepass_spin_limit;
@@ -120,6 +129,8 @@ struct fv_gather_args {
   int32_t *idx;
   int32_t *win;
   uint16_t *win16;  // the same winners as 16-bit values, for the grouping kernel
+  uint32_t *won;        // not null: bit r of row hstar is set (atomic OR; the rows are zero before)
+  uint32_t won_words;
   float *sc;
   // anti-Hebbian form only: the second neuron of every window and its scaled activation
   int32_t *win2;
@@ -270,7 +281,11 @@ __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, ui
     a.win[r] = (int32_t)hstar;
     a.win16[r] = (uint16_t)hstar;
     a.sc[r] = s;
+    if (a.won) atomicOr(&a.won[(uint64_t)hstar * a.won_words + (r >> 5)], 1u << (r & 31u));
   }
+  // the wave of the step's last window fills the 16-bit winners up to the next multiple of 64 with a
+  // value no neuron has
+  if (r == a.n - 1 && r + 1 + lane < ((a.n + 63) & ~63u)) a.win16[r + 1 + lane] = 0x7fffu;
   if (DELTA) {
     // flyvec/src/cuda_funcs.cu:495-548: the winner's activation becomes -9999.9999, the search repeats
     const uint32_t lost = fv_ord_key((float)-9999.9999);
@@ -380,13 +395,19 @@ __device__ __forceinline__ uint32_t fv_block_exclusive_scan(uint32_t v, uint32_t
   return before + incl - v;
 }
 
-// Exclusive prefix sum and total of one value per thread over the block, in one pass.
+// Barrier for data exchanged through LDS only: waits for the wave's LDS operations, not for its
+// global loads and stores still in flight.
+__device__ __forceinline__ void fv_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// Exclusive prefix sum and total of one value per thread over the block, in one pass. LDS_ONLY: the
+// barriers do not wait for the caller's global loads in flight.
+template <bool LDS_ONLY = false>
 __device__ __forceinline__ uint32_t fv_block_scan_total(uint32_t v, uint32_t *smem /*17*/, uint32_t *total) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
   const uint32_t incl = fv_wave_inclusive_scan_u32(v);
-  __syncthreads();
+  if (LDS_ONLY) fv_lds_barrier(); else __syncthreads();
   if (lane == 63) smem[wave] = incl;
-  __syncthreads();
+  if (LDS_ONLY) fv_lds_barrier(); else __syncthreads();
   uint32_t before = 0, all = 0;
   for (int i = 0; i < n_waves; ++i) {
     const uint32_t t = smem[i];
@@ -406,6 +427,8 @@ __device__ __forceinline__ uint32_t fv_winner_of(const int4 &v, int q) {
   const uint32_t word = (uint32_t)((q >> 1) == 0 ? v.x : (q >> 1) == 1 ? v.y : (q >> 1) == 2 ? v.z : v.w);
   return (q & 1) ? word >> 16 : word & 0xffffu;
 }
+
+typedef short fv_short2 __attribute__((ext_vector_type(2)));
 
 template <bool SMALL>
 __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_args a) {
@@ -584,11 +607,17 @@ struct fv_sparse_args {
   uint32_t *slot_n2;
   float delta;
   float lmid, lbase;  // weight of a window's centre position (columns >= V) and of the others
+  // grouping form only: the block finds the neuron's windows in the winner array itself
+  const uint32_t *won;        // row h: bit r set where neuron h won window r (won_words words, an even number)
+  const uint16_t *win;        // 16-bit winners; behind the last one, up to a multiple of 64 entries, 0x7fff
+  uint32_t won_words;
+  uint32_t *won_clear;  // the other buffer: the class-0 block of neuron h clears row h
+  const float *sc;      // scaled activations of the windows
+  uint32_t n;           // windows of the step
+  uint32_t *order_out;  // a neuron's window ids beyond what LDS stages go through here
+  uint32_t *group_base_out, *group_count_out;
+  float *xx_out;
 };
-
-// Barrier for data exchanged through LDS only: waits for the wave's LDS operations, not for its
-// global stores still in flight.
-__device__ __forceinline__ void fv_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // Counting pass of one class block over the windows whose ids are staged in LDS: ord[0 .. n_staged),
 // followed up to the next multiple of FV_SP_WPS * LOADS by the id of the padding row behind the
@@ -611,8 +640,8 @@ __device__ __forceinline__ void fv_sparse_count_entry(uint32_t *cnt, int32_t iv,
   }
 }
 
-template <bool NARROW, int LOADS>
-__device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const uint32_t *ord, uint32_t n_staged,
+template <bool NARROW, int LOADS, typename Ord>
+__device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const Ord *ord, uint32_t n_staged,
                                                 const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
                                                 uint32_t lo, uint32_t span, uint32_t tid) {
   const uint32_t c4 = 4u * (tid & 3u), slot = tid >> 2;
@@ -639,38 +668,124 @@ __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const uint32_t *o
 }
 
 // The same with the number of loads in flight fitted to the number of windows; pads ord[].
-template <bool NARROW>
-__device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, uint32_t *ord, uint32_t n_staged, uint32_t pad_row,
+template <bool NARROW, typename Ord>
+__device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uint32_t n_staged, uint32_t pad_row,
                                                     const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
                                                     uint32_t lo, uint32_t span, uint32_t tid) {
   static_assert(FV_SP_STAGE % (FV_SP_WPS * FV_SP_LOADS) == 0 && FV_SP_LOADS % 4 == 0, "padding of ord[] stays inside it");
   const uint32_t per = FV_SP_WPS * (n_staged <= FV_SP_WPS ? 1 : n_staged <= FV_SP_WPS * 4 ? 4 : FV_SP_LOADS);
   const uint32_t padded = (n_staged + per - 1) / per * per;
-  for (uint32_t i = n_staged + tid; i < padded; i += FV_SP_THREADS) ord[i] = pad_row;
+  for (uint32_t i = n_staged + tid; i < padded; i += FV_SP_THREADS) ord[i] = (Ord)pad_row;
   fv_lds_barrier();
   if (per == FV_SP_WPS)
-    fv_sparse_count<NARROW, 1>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+    fv_sparse_count<NARROW, 1, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
   else if (per == FV_SP_WPS * 4)
-    fv_sparse_count<NARROW, 4>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+    fv_sparse_count<NARROW, 4, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
   else
-    fv_sparse_count<NARROW, FV_SP_LOADS>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+    fv_sparse_count<NARROW, FV_SP_LOADS, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
 }
 
 // DELTA: the neuron's elements are counted over two lists of windows, those it won and those in
 // which it came second, into two counter arrays; a record carries both counts.
-template <bool DELTA>
+// GROUPING: no grouping launch has run. Every class block scans the winner array like the grouping
+// kernel's block of its neuron (a thread's run is at most 64 windows: the step has no more than
+// 64 * FV_SP_THREADS), stages the neuron's window ids in LDS straight from the scan, and adds the
+// neuron's scaled activations in the grouping kernel's order; the block of class 0 leaves xx[h],
+// the neuron's count and its base for the dense launch.
+template <bool DELTA, bool GROUPING>
 __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
+  static_assert(!(DELTA && GROUPING), "the anti-Hebbian form has its two lists grouped by launches of their own");
   __shared__ uint32_t cnt[FV_NB_CNT_WORDS];
   __shared__ uint32_t cnt2[DELTA ? FV_NB_CNT_WORDS : 4];
   __shared__ uint16_t list[FV_SP_LIST_CAP];
-  __shared__ uint32_t ord[FV_SP_STAGE];
+  // window ids of a grouping step (at most 64 * FV_SP_THREADS windows, and the padding row behind them)
+  // fit 16 bits: the smaller array lets one more block share a compute unit
+  static_assert(64 * FV_SP_THREADS < 65536, "ids of a grouping step fit 16 bits");
+  typedef typename std::conditional<GROUPING, uint16_t, uint32_t>::type ord_t;
+  __shared__ ord_t ord[FV_SP_STAGE];
   __shared__ uint32_t sh_pos;
+  __shared__ float sh_xx;
+  __shared__ float sc64[GROUPING ? 64 : 1];  // activations of a neuron with up to 64 windows, by rank
   __shared__ float wave_max[16];
+  __shared__ uint32_t red[17];
   constexpr uint32_t T = FV_SP_THREADS;
   const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT;
   const uint32_t q = blockIdx.x & (FV_NB_CLASSES - 1);
   const uint32_t tid = threadIdx.x;
-  const uint32_t c_h = a.group_count[h];
+  uint32_t c_h, base, my_off = 0, r0 = 0;
+  bool sc_complete = true;  // every thread's matches have their activations in pf[]
+  uint64_t mask = 0;
+  constexpr int PF = 4;
+  float pf[PF];
+  if (GROUPING) {
+    const uint32_t n = a.n;
+    // thread t takes windows 64 t .. 64 t + 63: two words of the neuron's row
+    r0 = 64 * tid;
+    uint2 mw = make_uint2(0u, 0u);
+    if (2 * tid < a.won_words) mw = *(const uint2 *)(a.won + (uint64_t)h * a.won_words + 2 * tid);
+    // Windows won by lower neurons: 16-byte pieces of the 16-bit winner array dealt over the threads,
+    // two winners compared per operation (winner - h is negative in a 16-bit half exactly where the
+    // winner is lower; both are below 2^15). The entries behind the step's last window, up to the
+    // end of its piece, hold 0x7fff.
+    const uint32_t n8 = (n + 7) / 8;
+    const fv_short2 hh = {(short)h, (short)h};
+    fv_short2 below = {0, 0};
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {  // n <= 8 * 8 * T
+      if (g * T < n8) {            // the same answer in the whole block
+        const uint32_t i4 = tid + g * T;
+        int4 v = ((const int4 *)a.win)[min(i4, n8 - 1)];
+        if (i4 >= n8) v = make_int4(0x7fff7fff, 0x7fff7fff, 0x7fff7fff, 0x7fff7fff);
+        below += (__builtin_bit_cast(fv_short2, v.x) - hh) >> 15;
+        below += (__builtin_bit_cast(fv_short2, v.y) - hh) >> 15;
+        below += (__builtin_bit_cast(fv_short2, v.z) - hh) >> 15;
+        below += (__builtin_bit_cast(fv_short2, v.w) - hh) >> 15;
+      }
+    }
+    const uint32_t lt = (uint32_t)(-((int)below.x + (int)below.y));
+    mask = (uint64_t)mw.x | ((uint64_t)mw.y << 32);
+    const uint32_t eq = (uint32_t)__popcll(mask);
+    if (q == 0) {
+      if (2 * tid < a.won_words) *(uint2 *)(a.won_clear + (uint64_t)h * a.won_words + 2 * tid) = make_uint2(0u, 0u);
+    }
+    // the scaled activations of a thread's first matches travel while the scan runs
+    uint64_t mm = mask;
+#pragma unroll
+    for (int e = 0; e < PF; ++e) {
+      const uint32_t r = mm ? r0 + (uint32_t)__ffsll((long long)mm) - 1 : r0;
+      pf[e] = a.sc[min(r, n - 1)];
+      mm &= mm - 1;
+    }
+    // one block scan carries both counts as the halves of a word, and tells whether any thread has
+    // more matches than it has fetched activations for
+    const bool wave_more = __ballot(eq > (uint32_t)PF) != 0ull;
+    const uint32_t v = lt | (eq << 16);
+    const uint32_t incl = fv_wave_inclusive_scan_u32(v);
+    if ((tid & 63u) == 63u) red[tid >> 6] = incl, red[8 + (tid >> 6)] = wave_more;
+    fv_lds_barrier();
+    uint32_t before = 0, total = 0;
+    bool more = false;
+#pragma unroll
+    for (uint32_t i = 0; i < T / 64; ++i) {
+      const uint32_t t = red[i];
+      before += i < (tid >> 6) ? t : 0u;
+      total += t;
+      more = more || red[8 + i] != 0;
+    }
+    before += incl - v;
+    base = total & 0xffffu;
+    c_h = total >> 16;
+    my_off = before >> 16;
+    sc_complete = !more;
+    for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+    if (q == 0 && tid == 0) {
+      a.group_base_out[h] = base;
+      a.group_count_out[h] = c_h;
+      if (c_h == 0) a.xx_out[h] = 0.0f;
+    }
+  } else {
+    c_h = a.group_count[h];
+  }
   const uint32_t c2_h = DELTA ? a.group_count2[h] : 0u;
   if (c_h == 0 && c2_h == 0) {
     if (tid == 0) {
@@ -682,24 +797,96 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
   // The launch lasts as long as its few heaviest blocks: their waves go first wherever they share a
   // SIMD with the waves of light blocks.
   if (c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
-  const uint32_t base = a.group_base[h];
+  if (!GROUPING) base = a.group_base[h];
   const uint32_t base2 = DELTA ? a.group_base2[h] : 0u;
-  const float x_h = a.xx[h];
+  float x_h = GROUPING ? 0.0f : a.xx[h];
   float ds_max = 0.0f;
-  const uint32_t *__restrict__ order = a.order + base;
+  const uint32_t *order = (GROUPING ? a.order_out : a.order) + base;  // GROUPING: also written here, through order_out
   const uint32_t n_cols = 2 * a.V;
   const uint32_t m_ent = max(c_h, c2_h) * a.w;
   // the block's records: no more than (c_h + c2_h) * w of them, behind those of the lower neurons
   const uint64_t slot_first = (uint64_t)q * a.slot_stride + (uint64_t)(base + base2) * a.w;
   fv_slot *slots = a.slots + slot_first;
 
-  for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
-  if (DELTA)
-    for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt2)[i] = make_uint4(0, 0, 0, 0);
   const bool staged_once = !DELTA && c_h <= FV_SP_STAGE;  // the usual case: the neuron's window ids are staged here
-  if (staged_once)
-    for (uint32_t i = tid; i < c_h; i += T) ord[i] = order[i];
-  fv_lds_barrier();
+  if (!GROUPING) {
+    for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+    if (DELTA)
+      for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt2)[i] = make_uint4(0, 0, 0, 0);
+  }
+  // xx[h] is added up in the grouping kernel's order: lane l of the first wave adds the values number
+  // l, l + 64, ... onto 0, then the partial sums are added onto 0 in lane order (those of the lanes
+  // from c_h on are +0 and change nothing). A neuron with up to 64 windows, each thread holding the
+  // activations of all its matches, does that behind the counting pass, where the value is first
+  // needed and the loads have long returned.
+  bool xx_pending = GROUPING && staged_once && sc_complete && c_h <= 64;
+  if (GROUPING) {
+    // Window ids by rank: into LDS, or (more than LDS stages) to the neuron's part of order[], where
+    // the neuron's four blocks write the same values.
+    uint32_t rank = my_off;
+    for (uint64_t mm = mask; mm; mm &= mm - 1) {
+      const uint32_t r = r0 + (uint32_t)__ffsll((long long)mm) - 1;
+      if (staged_once)
+        ord[rank++] = (ord_t)r;
+      else
+        a.order_out[base + rank++] = r;
+    }
+    if (!xx_pending) {
+      // A neuron with many windows: the activations are fetched by rank into the counter array
+      // (cleared behind the block scan, and again by the first wave once it has added them).
+      static_assert(FV_SP_STAGE <= FV_NB_CNT_WORDS && FV_SP_STAGE % 64 == 0 && FV_SP_STAGE <= 8 * T,
+                    "a stage of activations fits the counters and one trip to memory");
+      float *scbuf = (float *)cnt;
+      float part = 0.0f;
+      if (staged_once)
+        fv_lds_barrier();  // the ids are in LDS
+      else
+        __syncthreads();  // the ids are in memory
+      for (uint32_t j0 = 0; j0 < c_h; j0 += FV_SP_STAGE) {
+        const uint32_t mr = min(c_h - j0, (uint32_t)FV_SP_STAGE);
+        float v8[8];  // eight loads in flight per thread
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const uint32_t j = j0 + min(tid + u * T, mr - 1);
+          v8[u] = a.sc[staged_once ? (uint32_t)ord[j] : order[j]];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (tid + u * T < mr) scbuf[tid + u * T] = v8[u];
+        fv_lds_barrier();
+        if (tid < 64) {
+          uint32_t j = tid;
+          for (; j + 192 < mr; j += 256) {  // four values fetched together, added one after the other
+            const float v0 = scbuf[j], v1 = scbuf[j + 64], v2 = scbuf[j + 128], v3 = scbuf[j + 192];
+            part = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(part, v0), v1), v2), v3);
+          }
+          for (; j < mr; j += 64) part = __fadd_rn(part, scbuf[j]);
+        }
+        if (j0 + FV_SP_STAGE < c_h) fv_lds_barrier();  // before the next stage overwrites this one
+      }
+      if (tid < 64) {
+        float xx = 0.0f;
+        if (c_h >= 64) {
+#pragma unroll
+          for (int l = 0; l < 64; ++l) xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), l)));
+        } else {
+          for (uint32_t l = 0; l < c_h; ++l)
+            xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), (int)l)));
+        }
+        if (tid == 0) {
+          sh_xx = xx;
+          if (q == 0) a.xx_out[h] = xx;
+        }
+        const uint32_t used = (min(c_h, (uint32_t)FV_SP_STAGE) + 3) / 4;
+        for (uint32_t i = tid; i < used; i += 64) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+      }
+    }
+    // the counting pass starts behind a barrier; sh_xx is read behind that pass
+  } else {
+    if (staged_once)
+      for (uint32_t i = tid; i < c_h; i += T) ord[i] = (ord_t)order[i];
+    fv_lds_barrier();
+  }
 
   // No counter can exceed the neuron's number of window positions: below 2^16 of them, two 16-bit
   // counters share a word and one pass covers twice as many columns.
@@ -710,20 +897,20 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
 
   for (uint32_t lo = 0; lo < class_cols; lo += span) {
     for (int l = 0; l < (DELTA ? 2 : 1); ++l) {
-      const uint32_t *__restrict__ ids = l == 0 ? order : a.order2 + base2;
+      const uint32_t *ids = l == 0 ? order : a.order2 + base2;
       const uint32_t n_ids = l == 0 ? c_h : c2_h;
       uint32_t *counters = l == 0 ? cnt : cnt2;
       for (uint32_t j0 = 0; j0 < n_ids; j0 += FV_SP_STAGE) {
         const uint32_t n_staged = min(n_ids - j0, (uint32_t)FV_SP_STAGE);
         if (!staged_once) {
           fv_lds_barrier();  // the previous part has been counted
-          for (uint32_t i = tid; i < n_staged; i += T) ord[i] = ids[j0 + i];
+          for (uint32_t i = tid; i < n_staged; i += T) ord[i] = (ord_t)ids[j0 + i];
           fv_lds_barrier();
         }
         if (narrow)
-          fv_sparse_count_any<true>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
+          fv_sparse_count_any<true, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
         else
-          fv_sparse_count_any<false>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
+          fv_sparse_count_any<false, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
       }
     }
     // Every non-zero counter is one distinct element. Their positions are collected in LDS, up to
@@ -732,7 +919,30 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
     uint32_t found;
     do {
       if (tid == 0) sh_pos = 0;
+      if (GROUPING && xx_pending) {
+        uint32_t rk = my_off;
+        uint64_t mm = mask;
+#pragma unroll
+        for (int e = 0; e < PF; ++e)
+          if (mm) {
+            sc64[rk++] = pf[e];
+            mm &= mm - 1;
+          }
+      }
       fv_lds_barrier();
+      if (GROUPING && xx_pending) {
+        if (tid < 64) {
+          const float part = tid < c_h ? __fadd_rn(0.0f, sc64[tid]) : 0.0f;
+          float xx = 0.0f;
+          for (uint32_t l = 0; l < c_h; ++l)
+            xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), (int)l)));
+          if (tid == 0) {
+            sh_xx = xx;
+            if (q == 0) a.xx_out[h] = xx;
+          }
+        }
+        xx_pending = false;
+      }
       {
         // bit 8 * i + u of `mine`: counter u of the thread's i-th group of four words is non-zero
         constexpr int n_groups = (FV_NB_CNT_WORDS / 4 + T - 1) / T;
@@ -782,6 +992,7 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
       }
       fv_lds_barrier();
       found = sh_pos;
+      if (GROUPING) x_h = sh_xx;
       const uint32_t take = min(found, (uint32_t)FV_SP_LIST_CAP);
       // one element per thread (four in flight): save its weight and its count in a slot record,
       // plant the sentinel, take |ds| (the dense term plus count additions of 1/f; a row with
@@ -1415,6 +1626,7 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   (void)hipFree(t->bmax);
   (void)hipFree(t->win);
   (void)hipFree(t->win16);
+  (void)hipFree(t->won[0]);
   fv_trainer_free_delta(t);
   (void)hipFree(t->sc);
   (void)hipFree(t->xx);
@@ -1452,6 +1664,13 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMemsetAsync(t->win, 0, ((size_t)t->B + 16) * sizeof(int32_t), t->stream));
   FV_HIP(hipMalloc((void **)&t->win16, ((size_t)t->B + 64) * sizeof(uint16_t)));  // read in 16-byte pieces
   FV_HIP(hipMemsetAsync(t->win16, 0, ((size_t)t->B + 64) * sizeof(uint16_t), t->stream));
+  if (t->B <= 64 * FV_SP_THREADS) {  // steps of such a trainer can be grouped inside the sparse launch
+    t->won_words = 2 * ((t->B + 63) / 64);
+    const size_t row_words = (size_t)t->K * t->won_words;
+    FV_HIP(hipMalloc((void **)&t->won[0], 2 * row_words * sizeof(uint32_t)));
+    t->won[1] = t->won[0] + row_words;
+    FV_HIP(hipMemsetAsync(t->won[0], 0, 2 * row_words * sizeof(uint32_t), t->stream));
+  }
   FV_HIP(hipMalloc((void **)&t->scalars, 16 * sizeof(float)));
   FV_HIP(hipMemsetAsync(t->Wt, 0, elems * sizeof(float), t->stream));
   FV_HIP(hipMemsetAsync(t->xx, 0, (size_t)t->ldk * sizeof(float), t->stream));
@@ -1760,7 +1979,7 @@ static int fv_trainer_alloc_delta(fv_trainer *t) {
 }
 
 static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps, float delta, hipEvent_t *ev,
-                           unsigned which = 0x3f) {
+                           unsigned which = 0x3f, bool repeated = false) {
   const bool anti = delta != 0.0f;  // the second neuron of every window takes part (flyvec/src/cuda_funcs.cu:726-734)
   if (anti) FV_TRY(fv_trainer_alloc_delta(t));
   fv_gather_args g;
@@ -1787,6 +2006,24 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.lmid = t->cfg.lmid;
   g.lbase = t->cfg.lbase;
   const bool weighted = t->cfg.lmid != 1.0f || t->cfg.lbase != 1.0f;
+  // A step of a trainer with up to 64 windows per thread of a class block, without the anti-Hebbian
+  // term, has no grouping launch: the winner kernel marks every window in its winner's bit row, and
+  // the sparse launch's blocks group for themselves from those rows. A whole step takes the pair of
+  // buffers the last such step's sparse launch has cleared; a launch on its own (measurement) stays
+  // on the last step's pair, cleared here first unless it repeats the launch before it.
+  const bool grouping_in_sparse =
+      which == 0x3f ? !anti && t->won[0] && !t->separate_grouping : t->last_grouped_in_sparse;
+  if (which == 0x3f) t->last_grouped_in_sparse = grouping_in_sparse;
+  g.won = nullptr;
+  g.won_words = t->won_words;
+  if (grouping_in_sparse) {
+    if (which == 0x3f) {
+      t->won_parity ^= 1u;
+    } else if ((which & 1u) && !repeated) {
+      FV_HIP(hipMemsetAsync(t->won[t->won_parity], 0, (size_t)t->K * t->won_words * sizeof(uint32_t), t->stream));
+    }
+    g.won = t->won[t->won_parity];
+  }
   // a whole step whose windows the previous one has sampled ahead takes that buffer
   const bool whole = which == 0x3f;
   g.sampled = 0;
@@ -1834,7 +2071,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
       gr.scale = -delta;
       gr.accumulate = 1;
     }
-    if (which & 2u) {
+    if ((which & 2u) && !grouping_in_sparse) {
       if (n <= 64 * gr_threads && n < 65536)
         hipLaunchKernelGGL(fv_group_kernel<true>, dim3(t->K), dim3(gr_threads), 0, t->stream, gr);
       else
@@ -1866,11 +2103,24 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.ldk = t->ldk;
   sp.w = t->w;
   sp.V = (uint32_t)t->V;
+  sp.won = t->won[t->won_parity];
+  sp.win = t->win16;
+  sp.won_words = t->won_words;
+  sp.won_clear = t->won[t->won_parity ^ 1u];
+  sp.sc = t->sc;
+  sp.n = n;
+  sp.order_out = t->order;
+  sp.group_base_out = t->group_base;
+  sp.group_count_out = t->group_count;
+  sp.xx_out = t->xx;
   if (which & 4u) {
+    const dim3 sp_grid(t->K * FV_NB_CLASSES), sp_block(FV_SP_THREADS);
     if (anti)
-      hipLaunchKernelGGL(fv_sparse_kernel<true>, dim3(t->K * FV_NB_CLASSES), dim3(FV_SP_THREADS), 0, t->stream, sp);
+      hipLaunchKernelGGL((fv_sparse_kernel<true, false>), sp_grid, sp_block, 0, t->stream, sp);
+    else if (grouping_in_sparse)
+      hipLaunchKernelGGL((fv_sparse_kernel<false, true>), sp_grid, sp_block, 0, t->stream, sp);
     else
-      hipLaunchKernelGGL(fv_sparse_kernel<false>, dim3(t->K * FV_NB_CLASSES), dim3(FV_SP_THREADS), 0, t->stream, sp);
+      hipLaunchKernelGGL((fv_sparse_kernel<false, false>), sp_grid, sp_block, 0, t->stream, sp);
   }
   if (ev) FV_HIP(hipEventRecord(ev[3], t->stream));
   fv_dense_args d;
@@ -2036,6 +2286,19 @@ extern "C" int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches) {
   return FV_OK;
 }
 
+extern "C" int fv_trainer_set_grouping_launch(fv_trainer *t, uint32_t separate) {
+  FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
+  FV_REQUIRE(separate <= 1, FV_ERR_INVALID, "separate must be 0 or 1");
+  t->separate_grouping = separate != 0;
+  return FV_OK;
+}
+
+extern "C" int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate) {
+  FV_REQUIRE(t && out_separate, FV_ERR_INVALID, "null argument");
+  *out_separate = (t->won[0] && !t->separate_grouping) ? 0u : 1u;
+  return FV_OK;
+}
+
 extern "C" int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches) {
   FV_REQUIRE(t && out_launches, FV_ERR_INVALID, "null argument");
   *out_launches = t->onepass && fv_trainers_alive.load() == 1 ? 1u : 2u;
@@ -2142,8 +2405,11 @@ extern "C" int fv_trainer_time_kernel(fv_trainer *t, uint32_t kernel_index, uint
   int rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, t->last_delta, nullptr, 1u << kernel_index);  // warm-up
   FV_HIP(hipEventRecord(e0, t->stream));
   for (uint32_t r = 0; r < reps && rc == FV_OK; ++r)
-    rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, t->last_delta, nullptr, 1u << kernel_index);
+    rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, t->last_delta, nullptr, 1u << kernel_index, true);
   FV_HIP(hipEventRecord(e1, t->stream));
+  // the repeated winner launches have counted every window many times: once more from cleared buffers
+  if (kernel_index == 0 && rc == FV_OK)
+    rc = fv_enqueue_step(t, t->last_first, t->last_n, t->last_eps, t->last_delta, nullptr, 1u);
   FV_HIP(hipStreamSynchronize(t->stream));
   float ms = 0.0f;
   FV_HIP(hipEventElapsedTime(&ms, e0, e1));

@@ -148,6 +148,18 @@ class Trainer:
         2: two launches, 0: as chosen at creation.  Same results either way."""
         check(self.lib.fv_trainer_set_dense_launches(self.handle, int(launches)))
 
+    def set_grouping_launch(self, separate):
+        """True: the windows are grouped by winner in a launch of its own; False: inside the
+        sparse-element launch where the step allows it.  Same results either way."""
+        check(self.lib.fv_trainer_set_grouping_launch(self.handle, 1 if separate else 0))
+
+    @property
+    def grouping_launch(self):
+        """True when a step without the anti-Hebbian term groups in a launch of its own."""
+        out = C.c_uint32(0)
+        check(self.lib.fv_trainer_get_grouping_launch(self.handle, C.byref(out)))
+        return bool(out.value)
+
     @property
     def dense_launches(self):
         out = C.c_uint32(0)

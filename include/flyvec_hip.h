@@ -181,6 +181,12 @@ int fv_trainer_sync(fv_trainer *t);
  * step takes two launches whatever is set here. */
 int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches);
 int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches); /* 1 or 2: the form the next step takes */
+/* Grouping the windows of a step by winner (what flyvec/src/cuda_funcs.cu:1719-1721 leaves in
+ * max_IDs and xx) runs inside the sparse-element launch when the trainer's batch is at most 16384
+ * windows and the step has no anti-Hebbian term, as a launch of its own otherwise. separate = 1 forces the launch of its
+ * own, 0 returns to that rule. Results are bit-identical either way. */
+int fv_trainer_set_grouping_launch(fv_trainer *t, uint32_t separate);
+int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate); /* the form a step without the anti-Hebbian term takes */
 /* Test hook: between its two passes a single-launch dense pass waits for all its blocks, at most
  * `rounds` polling rounds (2^14 by default, tens of milliseconds); 0 makes every block give up at once, which
  * is how the error path of fv_trainer_sync is exercised. No counterpart in the reference. */

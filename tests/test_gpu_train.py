@@ -683,3 +683,87 @@ def test_dense_launch_forms_agree_over_an_epoch_of_the_headline_shape(gpu):
         t.close()
     assert np.isfinite(got[1]).all() and not np.array_equal(got[1], W0)
     assert np.array_equal(got[1], got[2])
+
+
+@pytest.mark.parametrize("V,K,w,B,steps", [
+    (300, 64, 7, 128, 6),        # a few windows per neuron
+    (500, 2, 5, 6000, 3),        # two neurons: each wins more windows than LDS stages at once
+    (800, 8, 11, 4096, 3),       # hundreds of windows per neuron: activations fetched by rank
+    (2000, 400, 11, 16384, 2),   # the largest batch the sparse launch groups for itself
+    (300, 70, 64, 200, 3),       # the widest window
+])
+def test_grouping_forms_agree_and_match_the_oracle(gpu, oracle_lib, V, K, w, B, steps):
+    """Grouping by winner inside the sparse launch (bit rows left by the winner kernel) and as a launch of
+    its own give the same matrix, xx and winners, bit for bit, and both equal the oracle's; a shorter
+    last step and a switch of form between steps are part of the run."""
+    from flyvec_amd import synthetic
+    to = oracle_lib
+    tokens, offsets = small_corpus(max(40000, 3 * B * steps), V, seed=3)
+    W0 = synthetic.synapses(K, V, seed=9)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    got = {}
+    for form in ("inside", "separate", "alternating"):
+        t, perm = make_trainer(tokens, offsets, V, K, w, B, W0)
+        assert t.grouping_launch is False
+        t.set_grouping_launch(form == "separate")
+        assert t.grouping_launch is (form == "separate")
+        first = 0
+        for s in range(steps):
+            if form == "alternating":
+                t.set_grouping_launch(s % 2 == 1)
+            n = B if s + 1 < steps else max(1, B // 3 + 1)
+            t.step(first, n, 1e-3)
+            first += n
+        got[form] = (t.get_weights(), t.winners(n).copy(), t.step_stats())
+        t.close()
+    for form in ("separate", "alternating"):
+        assert np.array_equal(got["inside"][0], got[form][0])
+        assert np.array_equal(got["inside"][1], got[form][1])
+        assert np.array_equal(got["inside"][2][0], got[form][2][0]) and got["inside"][2][1] == got[form][2][1]
+    Wo = W0.copy()
+    first = 0
+    for s in range(steps):
+        n = B if s + 1 < steps else max(1, B // 3 + 1)
+        to.train_steps(Wo, tokens, starts, perm, first, n, 1, w, invf, 1e-3, 1e-30)
+        first += n
+    assert np.array_equal(got["inside"][0], Wo)
+
+
+def test_batches_beyond_the_grouping_limit_take_the_separate_launch(gpu):
+    from flyvec_amd import Trainer, _lib
+    t = Trainer(300, 16, 5, 16385)
+    assert t.grouping_launch is True
+    t.set_grouping_launch(False)            # the rule, not a promise
+    assert t.grouping_launch is True
+    with pytest.raises(_lib.FlyvecError) as e:
+        _lib.check(t.lib.fv_trainer_set_grouping_launch(t.handle, 2))
+    assert e.value.code == _lib.FV_ERR_INVALID
+    t.close()
+
+
+def test_measurement_launches_leave_the_grouping_buffers_consistent(gpu, oracle_lib):
+    """time_kernels repeats single kernels of the last step (the winner kernel many times over the same bit
+    rows); the steps that follow still equal the oracle's from the matrix the measurement left."""
+    from flyvec_amd import synthetic
+    to = oracle_lib
+    V, K, w, B = 600, 96, 9, 1500
+    tokens, offsets = small_corpus(60000, V, seed=4)
+    W0 = synthetic.synapses(K, V, seed=2)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    for launches in (1, 2):
+        t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, launches=launches)
+        for s in range(3):
+            t.step(s * B, B, 1e-3)
+        t.time_kernels(reps=3)                 # leaves W in a state of its own
+        W1 = t.get_weights()
+        finite = np.isfinite(W1).all()
+        if not finite:                         # sentinels planted by the repeated sparse launch: start afresh
+            t.set_weights(W0)
+            W1 = W0.copy()
+        for s in range(3, 6):
+            t.step(s * B, B, 1e-3)
+        Wg = t.get_weights()
+        t.close()
+        Wo = W1.copy()
+        to.train_steps(Wo, tokens, starts, perm, 3 * B, B, 3, w, invf, 1e-3, 1e-30)
+        assert np.array_equal(Wg, Wo)
