@@ -47,25 +47,25 @@ HASH = dict(K=400, V=20000, w=11, k=32, n=1 << 20)
 # WRITE_SIZE reads them all: x1.0). Traffic below the algorithmic bytes means the rest was served
 # by the L2 caches.
 MEASURED_TRAFFIC = {
-    "dense_max_update": (33326.2 * 2.0 + 65231.5) * 1024,
-    "gather_winner": (28495.7 * 2.0 + 503.2) * 1024,
-    "sparse_owners": (4607.5 * 2.0 + 2483.7) * 1024,
-    "group_xx": (310.0 * 2.0 + 87.2) * 1024,
-    "hash": (2477777.6 * 2.0 + 82452.4) * 1024,
-    # the passes over W as two launches and the slot launch (--dense-launches 2)
-    "update": (32193.9 * 2.0 + 62498.2) * 1024,
-    "absmax_ds": (31270.0 * 2.0 + 64.0) * 1024,
-    "slot_update": (622.6 * 2.0 + 1501.2) * 1024,
+    "dense_max_update": (33303.5 * 2.0 + 65249.7) * 1024,
+    "gather_winner": (28514.5 * 2.0 + 817.5) * 1024,
+    "sparse_owners": (5819.5 * 2.0 + 2993.3) * 1024,  # grouping by winner included
+    "hash": (2478239.7 * 2.0 + 82381.6) * 1024,
+    # the step as six launches (--dense-launches 2 --separate-grouping)
+    "update": (32309.5 * 2.0 + 62498.2) * 1024,
+    "absmax_ds": (31275.5 * 2.0 + 64.0) * 1024,
+    "slot_update": (621.9 * 2.0 + 1501.2) * 1024,
+    "group_xx": (312.9 * 2.0 + 87.2) * 1024,
 }
 
 # the same for --workload large-step (profiles/train_step_K1000_V50000_B50000.txt)
 MEASURED_TRAFFIC_LARGE = {
-    "gather_winner": (759026.2 * 2.0 + 5566.8) * 1024,
-    "group_xx": (1246.9 * 2.0 + 316.0) * 1024,
-    "sparse_owners": (32998.9 * 2.0 + 18007.4) * 1024,
-    "absmax_ds": (195342.3 * 2.0 + 68.0) * 1024,
-    "update": (195628.9 * 2.0 + 390612.4) * 1024,
-    "slot_update": (3551.5 * 2.0 + 11354.9) * 1024,
+    "gather_winner": (760768.6 * 2.0 + 5100.7) * 1024,
+    "group_xx": (1249.9 * 2.0 + 316.0) * 1024,
+    "sparse_owners": (30823.7 * 2.0 + 17905.1) * 1024,
+    "absmax_ds": (195347.6 * 2.0 + 67.9) * 1024,
+    "update": (195624.6 * 2.0 + 390612.4) * 1024,
+    "slot_update": (3550.7 * 2.0 + 11373.4) * 1024,
 }
 
 # the two passes over W of a step (and the sparse elements' update) as one launch: W stays in

@@ -2,8 +2,8 @@
 //
 // Replaces the kernel chain of flyvec/src/cuda_funcs.cu:1662-1803 (sparse input, frequency
 // scaling, p = 2; delta, Lmid / Lbase and the pruning sampler included).  The reference
-// materialises ds (K x N) and walks it five times per step; here ds is never stored and nothing
-// uses global atomics:
+// materialises ds (K x N) and walks it five times per step; here ds is never stored and the only
+// global atomic is the OR that marks a window in its winner's bit row:
 //
 //   1. gather+winner   one wavefront per window: sampler (cuda_funcs.cu:915-936), raw
 //                      activation = sum of ~w token rows of the token-major matrix with the K
@@ -13,6 +13,9 @@
 //   2. group + xx      one block per neuron h: the ordered list of the windows h won and xx[h], the
 //                      sum of their scaled activations (:722-744 -- the reference's atomic order
 //                      is undefined, this one is fixed, so a step is reproducible bit for bit).
+//                      A launch of its own only for batches beyond 16384 windows and for steps
+//                      with the anti-Hebbian term: otherwise the blocks of launch 3 do it
+//                      themselves, from the bit rows launch 1 leaves.
 //   3. sparse owners   four blocks per neuron, one per column class: the sparse Hebbian term of
 //                      row h (:657-672). A block alone owns its elements (h, column), so it counts
 //                      repeated columns in LDS and for each distinct one saves the true weight and
