@@ -690,11 +690,12 @@ __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uin
 
 // DELTA: the neuron's elements are counted over two lists of windows, those it won and those in
 // which it came second, into two counter arrays; a record carries both counts.
-// GROUPING: no grouping launch has run. Every class block scans the winner array like the grouping
-// kernel's block of its neuron (a thread's run is at most 64 windows: the step has no more than
-// 64 * FV_SP_THREADS), stages the neuron's window ids in LDS straight from the scan, and adds the
-// neuron's scaled activations in the grouping kernel's order; the block of class 0 leaves xx[h],
-// the neuron's count and its base for the dense launch.
+// GROUPING: no grouping launch has run. Every class block takes its neuron's windows from the bit row
+// the winner kernel has filled (a thread's two words are 64 windows: the step has no more than
+// 64 * FV_SP_THREADS), counts the windows of lower neurons in the 16-bit winner array, stages the
+// window ids in LDS by rank, and adds the neuron's scaled activations in the grouping kernel's order;
+// the block of class 0 leaves xx[h], the neuron's count and its base for the dense launch and clears
+// the neuron's row of the other bit-row buffer.
 template <bool DELTA, bool GROUPING>
 __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
   static_assert(!(DELTA && GROUPING), "the anti-Hebbian form has its two lists grouped by launches of their own");

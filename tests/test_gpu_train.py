@@ -671,18 +671,20 @@ def test_dense_launch_forms_agree_over_an_epoch_of_the_headline_shape(gpu):
     tokens, offsets = synthetic.corpus(18_000_000, V)
     W0 = synthetic.synapses(K, V, seed=5)
     got = {}
-    for launches in (1, 2):
+    for launches, separate in ((1, False), (2, False), (1, True)):
         t = Trainer(V, K, w, B, initial_learning_rate=2e-4)
         t.set_dense_launches(launches)
+        t.set_grouping_launch(separate)      # grouped inside the sparse launch, or by a launch of its own
         t.set_corpus(tokens, offsets)
         assert t.num_windows // B >= 1100
         t.set_weights(W0)
         t.shuffle(11)
         t.run_epoch(0, 15)
-        got[launches] = t.get_weights()
+        got[launches, separate] = t.get_weights()
         t.close()
-    assert np.isfinite(got[1]).all() and not np.array_equal(got[1], W0)
-    assert np.array_equal(got[1], got[2])
+    assert np.isfinite(got[1, False]).all() and not np.array_equal(got[1, False], W0)
+    assert np.array_equal(got[1, False], got[2, False])
+    assert np.array_equal(got[1, False], got[1, True])
 
 
 @pytest.mark.parametrize("V,K,w,B,steps", [
