@@ -172,16 +172,21 @@ extern "C" int fv_hasher_create(const float *W, uint32_t hid, uint64_t n_columns
   h->K = hid;
   h->ldk = fv_ldk(hid);
   h->N = n_columns;
+  if (fv_matrix_gather_reach(h->K, h->N) > fv_matrix_alloc_elems(h->K, h->N)) {
+    delete h;
+    return fv_fail(FV_ERR_INVALID, "a gather of a %u x %llu matrix would read past its allocation", hid,
+                   (unsigned long long)n_columns);
+  }
   int cus = 0;
   int rc = fv_device_info(nullptr, 0, &cus, nullptr);
   h->max_blocks = (unsigned)(cus > 0 ? cus : 256) * 8;
   hipError_t e = hipSuccess;
   if (rc == FV_OK) {
     e = hipStreamCreate(&h->stream);
-    // the rows behind the matrix that the gather reads for masked positions and past K: zeros
-    if (e == hipSuccess) e = hipMalloc((void **)&h->Wt, (size_t)(h->N + FV_PAD_ROWS) * h->ldk * sizeof(float));
+    // behind the matrix, what the gather reads for masked positions and in its lanes past K: zeros
+    if (e == hipSuccess) e = hipMalloc((void **)&h->Wt, (size_t)fv_matrix_alloc_elems(h->K, h->N) * sizeof(float));
     if (e == hipSuccess)
-      e = hipMemsetAsync(h->Wt + (size_t)h->N * h->ldk, 0, (size_t)FV_PAD_ROWS * h->ldk * sizeof(float), h->stream);
+      e = hipMemsetAsync(h->Wt + (size_t)h->N * h->ldk, 0, (size_t)fv_matrix_pad_elems(h->K) * sizeof(float), h->stream);
     if (e == hipSuccess) e = hipMalloc((void **)&h->err, sizeof(uint32_t));
     if (e == hipSuccess) e = hipMemsetAsync(h->err, 0, sizeof(uint32_t), h->stream);
     if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "hasher allocation failed: %s", hipGetErrorString(e));

@@ -7,6 +7,7 @@
 #include <stdio.h>
 
 #include "flyvec_hip.h"
+#include "fv_layout.h"
 
 #define FV_WAVE 64
 #define FV_MAX_HID 2048   // 32 values per lane in the wave-per-window kernels
@@ -37,9 +38,8 @@ void fv_clear_error();
 
 // ---- device layout of the synapse matrix -----------------------------------------
 // Token-major: column i of the K x N checkpoint matrix is the contiguous row
-// Wt[i * ldk .. i * ldk + K), ldk = K rounded up to a multiple of 4 floats so every
-// row starts 16-byte aligned; the pad is kept at zero.
-static inline uint32_t fv_ldk(uint32_t K) { return (K + 3u) & ~3u; }
+// Wt[i * ldk .. i * ldk + K), ldk = K rounded up to a multiple of 4 floats (fv_ldk) so every
+// row starts 16-byte aligned; the pad is kept at zero. fv_layout.h sizes the allocation.
 
 // K x N row-major (staging, device) <-> token-major N x ldk (device). Asynchronous.
 int fv_launch_to_token_major(const float *W_rowmajor_dev, float *Wt_dev, uint32_t K, uint64_t N,
@@ -159,18 +159,16 @@ __device__ __forceinline__ uint32_t fv_wave_sum_u32(uint32_t v) {
 
 // ---- gather-sum of one window, shared by the training and the hashing kernel ----------------
 // Lane l holds neurons l, l + 64, ... of the window's activation. acc[j] += W[idx_c][l + 64 j]
-// for every window position c in order (idx_c is held by lane c of idx_lane). The matrix carries
-// FV_PAD_ROWS rows behind its n_cols real ones: row n_cols is all zeros and is what a position
-// whose index is outside [0, n_cols) reads (adding +0 leaves a sum that started at +0 unchanged),
-// and lanes past K read on into the following row (the last one is never written) and accumulate
-// values nobody uses. So every load is unconditional and no value is selected afterwards: a
+// for every window position c in order (idx_c is held by lane c of idx_lane). The allocation
+// carries zeros behind its n_cols real rows (fv_matrix_alloc_elems): row n_cols is all zeros and is
+// what a position whose index is outside [0, n_cols) reads (adding +0 leaves a sum that started at
+// +0 unchanged), and lanes past K read on into what follows, up to fv_matrix_gather_reach, and
+// accumulate values nobody uses. So every load is unconditional and no value is selected afterwards: a
 // batch of RB rows is RB * NV independent loads in flight per lane with no branch between them,
 // and one conversion and one addition per element.
 // WEIGHTED: every weight is first multiplied, in fp32, by the weight of its window position --
 // l_mid for the centre, whose column lies in the second half of the columns, l_base for the others
 // (flyvec/src/cuda_funcs.cu:266-286).
-#define FV_PAD_ROWS 2
-
 template <int NV, int RB, typename Acc, bool WEIGHTED = false>
 __device__ __forceinline__ void fv_gather_batch(const float *__restrict__ Wt, uint32_t ldk, uint32_t n_cols, int lane,
                                                 int c0, int32_t idx_lane, Acc (&acc)[NV], float l_mid = 1.0f,

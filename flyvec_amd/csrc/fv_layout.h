@@ -1,0 +1,37 @@
+// Size of the device allocation that holds the token-major synapse matrix, and the farthest element
+// a window gather reads from it. Plain C: the kernels' host code and the CPU test-suite both use it.
+//
+// The matrix is N rows (one per column of the K x N checkpoint matrix) of ldk floats, ldk = K rounded
+// up to 4. A window gather (fv_gather_batch) loads, for every row it touches, the floats
+// row * ldk + lane + 64 * j for all 64 lanes and j < NV = ceil(K / 64), with no bound on the lane: the
+// values past K are accumulated and never used. The rows it touches are 0 .. N, row N being the row
+// of zeros that a masked position reads. So the farthest element read is N * ldk + 64 * NV - 1, and
+// the allocation holds N * ldk + max(FV_PAD_ROWS * ldk, 64 * NV) floats; everything behind the N real
+// rows is zero and no pass writes it. (Two rows cover the overrun only while 64 * NV <= 2 * ldk,
+// which fails for K <= 28.)
+#pragma once
+
+#include <stdint.h>
+
+#define FV_PAD_ROWS 2
+
+static inline uint32_t fv_ldk(uint32_t K) { return (K + 3u) & ~3u; }
+
+// 64-float registers per lane of a wave that holds K values.
+static inline uint32_t fv_lane_values(uint32_t K) { return (K + 63u) / 64u; }
+
+// Floats behind the N real rows.
+static inline uint64_t fv_matrix_pad_elems(uint32_t K) {
+  const uint64_t rows = (uint64_t)FV_PAD_ROWS * fv_ldk(K), reach = 64ull * fv_lane_values(K);
+  return rows > reach ? rows : reach;
+}
+
+// Floats of the whole allocation.
+static inline uint64_t fv_matrix_alloc_elems(uint32_t K, uint64_t N) {
+  return N * fv_ldk(K) + fv_matrix_pad_elems(K);
+}
+
+// One past the farthest element index a gather of rows 0 .. N reads.
+static inline uint64_t fv_matrix_gather_reach(uint32_t K, uint64_t N) {
+  return N * fv_ldk(K) + 64ull * fv_lane_values(K);
+}

@@ -1646,8 +1646,10 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
 }
 
 static int fv_trainer_alloc(fv_trainer *t) {
-  // FV_PAD_ROWS rows of zeros behind the matrix: what the gather reads for masked positions and past K
-  const size_t elems = (size_t)(t->N + FV_PAD_ROWS) * t->ldk;
+  // zeros behind the matrix: what the gather reads for masked positions and in its lanes past K
+  const size_t elems = (size_t)fv_matrix_alloc_elems(t->K, t->N);
+  FV_REQUIRE(fv_matrix_gather_reach(t->K, t->N) <= elems, FV_ERR_INVALID,
+             "a gather of a %u x %llu matrix would read past its allocation", t->K, (unsigned long long)t->N);
   FV_HIP(hipStreamCreate(&t->stream));
   FV_HIP(hipMalloc((void **)&t->Wt, elems * sizeof(float)));
   t->idx_stride = (t->w + 3u) & ~3u;

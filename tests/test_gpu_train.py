@@ -769,3 +769,59 @@ def test_measurement_launches_leave_the_grouping_buffers_consistent(gpu, oracle_
         Wo = W1.copy()
         to.train_steps(Wo, tokens, starts, perm, 3 * B, B, 3, w, invf, 1e-3, 1e-30)
         assert np.array_equal(Wg, Wo)
+
+
+def _random_case(case):
+    rng = np.random.default_rng(1000 + case)
+    c = dict(V=int(rng.integers(50, 3000)), K=int(rng.integers(1, 600)), w=int(rng.integers(1, 33)) | 1,
+             B=int(rng.integers(1, 9000)), steps=int(rng.integers(1, 4)), tie=int(rng.integers(0, 2)),
+             lmid=float(rng.choice([1.0, 1.0, 0.5, 2.0])), lbase=float(rng.choice([1.0, 1.0, 1.5])),
+             prune=bool(rng.integers(0, 2)), launches=int(rng.integers(1, 3)),
+             zipf_s=1.0 + float(rng.random()) * 0.3, sigma=float(rng.choice([0.02, 0.02, 1e-6, 0.0])))
+    c["mean_chunk"] = int(rng.integers(c["w"] + 2, 60))
+    c["last_n"] = int(rng.integers(1, c["B"] + 1))
+    return c
+
+
+@pytest.mark.parametrize("case", range(30))
+def test_random_configurations_match_the_oracle(gpu, oracle_lib, case):
+    """Seeded random combinations of shape (K, V, w, B), tie rule, position weights, duplicate pruning, dense-launch
+    form and a partial last minibatch: both grouping forms against the checker, step by step, bit for bit."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    c = _random_case(case)
+    V, K, w, B = c["V"], c["K"], c["w"], c["B"]
+    n_tokens = max(20000, 3 * B * c["steps"] + 1000)
+    tokens, offsets = synthetic.corpus(n_tokens, V, s=c["zipf_s"], mean_chunk=c["mean_chunk"],
+                                       seed_tokens=case + 3, seed_chunks=case + 4)
+    W0 = synthetic.synapses(K, V, seed=case, sigma=c["sigma"])
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    if len(starts) < B * c["steps"]:
+        pytest.skip(f"{len(starts)} windows for {c}")
+    perm = np.random.default_rng(case).permutation(len(starts)).astype(np.uint64)
+    inflate = to.inflate_prune if c["prune"] else to.inflate
+    sizes = [B] * (c["steps"] - 1) + [c["last_n"]]
+    Wo, ref = W0.copy(), []
+    first = 0
+    for n in sizes:
+        idx = inflate(tokens, starts, perm, first, n, w, V)
+        ref.append(to.train_step(Wo, idx, invf, 1e-3, tie_rule=c["tie"], lmid=c["lmid"], lbase=c["lbase"]))
+        first += n
+    for separate in (False, True):
+        t = Trainer(V, K, w, B, initial_learning_rate=1e-3, tie_rule=c["tie"], lmid=c["lmid"], lbase=c["lbase"],
+                    prune_duplicates=c["prune"])
+        t.set_dense_launches(c["launches"])
+        t.set_grouping_launch(separate)
+        t.set_corpus(tokens, offsets)
+        t.set_permutation(perm)
+        t.set_weights(W0)
+        first = 0
+        for s, n in enumerate(sizes):
+            t.step(first, n, 1e-3)
+            first += n
+            assert np.array_equal(t.winners(n), ref[s]["winners"]), f"winners, step {s}, {c}"
+            xx, nc = t.step_stats()
+            assert np.array_equal(xx, ref[s]["xx"]) and nc == ref[s]["nc"], f"xx / max|ds|, step {s}, {c}"
+        Wg = t.get_weights()
+        t.close()
+        assert np.array_equal(Wg.view(np.uint32), Wo.view(np.uint32)), f"W, separate grouping {separate}, {c}"
