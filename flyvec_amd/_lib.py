@@ -59,6 +59,7 @@ SIGNATURES = {
     "fv_count_windows": [_vp, _u64, _u64, C.POINTER(_u64)],
     "fv_build_window_starts": [_vp, _u64, _u64, _vp, _u64],
     "fv_inverse_frequency": [_vp, _u64, _u64, _vp],
+    "fv_inverse_frequency_static": [_vp, _u64, _u64, _vp],
     "fv_mask_tokens": [_vp, _u64, _vp, _u64, _u64],
     "fv_prune_windows": [_vp, _u64, _u64],
     "fv_trainer_create": [C.POINTER(TrainConfig), _pp],

@@ -323,6 +323,78 @@ extern "C" int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, ui
   return rc;
 }
 
+// ---- inverse unigram frequency without any allocation -------------------------------------------------
+// For callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+// harnesses that forbid hipMalloc): the occurrence counters and the id range live in a file-scope
+// device array instead of a buffer from hipMalloc. Every device the library runs on holds its own
+// copy of the array, at its own address, until the process ends; host code reaches it only through
+// the address hipGetSymbolAddress returns for the device that is current.
+#define FV_STATIC_MAX_VOCAB (1u << 20)  // counters of the array: 4 MiB
+#define FV_STATIC_MAX_DEVICES 64
+
+static __device__ __align__(256) uint32_t fv_static_scratch[FV_STATIC_MAX_VOCAB + 64];  // counters, then {min, max} of the ids
+static uint32_t *fv_static_scratch_addr[FV_STATIC_MAX_DEVICES];  // per device, filled on first use
+
+// The array's address on the current device.
+static int fv_static_scratch_on_device(uint32_t **out) {
+  int dev = -1;
+  FV_HIP(hipGetDevice(&dev));
+  FV_REQUIRE(dev >= 0 && dev < FV_STATIC_MAX_DEVICES, FV_ERR_INVALID, "device %d is beyond the %d this entry point serves",
+             dev, FV_STATIC_MAX_DEVICES);
+  if (!fv_static_scratch_addr[dev]) {
+    void *p = nullptr;
+    FV_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(fv_static_scratch)));
+    FV_REQUIRE(p, FV_ERR_HIP, "hipGetSymbolAddress returned no address for the scratch array");
+    fv_static_scratch_addr[dev] = (uint32_t *)p;
+  }
+  *out = fv_static_scratch_addr[dev];
+  return FV_OK;
+}
+
+// counters[0 .. vocab) = 0 and the id range to (INT_MAX, INT_MIN): a kernel, not a memset, so that a
+// caller may capture the call sequence in a graph.
+__global__ __launch_bounds__(256) void fv_static_clear_kernel(uint32_t *__restrict__ counts, uint32_t vocab,
+                                                              int32_t *__restrict__ minmax) {
+  for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < vocab; i += gridDim.x * 256) counts[i] = 0;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    minmax[0] = 0x7fffffff;
+    minmax[1] = -0x7fffffff - 1;
+  }
+}
+
+extern "C" int fv_inverse_frequency_static(const int32_t *corpus_dev, uint64_t n_tokens, uint64_t vocab,
+                                           float *out_invf_dev) {
+  FV_REQUIRE(out_invf_dev, FV_ERR_INVALID, "fv_inverse_frequency_static: null output");
+  FV_REQUIRE(corpus_dev || n_tokens == 0, FV_ERR_INVALID, "fv_inverse_frequency_static: null corpus");
+  FV_REQUIRE(vocab >= 1 && vocab <= FV_STATIC_MAX_VOCAB, FV_ERR_INVALID,
+             "fv_inverse_frequency_static: vocabulary of %llu ids; the built-in scratch array holds counters for at "
+             "most %u (use fv_inverse_frequency, which allocates)",
+             (unsigned long long)vocab, FV_STATIC_MAX_VOCAB);
+  FV_REQUIRE(n_tokens < (1ull << 32), FV_ERR_INVALID, "fv_inverse_frequency_static: corpus of %llu tokens exceeds 2^32",
+             (unsigned long long)n_tokens);
+  uint32_t *counts = nullptr;
+  FV_TRY(fv_static_scratch_on_device(&counts));
+  int32_t *minmax = (int32_t *)(counts + FV_STATIC_MAX_VOCAB);
+  hipStream_t stream = 0;
+  // the array keeps the last call's counts: clear what this call uses
+  const unsigned clear_blocks = (unsigned)((vocab + 255) / 256 < 1024 ? (vocab + 255) / 256 : 1024);
+  hipLaunchKernelGGL(fv_static_clear_kernel, dim3(clear_blocks), dim3(256), 0, stream, counts, (uint32_t)vocab, minmax);
+  if (n_tokens) {
+    const uint64_t want = (n_tokens + 256 * 16 - 1) / (256 * 16);
+    const unsigned blocks = (unsigned)(want < 1 ? 1 : (want > 2048 ? 2048 : want));
+    hipLaunchKernelGGL(fv_histogram_kernel, dim3(blocks), dim3(256), 0, stream, corpus_dev, n_tokens, (uint32_t)vocab,
+                       counts, minmax);
+  }
+  hipLaunchKernelGGL(fv_invert_counts_kernel, dim3((unsigned)((vocab + 255) / 256)), dim3(256), 0, stream, counts,
+                     (uint32_t)vocab, out_invf_dev);
+  FV_HIP(hipGetLastError());
+  int32_t mm[2] = {0, 0};
+  FV_HIP(hipMemcpy(mm, minmax, sizeof mm, hipMemcpyDeviceToHost));  // waits for the kernels above
+  if (n_tokens && mm[1] >= 0 && (uint64_t)mm[1] >= vocab)
+    return fv_fail(FV_ERR_DATA, "token id %d is outside the vocabulary of %llu", mm[1], (unsigned long long)vocab);
+  return FV_OK;
+}
+
 // ---- masking of token ids ---------------------------------------------------------------------------
 // The reference removes stop words from an encoded corpus off line, one pass over the whole corpus
 // per id (flyvec/src/remove_words.cpp:28-37: data[w] == id ? -1). Here a bit per vocabulary id

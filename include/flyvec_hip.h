@@ -79,6 +79,18 @@ int fv_build_window_starts(const uint64_t *offsets, uint64_t n_chunks, uint64_t 
  * reference's fp32 counter does. */
 int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, uint64_t vocab, float *out_invf);
 
+/* fv_inverse_frequency for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Corpus
+ * and output are DEVICE memory of the caller (fv_dev_alloc or any other device allocation); the
+ * occurrence counters live in an array built into the library (4 MiB on every device the library
+ * runs on, kept until the process ends), so vocab is at most 2^20 = 1,048,576 ids and a larger one is
+ * refused with FV_ERR_INVALID. Calls nothing that allocates or frees; runs on the default stream and
+ * returns when the result is in out_invf_dev. FV_ERR_DATA on an id >= vocab (the output then ignores
+ * such ids). All calls on one device share that device's array: calls that overlap on one device
+ * race, results of calls made one after the other do not depend on earlier ones. */
+int fv_inverse_frequency_static(const int32_t *corpus_dev, uint64_t n_tokens, uint64_t vocab,
+                                float *out_invf_dev);
+
 /* flyvec/src/remove_words.cpp:28-37 (an off-line tool of the reference: for every id of a stop list,
  * data[w] == id ? -1): rewrites `tokens` in place, every occurrence of an id of `remove_ids`
  * becomes -1 (masked: such a position contributes nothing to a window). One pass on the device,
