@@ -82,6 +82,7 @@ SIGNATURES = {
     "fv_trainer_sync": [_vp],
     "fv_trainer_set_dense_launches": [_vp, _u32],
     "fv_trainer_get_dense_launches": [_vp, C.POINTER(_u32)],
+    "fv_trainer_get_dense_path_counts": [_vp, C.POINTER(_u64), C.POINTER(_u64)],
     "fv_trainer_set_wait_limit": [_vp, _u32],
     "fv_trainer_set_grouping_launch": [_vp, _u32],
     "fv_trainer_get_grouping_launch": [_vp, C.POINTER(_u32)],

@@ -42,9 +42,16 @@
 #include "fv_permute.h"
 #include "fv_repeat_add.h"
 
-// Written over W[p] while the true weight of a sparse element waits in its slot record. A quiet
-// NaN with a payload no arithmetic produces.
-#define FV_SENTINEL 0x7fc5ca1eu
+// Written over W[p] while the true weight of a sparse element waits in its slot record: a NaN whose
+// 23 mantissa bits hold the number of that record plus one (so they are never all zero, which would
+// be an infinity), saturated at the largest value. A step whose record numbers all fit takes the
+// single dense launch, where the thread that meets the NaN finds the record through it; the other
+// launch forms only rely on it being a NaN.
+#define FV_SENTINEL_EXP 0x7f800000u
+#define FV_SENTINEL_MAX 0x007fffffu
+__device__ __forceinline__ float fv_sentinel(uint32_t record) {
+  return __uint_as_float(FV_SENTINEL_EXP | min(record + 1u, FV_SENTINEL_MAX));
+}
 
 struct __attribute__((aligned(16))) fv_slot {
   uint32_t p;  // element index i * ldk + h
@@ -112,7 +119,18 @@ struct fv_trainer {
   // groups per thread (0 = two launches), the arrival word of every block, launches so far, and a
   // host-visible word a block sets when it gave up waiting for the others
   unsigned onepass_blocks, onepass_unroll;
+  unsigned onepass_active;  // threads of a block of that launch that own elements (a multiple of ldk / 4)
   bool onepass;  // in use (fv_trainer_set_dense_launches)
+  // The two largest |W| of every row, kept by the single dense launch so that it knows max|ds| without
+  // a pass over the matrix: each block's share after a launch (top2_part), merged by the next step's
+  // winner kernel (row_top2); what the sparse launch reports on them (row_hits); whether top2_part
+  // describes the matrix as it is (top2_valid: set by a single dense launch, cleared by every other
+  // write of the matrix), and whether the last whole step used them.
+  float2 *row_top2, *top2_part;
+  uint32_t *row_hits;
+  uint32_t *path_count;  // device: launches that took max|ds| from them / that made the pass
+  bool top2_valid, last_top2_known;
+  unsigned sparse_base;  // index in bmax of the sparse launch's first block maximum
   bool separate_grouping;  // the grouping kernel always runs as a launch of its own (fv_trainer_set_grouping_launch)
   bool last_grouped_in_sparse;  // the form the last whole step took: a launch on its own repeats that form
   unsigned long long *arrive;
@@ -121,6 +139,43 @@ struct fv_trainer {
   uint32_t *onepass_status;
   float update_cut;  // largest fp32 <= 1e-10
 };
+
+// ---- the two largest weights of every row ------------------------------------------------------------
+
+// The two largest of a multiset of non-negative values, kept as (m1 >= m2): one more value, and the
+// union with another pair.
+__device__ __forceinline__ void fv_top2_insert(float &m1, float &m2, float a) {
+  m2 = fmaxf(m2, fminf(m1, a));
+  m1 = fmaxf(m1, a);
+}
+__device__ __forceinline__ void fv_top2_merge(float &m1, float &m2, float b1, float b2) {
+  const float lo = fminf(m1, b1);
+  m1 = fmaxf(m1, b1);
+  m2 = fmaxf(lo, fmaxf(m2, b2));
+}
+
+// The shares of every row's two largest weights that the blocks of the last single dense launch left,
+// merged: row_top2[h] for the step that begins. One block per neuron, run as the first blocks of the
+// winner kernel's launch.
+__device__ __forceinline__ void fv_merge_row_top2(const float2 *__restrict__ part, uint32_t part_stride, uint32_t n_part,
+                                                  float2 *__restrict__ row_top2, uint32_t h) {
+  __shared__ float2 wave_pair[4];
+  float m1 = 0.0f, m2 = 0.0f;
+  for (uint32_t j = threadIdx.x; j < n_part; j += 256) {
+    const float2 b = part[(uint64_t)h * part_stride + j];
+    fv_top2_merge(m1, m2, b.x, b.y);
+  }
+  for (int d = 32; d >= 1; d >>= 1) {  // the partner's pair covers other shares: no value is counted twice
+    const float b1 = __shfl_xor(m1, d, 64), b2 = __shfl_xor(m2, d, 64);
+    fv_top2_merge(m1, m2, b1, b2);
+  }
+  if ((threadIdx.x & 63) == 0) wave_pair[threadIdx.x >> 6] = make_float2(m1, m2);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int i = 1; i < 4; ++i) fv_top2_merge(m1, m2, wave_pair[i].x, wave_pair[i].y);
+    row_top2[h] = make_float2(m1, m2);
+  }
+}
 
 // ---- kernel 1: sampler + gather-sum + winner ----------------------------------------------------
 
@@ -145,6 +200,12 @@ struct fv_gather_args {
   uint32_t sampled;  // idx already holds this minibatch
   uint32_t prune;    // in-window duplicate pruning while sampling
   float lmid, lbase; // weight of a window's centre position and of the others (WEIGHTED kernels)
+  // the first merge_rows blocks of the launch merge the shares of the rows' two largest weights that the
+  // last single dense launch left (fv_merge_row_top2); 0: none
+  uint32_t merge_rows;
+  const float2 *top2_part;
+  uint32_t part_stride, n_part;
+  float2 *row_top2;
 };
 
 // FV_GATHER_WINDOWS windows per wavefront, one after the other: the grid then fits the machine in
@@ -181,8 +242,12 @@ __device__ __forceinline__ int32_t fv_column_index(int32_t tok, uint32_t c, uint
 // receives the anti-Hebbian terms. WEIGHTED: position weights other than 1 (:266-286, :307-327).
 template <int NV, bool DELTA, bool WEIGHTED>
 __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a) {
+  if (blockIdx.x < a.merge_rows) {
+    fv_merge_row_top2(a.top2_part, a.part_stride, a.n_part, a.row_top2, blockIdx.x);
+    return;
+  }
   const int lane = threadIdx.x & 63;
-  const uint32_t g = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t g = (blockIdx.x - a.merge_rows) * 4 + (threadIdx.x >> 6);
   const uint32_t per = (a.n + FV_GATHER_WINDOWS - 1) / FV_GATHER_WINDOWS;  // wave g takes windows g, g + per, ...
   if (g >= per) return;
 
@@ -622,6 +687,13 @@ struct fv_sparse_args {
   uint32_t *order_out;  // a neuron's window ids beyond what LDS stages go through here
   uint32_t *group_base_out, *group_count_out;
   float *xx_out;
+  // The two largest |W[h][i]| of every row as the step finds the matrix (row_top2[h] = (v1, v2), v1 >= v2),
+  // when known: the block reports in row_hits how many of its elements hold v1 and, where v2 < v1, how
+  // many hold v2 (bits 0-1 and 2-3, each saturated at 3). The dense launch then knows whether the
+  // largest weight of a row is one of the step's sparse elements.
+  const float2 *row_top2;
+  uint32_t *row_hits;
+  uint32_t top2_known;
 };
 
 // Counting pass of one class block over the windows whose ids are staged in LDS: ord[0 .. n_staged),
@@ -699,7 +771,7 @@ __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uin
 // the block of class 0 leaves xx[h], the neuron's count and its base for the dense launch and clears
 // the neuron's row of the other bit-row buffer.
 template <bool DELTA, bool GROUPING>
-__global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
+__global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6))) void fv_sparse_kernel(fv_sparse_args a) {
   static_assert(!(DELTA && GROUPING), "the anti-Hebbian form has its two lists grouped by launches of their own");
   __shared__ uint32_t cnt[FV_NB_CNT_WORDS];
   __shared__ uint32_t cnt2[DELTA ? FV_NB_CNT_WORDS : 4];
@@ -711,6 +783,8 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
   __shared__ ord_t ord[FV_SP_STAGE];
   __shared__ uint32_t sh_pos;
   __shared__ float sh_xx;
+  __shared__ float2 sh_top2;
+  __shared__ uint32_t sh_hits[2];
   __shared__ float sc64[GROUPING ? 64 : 1];  // activations of a neuron with up to 64 windows, by rank
   __shared__ float wave_max[16];
   __shared__ uint32_t red[17];
@@ -797,8 +871,15 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
     if (tid == 0) {
       a.bmax_sparse[blockIdx.x] = 0.0f;
       a.slot_count[blockIdx.x] = 0;
+      a.row_hits[blockIdx.x] = 0;
     }
     return;
+  }
+  // the row's two largest weights wait in LDS for the elements (every path to them passes a barrier)
+  // and so do the counts of the block's elements that hold the largest / the second largest
+  if (tid == 0) {
+    sh_top2 = a.top2_known ? a.row_top2[h] : make_float2(0.0f, 0.0f);
+    sh_hits[0] = sh_hits[1] = 0;
   }
   // The launch lasts as long as its few heaviest blocks: their waves go first wherever they share a
   // SIMD with the waves of light blocks.
@@ -1003,6 +1084,9 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
       // one element per thread (four in flight): save its weight and its count in a slot record,
       // plant the sentinel, take |ds| (the dense term plus count additions of 1/f; a row with
       // xx == 0 has ds == 0)
+      // number of the round's first record, for the sentinels (saturated: a step with more records than a
+      // sentinel can name is not finished by the launch that reads the numbers)
+      const uint32_t record0 = (uint32_t)min(slot_first + emitted, (uint64_t)FV_SENTINEL_MAX);
       for (uint32_t eb = tid; eb < take; eb += 4 * T) {
         uint32_t pe[4], ne[4], n2e[4];
         float wv[4], fe[4], le[4];
@@ -1041,7 +1125,11 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
             rec.f = fe[u];
             slots[emitted + eb + u * T] = rec;
             if (DELTA) a.slot_n2[slot_first + emitted + eb + u * T] = n2e[u];
-            a.Wt[pe[u]] = __uint_as_float(FV_SENTINEL);
+            a.Wt[pe[u]] = fv_sentinel(record0 + eb + u * T);
+            const float aw = fabsf(wv[u]);
+            const float2 top2 = sh_top2;
+            if (aw == top2.x) atomicAdd(&sh_hits[0], 1u);  // a few per step over the whole grid
+            else if (aw == top2.y) atomicAdd(&sh_hits[1], 1u);
             if (x_h != 0.0f)
               ds_max = fv_absmax_keep(ds_max, DELTA ? fv_sparse_ds2(x_h, wv[u], fe[u], ne[u], a.delta, n2e[u], le[u])
                                                     : fv_sparse_ds(x_h, wv[u], fe[u], ne[u], le[u]));
@@ -1051,10 +1139,11 @@ __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args
       fv_lds_barrier();
     } while (found > FV_SP_LIST_CAP);
   }
-  const float bm = fv_block_max_nonneg(ds_max, wave_max);
+  const float bm = fv_block_max_nonneg(ds_max, wave_max);  // behind its barriers every thread's hits are counted
   if (tid == 0) {
     a.bmax_sparse[blockIdx.x] = bm;
     a.slot_count[blockIdx.x] = emitted;
+    a.row_hits[blockIdx.x] = min(sh_hits[0], 3u) | (min(sh_hits[1], 3u) << 2);
   }
 }
 
@@ -1087,9 +1176,21 @@ struct fv_dense_args {
   uint64_t ahead_first;
   uint32_t ahead_n;
   uint32_t idx_stride;  // entries per row of idx_ahead
+  uint32_t sparse_base;  // index in bmax of the sparse launch's first block maximum (a multiple of 4)
+  // single-launch form: the rows of the token-major matrix are dealt over the blocks in turn, and of a
+  // block's threads the first `active` (the largest multiple of ldk4 it holds) own elements, so that a
+  // thread keeps the same four neurons in every round
+  uint32_t n_rows, active;
+  uint32_t n_slots;  // records the slot regions hold (what a sentinel can name)
+  // the two largest |W[h][i]| of every row before this step (v1 >= v2), when known, and for every block of
+  // the sparse launch how many of its elements hold them (fv_sparse_args.row_hits)
+  const float2 *row_top2;
+  const uint32_t *row_hits;
+  uint32_t top2_known;
+  float2 *top2_part;     // out: the same of the matrix this launch leaves, over each block's share: [neuron][block]
+  uint32_t part_stride;  // blocks of a row of top2_part
+  uint32_t *path_count;  // [0] launches that knew max|ds| when they started, [1] launches that made the pass for it
 };
-
-__device__ __forceinline__ bool fv_is_sentinel(float w) { return __float_as_uint(w) == FV_SENTINEL; }
 
 // ds of a dense element is -xx[h] * W (flyvec/src/cuda_funcs.cu:657-672 without the sparse term). No
 // test for a sentinel or for xx == 0 is needed in the two passes: a sentinel is a NaN and so are
@@ -1222,18 +1323,33 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
 }
 
 // Kernels 4, 5 and 6 as ONE launch, for a matrix that fits the register file of the machine: one
-// block per compute unit, every thread keeps its U 16-byte groups of W in registers from the
-// maximum pass to the update, so W is read once and written once in a step. Between the passes
-// every block publishes its maximum of |ds| as (launch number, value) in one 64-bit word and one
-// wave of it reads the words of all blocks until each carries this launch's number; the values it
+// block per compute unit.
+//
+// max|ds| without a pass over the matrix. A dense element has ds = -xx[h] * W[h][i], and fp32
+// rounding is monotone, so the largest |ds| of the dense elements of row h is fl(|xx[h]| * m) with m
+// the largest |W[h][i]| over the row's dense elements. Every launch leaves, for every row, the two
+// largest |W| of the matrix it has written (each block over its share; the winner kernel of the next
+// step merges the shares). The sparse launch reports how many of a row's sparse elements hold those two
+// values, so this launch knows for every row either m exactly (the largest value, or the second
+// largest when the largest is sparse and the second is not) or an upper bound of it. When the largest
+// exact figure (the sparse elements' own |ds| included) is at least every upper bound, it is max|ds|:
+// s = eps / max(prec, max|ds|) is known before the first weight arrives and the launch is one streaming
+// read-modify-write of the matrix, with no exchange between the blocks and nothing to wait for.
+// Otherwise (or when the largest weights are not known: the first step on a new matrix, or after a step
+// in another launch form) the launch makes the pass: every thread keeps its U 16-byte groups of W in
+// registers from the maximum pass to the update, so W is still read once and written once. Between
+// the passes every block publishes its maximum of |ds| as (launch number, value) in one 64-bit word and
+// one wave of it reads the words of all blocks until each carries this launch's number; the values it
 // read are the maxima, no second look-up follows. The wait is bounded: a block that does not see
 // the others within spin_limit rounds (they are not resident together: the launch was given fewer
 // compute units than it was sized for) marks its word as abandoned, so that blocks arriving later
 // give up as well, sets the status word and leaves its part of W as it is.
-// No thread reads W after the wait, so the sparse elements are finished here as well: the slot
-// records are dealt evenly over the blocks, a thread fetches its record and forms ds while W is
-// in flight and during the wait, and afterwards writes the element; a dense thread never writes a
-// sentinel's position.
+//
+// The sparse elements are finished here as well, by the block that owns them: a thread that meets a
+// sentinel leaves it alone and notes (sentinel, element) in an LDS list; when the block has updated its
+// dense elements the list is dealt over its threads, each of which finds the record through the
+// sentinel's number, forms ds and writes the element. No other block ever reads or writes that element
+// in this launch.
 #ifndef FV_ONEPASS_THREADS
 #define FV_ONEPASS_THREADS 1024
 #endif
@@ -1246,184 +1362,47 @@ __global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
 #endif
 #define FV_ONEPASS_SPIN_LIMIT (1u << 14)  // rounds of a few microseconds each: tens of milliseconds
 #define FV_ONEPASS_ABANDONED 0xffffffffu  // in place of a block's maximum (no maximum is a NaN): it gave up
+#define FV_ONEPASS_HIT_CAP 2048           // sentinels a block notes in LDS; one beyond that is finished on the spot
 
-// The record number r of the step -> its place in the slot regions and its neuron. seg_end holds the
-// running totals of the record counts of the sparse launch's blocks (block g = neuron g / 4, class g % 4),
-// first_window the first window position of every neuron's part of a slot region.
-__device__ __forceinline__ uint64_t fv_slot_locate(const fv_dense_args &a, const uint32_t *seg_end, uint32_t n_seg,
-                                                   const uint32_t *first_window, uint32_t r, uint32_t *h_out) {
-  uint32_t lo = 0, hi = n_seg - 1;  // the smallest g with seg_end[g] > r
-  while (lo < hi) {
-    const uint32_t mid = (lo + hi) >> 1;
-    if (seg_end[mid] > r) hi = mid; else lo = mid + 1;
+// The same on two LDS words per neuron, from many threads at once: the value that loses at the first
+// word -- the newcomer, or the value it displaced -- goes on to the second; every value but the
+// largest is handed on exactly once. Non-negative floats order like their bit patterns.
+__device__ __forceinline__ void fv_top2_insert_lds(uint32_t *s1, uint32_t *s2, uint32_t h, float a) {
+  const uint32_t b = __float_as_uint(a);
+  const uint32_t old = atomicMax(&s1[h], b);
+  atomicMax(&s2[h], min(old, b));
+}
+// |w| for that bookkeeping; a NaN (a sentinel) counts as 0
+__device__ __forceinline__ float fv_abs_or_zero(float w) { return w == w ? fabsf(w) : 0.0f; }
+
+// The element p holds the sentinel `bits`: its final value from the record the sentinel names. The saved
+// weight goes back where the row is not updated (xx == 0) or the launch gave up, else the updated one.
+template <bool DELTA>
+__device__ __forceinline__ void fv_finish_sparse_element(const fv_dense_args &a, uint32_t bits, uint32_t p, float s,
+                                                         bool ok, const float *xs, uint32_t *sp1, uint32_t *sp2) {
+  const uint32_t at = (bits & FV_SENTINEL_MAX) - 1u;
+  if (at >= a.n_slots) return;  // a NaN of another origin stays what it is
+  const fv_slot sl = a.slots[at];
+  if (sl.p != p) return;
+  const uint32_t h = p % a.ldk;
+  const float x = xs[h];
+  float out = sl.wv;
+  if (ok && x != 0.0f) {
+    const float l = p >= a.V * a.ldk ? a.lmid : a.lbase;
+    const float ds = DELTA ? fv_sparse_ds2(x, sl.wv, sl.f, sl.n, a.delta, a.slot_n2[at], l)
+                           : fv_sparse_ds(x, sl.wv, sl.f, sl.n, l);
+    const float d = __fmul_rn(s, ds);
+    if (fabsf(d) > a.update_cut) out = __fadd_rn(sl.wv, d);
   }
-  const uint32_t h = lo >> FV_NB_CLASS_SHIFT, q = lo & (FV_NB_CLASSES - 1);
-  *h_out = h;
-  return (uint64_t)q * a.slot_stride + (uint64_t)first_window[h] * a.w + (r - (lo ? seg_end[lo - 1] : 0u));
+  ((float *)a.Wt4)[p] = out;
+  fv_top2_insert_lds(sp1, sp2, h, fv_abs_or_zero(out));
 }
 
-// The update of the single launch: a sentinel's position is never written, another thread of the
-// same launch puts the finished sparse element there. A sentinel is a NaN, and no NaN is ever
-// changed by the update, so NaN positions are simply left out of the store.
-__device__ __forceinline__ void fv_update_four_around(const fv_dense_args &a, uint32_t p4, float4 w, const float4 x,
-                                                      const float s) {
-  if (!fv_apply_four(w, x, s, a.update_cut)) return;
-  if (!(__builtin_isunordered(w.x, w.y) || __builtin_isunordered(w.z, w.w))) {
-    a.Wt4[p4] = w;
-    return;
-  }
-  float *e = (float *)&a.Wt4[p4];
-  if (w.x == w.x) e[0] = w.x;
-  if (w.y == w.y) e[1] = w.y;
-  if (w.z == w.z) e[2] = w.z;
-  if (w.w == w.w) e[3] = w.w;
-}
-
-static_assert(FV_MAX_HID <= 2 * FV_ONEPASS_THREADS, "two first-window words per thread cover every neuron");
-static_assert(FV_MAX_HID * FV_NB_CLASSES <= 8 * FV_ONEPASS_THREADS, "eight record counts per thread cover every block");
-
-// P: counts of the sparse launch's blocks a thread sums (FV_NB_CLASSES * K <= P * FV_ONEPASS_THREADS)
-template <int U, int P, bool DELTA>
-__global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv_dense_args a) {
-  constexpr uint32_t T = FV_ONEPASS_THREADS;
-  // xx (a 16-byte word per thread, ldk floats used), the first window of every neuron's slot
-  // records (two words per thread), the running totals of the record counts
-  extern __shared__ float4 xs4[];
-  uint32_t *first_window = (uint32_t *)(xs4 + T);
-  uint32_t *seg_end = first_window + 2 * T;
-  __shared__ float smem16[16];
-  __shared__ uint32_t red[17];
-  __shared__ float sh_s;
-  __shared__ uint32_t sh_ok;
-  const uint32_t n_seg = a.K * FV_NB_CLASSES;
-  const uint32_t stride = gridDim.x * T;
-  const uint32_t p4 = blockIdx.x * T + threadIdx.x;
-  const uint32_t dq = stride % a.ldk4;
-  const uint32_t q0 = p4 % a.ldk4;
-  // The small loads first, every one unconditional, then all of this thread's W: loads return in
-  // the order of issue, so what is issued here is used while W is in flight, and nothing that is
-  // issued after W is needed before W has arrived.
-  uint32_t segc[P];
-  float sparse_max[P];  // the sparse launch's block maxima, dealt over the blocks of this one
-#pragma unroll
-  for (int j = 0; j < P; ++j) {
-    segc[j] = a.slot_count[min(threadIdx.x * P + j, n_seg - 1)];
-    sparse_max[j] = a.bmax[a.dense_blocks + min(blockIdx.x + gridDim.x * (threadIdx.x + T * j), n_seg - 1)];
-  }
-  const float4 x_stage = ((const float4 *)a.xx)[min(threadIdx.x, a.ldk4 - 1)];
-  uint32_t fw[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const uint32_t h = min(threadIdx.x + T * j, a.K - 1);
-    fw[j] = a.group_base[h] + (DELTA ? a.group_base2[h] : 0u);
-  }
-  // after one launch has given up, the launches already enqueued behind it do not wait at all
-  const uint32_t limit = a.scalars[1] != 0.0f ? 0u : a.spin_limit;
-  float4 w[U];
-  __builtin_amdgcn_sched_barrier(0);  // nothing that uses a small load moves up between the loads of W
-  const uint32_t inside = min(p4, a.total4 - 1);  // read again, and not used, by a load past the end
-#pragma unroll
-  for (int u = 0; u < (FV_ONEPASS_DEPTH < U ? FV_ONEPASS_DEPTH : U); ++u)
-    w[u] = a.Wt4[p4 + u * stride < a.total4 ? p4 + u * stride : inside];
-  __builtin_amdgcn_sched_barrier(0);
-
-  xs4[threadIdx.x] = x_stage;
-  first_window[threadIdx.x] = fw[0];
-  first_window[threadIdx.x + T] = fw[1];
-  uint32_t mine = 0;
-  float m = 0.0f;
-#pragma unroll
-  for (int j = 0; j < P; ++j) {
-    if (threadIdx.x * P + j >= n_seg) segc[j] = 0;
-    mine += segc[j];
-    m = fmaxf(m, sparse_max[j]);  // an index past the end repeats the last maximum
-  }
-  uint32_t n_records;
-  uint32_t run = fv_block_scan_total(mine, red, &n_records);
-#pragma unroll
-  for (int j = 0; j < P; ++j) {
-    run += segc[j];
-    if (threadIdx.x * P + j < n_seg) seg_end[threadIdx.x * P + j] = run;
-  }
-  __syncthreads();
-  // this block's share of the records; a thread's first one is fetched now, behind W
-  const uint32_t r_lo = (uint32_t)((uint64_t)n_records * blockIdx.x / gridDim.x);
-  const uint32_t r_hi = (uint32_t)((uint64_t)n_records * (blockIdx.x + 1) / gridDim.x);
-  const uint32_t r0 = r_lo + threadIdx.x;
-  const bool live0 = r0 < r_hi;
-  uint32_t h0 = 0;
-  uint64_t at0 = 0;  // a thread without a record reads the first one of the buffer and does not use it
-  if (live0) at0 = fv_slot_locate(a, seg_end, n_seg, first_window, r0, &h0);
-  const fv_slot sl0 = a.slots[at0];
-  const uint32_t n20 = DELTA ? a.slot_n2[at0] : 0u;
-  // the next minibatch's column indices, by all waves but the first: the window's start now
-  constexpr uint32_t TS = T - 64;
-  const uint32_t ahead_entries = a.ahead_n * a.idx_stride;  // the entries past w of a row get -1
-  const uint32_t e0 = blockIdx.x * TS + (threadIdx.x - 64);
-  const bool samples0 = threadIdx.x >= 64 && e0 < ahead_entries;
-  const uint32_t er0 = samples0 ? e0 / a.idx_stride : 0u;
-  const uint64_t start0 = a.ahead_n ? a.pstart[a.ahead_first + er0] : 0ull;
-  uint32_t q = q0;
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    if (p4 + u * stride < a.total4) {
-      m = fv_absmax_four(m, xs4[q], w[u]);
-    }
-    if (u + FV_ONEPASS_DEPTH < U) {  // the next load takes the place of the one just used
-      const uint32_t p = p4 + (u + FV_ONEPASS_DEPTH) * stride;
-      w[u + FV_ONEPASS_DEPTH] = a.Wt4[p < a.total4 ? p : inside];
-    }
-    q += dq;
-    if (q >= a.ldk4) q -= a.ldk4;
-  }
-  // the block's maximum, needed by its first wave only: one barrier
-  {
-    const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
-    if ((threadIdx.x & 63) == 0) smem16[threadIdx.x >> 6] = __uint_as_float(wm);
-  }
-  __syncthreads();
-  if (threadIdx.x < 64) {
-    float bm = threadIdx.x < T / 64 ? smem16[threadIdx.x] : 0.0f;
-    bm = __uint_as_float(fv_wave_max_u32(__float_as_uint(bm)));
-    if (threadIdx.x == 0)
-      __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | __float_as_uint(bm),
-                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  if (threadIdx.x < 64) {
-    uint32_t mx = 0;
-    bool done = false, abandoned = false;
-    for (uint32_t spin = 0; spin < limit && !done && !abandoned; ++spin) {
-      bool ok = true, bad = false;
-      mx = 0;
-      for (uint32_t i = threadIdx.x; i < gridDim.x; i += 64) {
-        const unsigned long long v = __hip_atomic_load(&a.arrive[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ok = ok && (uint32_t)(v >> 32) == a.epoch;
-        bad = bad || ((uint32_t)(v >> 32) == a.epoch && (uint32_t)v == FV_ONEPASS_ABANDONED);
-        mx = max(mx, (uint32_t)v);  // non-negative floats order like their bit patterns
-      }
-      abandoned = __any(bad);
-      done = !abandoned && __all(ok);
-      if (!done && !abandoned) __builtin_amdgcn_s_sleep(2);
-    }
-    mx = fv_wave_max_u32(mx);
-    if (threadIdx.x == 0) {
-      const float nc = __uint_as_float(mx);
-      sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
-      sh_ok = done;
-      if (!done) {
-        // blocks that arrive later must not update either
-        __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | FV_ONEPASS_ABANDONED,
-                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        *a.status = 1u;
-        a.scalars[0] = __uint_as_float(0x7fc00000u);
-        a.scalars[1] = 1.0f;
-      } else if (blockIdx.x == 0) {
-        a.scalars[0] = nc;
-      }
-    }
-  }
-  // the token of the sampled position while the first wave waits; then, for a minibatch with more
-  // positions than the launch has sampling threads, the rest
+// The next minibatch's column indices, by all waves but the first (which polls in the exchange): the
+// window's start was fetched behind the loads of W, the token follows here; then, for a minibatch with more
+// positions than the launch has sampling threads, the rest.
+__device__ __forceinline__ void fv_sample_ahead(const fv_dense_args &a, bool samples0, uint32_t e0, uint32_t er0,
+                                                uint64_t start0, uint32_t ahead_entries, uint32_t TS) {
   if (samples0) {
     const uint32_t c = e0 - er0 * a.idx_stride;
     a.idx_ahead[e0] = c < a.w ? fv_column_index(a.corpus[start0 + c], c, a.w, a.V) : -1;
@@ -1433,64 +1412,262 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
       const uint32_t r = e / a.idx_stride, c = e - r * a.idx_stride;
       a.idx_ahead[e] = c < a.w ? fv_column_index(a.corpus[a.pstart[a.ahead_first + r] + c], c, a.w, a.V) : -1;
     }
-  // ds of the first record does not depend on the scale: formed while the first wave waits
-  // (every thread takes this path, with no additions where it has no record: the fetch is then
-  // complete in every thread before the stores below)
-  const float *xs = (const float *)xs4;
-  const float x0 = xs[h0];
-  const bool update0 = live0 && x0 != 0.0f;
-  const float l0 = sl0.p >= a.V * a.ldk ? a.lmid : a.lbase;
-  const float ds0 = DELTA ? fv_sparse_ds2(x0, sl0.wv, sl0.f, update0 ? sl0.n : 0u, a.delta, update0 ? n20 : 0u, l0)
-                          : fv_sparse_ds(x0, sl0.wv, sl0.f, update0 ? sl0.n : 0u, l0);
+}
+
+static_assert(FV_MAX_HID <= 2 * FV_ONEPASS_THREADS, "two neurons per thread cover every row");
+static_assert(FV_NB_CLASSES == 4, "a neuron's block maxima and hit counts are read as one 16-byte word each");
+
+template <int U, bool DELTA>
+__global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv_dense_args a) {
+  constexpr uint32_t T = FV_ONEPASS_THREADS;
+  constexpr int DEPTH = FV_ONEPASS_DEPTH < U ? FV_ONEPASS_DEPTH : U;
+  // xx (ldk floats); the two largest finished sparse elements of every neuron (2 x ldk words); the
+  // sentinels met (FV_ONEPASS_HIT_CAP pairs); the threads' two largest weights (4 x active pairs)
+  extern __shared__ float4 dyn4[];
+  float *xs = (float *)dyn4;
+  uint32_t *sp1 = (uint32_t *)(xs + a.ldk);
+  uint32_t *sp2 = sp1 + a.ldk;
+  uint2 *hit_list = (uint2 *)(sp2 + a.ldk);
+  float2 *pairs = (float2 *)(hit_list + FV_ONEPASS_HIT_CAP);
+  __shared__ uint32_t red3[T / 64][3];
+  __shared__ float smem16[16];
+  __shared__ float sh_s;
+  __shared__ uint32_t sh_ok, sh_hits;
+  const uint32_t tid = threadIdx.x;
+  const bool active = tid < a.active;
+  const uint32_t q = tid % a.ldk4, r = tid / a.ldk4;
+  const uint32_t rows_per_round = a.active / a.ldk4;
+  const uint32_t row0 = blockIdx.x + gridDim.x * r;  // the thread's row in round 0
+  const uint32_t row_step = gridDim.x * rows_per_round;
+  const uint32_t row_inside = min(row0, a.n_rows - 1);  // read again, and not used, by a load past the end
+  // The small loads first, every one unconditional, then this thread's W: loads return in the order
+  // of issue, so what is issued here is in hand while W is in flight.
+  float xh[2];
+  float2 rm[2];
+  uint4 hit4[2];
+  float4 smx[2];  // the sparse launch's block maxima of |ds|
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t h = min(tid + T * j, a.K - 1);
+    xh[j] = a.xx[min(tid + T * j, a.ldk - 1)];
+    rm[j] = a.row_top2[h];
+    hit4[j] = ((const uint4 *)a.row_hits)[h];
+    smx[j] = ((const float4 *)(a.bmax + a.sparse_base))[h];
+  }
+  // after one launch has given up, the launches already enqueued behind it do not wait at all
+  const uint32_t limit = a.scalars[1] != 0.0f ? 0u : a.spin_limit;
+  float4 w[U];
+  __builtin_amdgcn_sched_barrier(0);  // nothing that uses a small load moves up between the loads of W
+#pragma unroll
+  for (int u = 0; u < DEPTH; ++u) {
+    const uint32_t row = row0 + u * row_step;
+    w[u] = a.Wt4[(row < a.n_rows ? row : row_inside) * a.ldk4 + q];
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // the next minibatch's column indices, by all waves but the first: the window's start now
+  constexpr uint32_t TS = T - 64;
+  const uint32_t ahead_entries = a.ahead_n * a.idx_stride;  // the entries past w of a row get -1
+  const uint32_t e0 = blockIdx.x * TS + (tid - 64);
+  const bool samples0 = tid >= 64 && e0 < ahead_entries;
+  const uint32_t er0 = samples0 ? e0 / a.idx_stride : 0u;
+  const uint64_t start0 = a.ahead_n ? a.pstart[a.ahead_first + er0] : 0ull;
+
+  // What is known of max|ds| before the matrix is seen: S, the largest |ds| of a sparse element; E, the
+  // largest over the rows whose largest dense weight is known of fl(|xx| * that weight); F, the same over
+  // the other rows with an upper bound of that weight.
+  uint32_t S = 0, E = 0, F = 0;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t h = tid + T * j;
+    if (h < a.ldk) {
+      xs[h] = xh[j];
+      sp1[h] = 0;
+      sp2[h] = 0;
+    }
+    if (h < a.K) {
+      const uint32_t n1 = (hit4[j].x & 3u) + (hit4[j].y & 3u) + (hit4[j].z & 3u) + (hit4[j].w & 3u);
+      const uint32_t n2 = ((hit4[j].x >> 2) & 3u) + ((hit4[j].y >> 2) & 3u) + ((hit4[j].z >> 2) & 3u) + ((hit4[j].w >> 2) & 3u);
+      const float v1 = rm[j].x, v2 = rm[j].y;
+      // v1 == v2: two elements hold the largest value, one of them is dense unless two sparse ones hold it.
+      // v1 > v2: one element holds v1; if it is sparse, v2 bounds the rest, and is reached unless a
+      // sparse element holds it.
+      const bool first = v1 == v2 ? n1 <= 1 : n1 == 0;
+      const bool exact = first || (v1 != v2 && n2 == 0);
+      const uint32_t cand = __float_as_uint(__fmul_rn(fabsf(xh[j]), first ? v1 : v2));
+      if (exact) E = max(E, cand); else F = max(F, cand);
+      S = max(S, __float_as_uint(fmaxf(fmaxf(smx[j].x, smx[j].y), fmaxf(smx[j].z, smx[j].w))));
+    }
+  }
+  if (tid == 0) sh_hits = 0;
+  {
+    const uint32_t ws = fv_wave_max_u32(S), we = fv_wave_max_u32(E), wf = fv_wave_max_u32(F);
+    if ((tid & 63) == 0) {
+      red3[tid >> 6][0] = ws;
+      red3[tid >> 6][1] = we;
+      red3[tid >> 6][2] = wf;
+    }
+  }
   __syncthreads();
-  const bool ok = sh_ok != 0;
-  const float s = sh_s;
-  if (ok) {
-    q = q0;
+  S = E = F = 0;
+#pragma unroll
+  for (uint32_t i = 0; i < T / 64; ++i) {
+    S = max(S, red3[i][0]);
+    E = max(E, red3[i][1]);
+    F = max(F, red3[i][2]);
+  }
+  const bool fast = a.top2_known && F <= max(S, E);  // the same answer in every thread of every block
+  const float4 xq = ((const float4 *)xs)[q];
+
+  float s;
+  bool ok = true;
+  if (fast) {
+    const float nc = __uint_as_float(max(S, E));
+    s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
+    if (blockIdx.x == 0 && tid == 0) {
+      a.scalars[0] = nc;
+      a.path_count[0] += 1;
+    }
+  } else {
+    // the pass for the maximum, on registers; the loads not yet issued take the places of those used
+    float m = __uint_as_float(S);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      if (p4 + u * stride < a.total4) fv_update_four_around(a, p4 + u * stride, w[u], xs4[q], s);
-      q += dq;
-      if (q >= a.ldk4) q -= a.ldk4;
+      const uint32_t row = row0 + u * row_step;
+      if (active && row < a.n_rows) m = fv_absmax_four(m, xq, w[u]);
+      if (u + DEPTH < U) {
+        const uint32_t rown = row0 + (u + DEPTH) * row_step;
+        w[u + DEPTH] = a.Wt4[(rown < a.n_rows ? rown : row_inside) * a.ldk4 + q];
+      }
+    }
+    // the block's maximum, needed by its first wave only: one barrier
+    {
+      const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
+      if ((tid & 63) == 0) smem16[tid >> 6] = __uint_as_float(wm);
+    }
+    __syncthreads();
+    if (tid < 64) {
+      float bm = tid < T / 64 ? smem16[tid] : 0.0f;
+      bm = __uint_as_float(fv_wave_max_u32(__float_as_uint(bm)));
+      if (tid == 0)
+        __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | __float_as_uint(bm),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      uint32_t mx = 0;
+      bool done = false, abandoned = false;
+      for (uint32_t spin = 0; spin < limit && !done && !abandoned; ++spin) {
+        bool all = true, bad = false;
+        mx = 0;
+        for (uint32_t i = tid; i < gridDim.x; i += 64) {
+          const unsigned long long v = __hip_atomic_load(&a.arrive[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          all = all && (uint32_t)(v >> 32) == a.epoch;
+          bad = bad || ((uint32_t)(v >> 32) == a.epoch && (uint32_t)v == FV_ONEPASS_ABANDONED);
+          mx = max(mx, (uint32_t)v);  // non-negative floats order like their bit patterns
+        }
+        abandoned = __any(bad);
+        done = !abandoned && __all(all);
+        if (!done && !abandoned) __builtin_amdgcn_s_sleep(2);
+      }
+      mx = fv_wave_max_u32(mx);
+      if (tid == 0) {
+        const float nc = __uint_as_float(mx);
+        sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
+        sh_ok = done;
+        if (!done) {
+          // blocks that arrive later must not update either
+          __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | FV_ONEPASS_ABANDONED,
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          *a.status = 1u;
+          a.scalars[0] = __uint_as_float(0x7fc00000u);
+          a.scalars[1] = 1.0f;
+        } else if (blockIdx.x == 0) {
+          a.scalars[0] = nc;
+          a.path_count[1] += 1;
+        }
+      }
+    }
+    fv_sample_ahead(a, samples0, e0, er0, start0, ahead_entries, TS);  // while the first wave waits
+    __syncthreads();
+    ok = sh_ok != 0;
+    s = sh_s;
+  }
+
+  // The update. A group without a sentinel is stored whole where something changed; in a group with
+  // one the other elements are stored one by one and the sentinel is noted for later. The two largest
+  // |W| of what the thread leaves behind are kept per neuron.
+  float t1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, t2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#define FV_ONEPASS_ELEMENT(member, lane4)                                                      \
+  if (v.member == v.member) {                                                                  \
+    if (changed) e[lane4] = v.member;                                                          \
+  } else {                                                                                     \
+    const uint32_t k = atomicAdd(&sh_hits, 1u);                                                \
+    if (k < FV_ONEPASS_HIT_CAP)                                                                \
+      hit_list[k] = make_uint2(__float_as_uint(v.member), 4u * p4 + lane4);                    \
+    else                                                                                       \
+      fv_finish_sparse_element<DELTA>(a, __float_as_uint(v.member), 4u * p4 + lane4, s, ok, xs, sp1, sp2); \
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const uint32_t row = row0 + u * row_step;
+    if (active && row < a.n_rows) {
+      const uint32_t p4 = row * a.ldk4 + q;
+      float4 v = w[u];
+      const bool has_nan = __builtin_isunordered(v.x, v.y) || __builtin_isunordered(v.z, v.w);
+      const bool changed = ok && fv_apply_four(v, xq, s, a.update_cut);
+      if (!has_nan) {
+        if (changed) a.Wt4[p4] = v;
+      } else {
+        float *e = (float *)&a.Wt4[p4];
+        FV_ONEPASS_ELEMENT(x, 0)
+        FV_ONEPASS_ELEMENT(y, 1)
+        FV_ONEPASS_ELEMENT(z, 2)
+        FV_ONEPASS_ELEMENT(w, 3)
+      }
+      fv_top2_insert(t1[0], t2[0], fv_abs_or_zero(v.x));
+      fv_top2_insert(t1[1], t2[1], fv_abs_or_zero(v.y));
+      fv_top2_insert(t1[2], t2[2], fv_abs_or_zero(v.z));
+      fv_top2_insert(t1[3], t2[3], fv_abs_or_zero(v.w));
+    }
+    if (fast && u + DEPTH < U) {  // the next load takes the place of the one just used
+      const uint32_t rown = row0 + (u + DEPTH) * row_step;
+      w[u + DEPTH] = a.Wt4[(rown < a.n_rows ? rown : row_inside) * a.ldk4 + q];
     }
   }
-  // the sparse elements: the saved weight goes back where the row is not updated (xx == 0) or the
-  // launch gave up, else the updated one
-  if (live0) {
-    float out = sl0.wv;
-    if (ok && x0 != 0.0f) {
-      const float d = __fmul_rn(s, ds0);
-      if (fabsf(d) > a.update_cut) out = __fadd_rn(sl0.wv, d);
-    }
-    ((float *)a.Wt4)[sl0.p] = out;
+#undef FV_ONEPASS_ELEMENT
+  if (fast) fv_sample_ahead(a, samples0, e0, er0, start0, ahead_entries, TS);
+  if (active) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pairs[(e * rows_per_round + r) * a.ldk4 + q] = make_float2(t1[e], t2[e]);
   }
-  for (uint32_t r = r0 + T; r < r_hi; r += T) {  // more records than threads: fetched only now
-    uint32_t h;
-    const uint64_t at = fv_slot_locate(a, seg_end, n_seg, first_window, r, &h);
-    const fv_slot sl = a.slots[at];
-    float out = sl.wv;
-    if (ok && xs[h] != 0.0f) {
-      const float l = sl.p >= a.V * a.ldk ? a.lmid : a.lbase;
-      const float ds = DELTA ? fv_sparse_ds2(xs[h], sl.wv, sl.f, sl.n, a.delta, a.slot_n2[at], l)
-                             : fv_sparse_ds(xs[h], sl.wv, sl.f, sl.n, l);
-      const float d = __fmul_rn(s, ds);
-      if (fabsf(d) > a.update_cut) out = __fadd_rn(sl.wv, d);
+  __syncthreads();
+  // the sentinels the block has met, dealt over its threads
+  const uint32_t n_hits = min(sh_hits, (uint32_t)FV_ONEPASS_HIT_CAP);
+  for (uint32_t i = tid; i < n_hits; i += T) {
+    const uint2 hit = hit_list[i];
+    fv_finish_sparse_element<DELTA>(a, hit.x, hit.y, s, ok, xs, sp1, sp2);
+  }
+  __syncthreads();
+  // the block's share of every row's two largest weights: its threads' pairs and the finished sparse elements
+  for (uint32_t h = tid; h < a.K; h += T) {
+    const uint32_t e = h & 3u, qq = h >> 2;
+    float m1 = __uint_as_float(sp1[h]), m2 = __uint_as_float(sp2[h]);
+    for (uint32_t rr = 0; rr < rows_per_round; ++rr) {
+      const float2 b = pairs[(e * rows_per_round + rr) * a.ldk4 + qq];
+      fv_top2_merge(m1, m2, b.x, b.y);
     }
-    ((float *)a.Wt4)[sl.p] = out;
+    a.top2_part[(uint64_t)h * a.part_stride + blockIdx.x] = make_float2(m1, m2);
   }
 }
 
-template <int U, int P, bool DELTA>
+template <int U, bool DELTA>
 static void fv_launch_onepass(const fv_dense_args &d, unsigned blocks, size_t smem, hipStream_t stream) {
-  hipLaunchKernelGGL((fv_dense_onepass_kernel<U, P, DELTA>), dim3(blocks), dim3(FV_ONEPASS_THREADS), smem, stream, d);
+  hipLaunchKernelGGL((fv_dense_onepass_kernel<U, DELTA>), dim3(blocks), dim3(FV_ONEPASS_THREADS), smem, stream, d);
 }
 
-template <int U, int P>
+template <int U>
 static int fv_onepass_fits(size_t smem) {
   int nb = 0, nb2 = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fv_dense_onepass_kernel<U, P, false>, FV_ONEPASS_THREADS,
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fv_dense_onepass_kernel<U, false>, FV_ONEPASS_THREADS,
                                                    smem) != hipSuccess ||
-      hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb2, fv_dense_onepass_kernel<U, P, true>, FV_ONEPASS_THREADS,
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb2, fv_dense_onepass_kernel<U, true>, FV_ONEPASS_THREADS,
                                                    smem) != hipSuccess) {
     (void)hipGetLastError();
     return 0;
@@ -1638,6 +1815,10 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   (void)hipFree(t->xx);
   (void)hipFree(t->scalars);
   (void)hipFree(t->arrive);
+  (void)hipFree(t->row_top2);
+  (void)hipFree(t->top2_part);
+  (void)hipFree(t->row_hits);
+  (void)hipFree(t->path_count);
   if (t->onepass_status) (void)hipHostFree(t->onepass_status);
   if (t->stream) (void)hipStreamDestroy(t->stream);
   fv_trainers_alive.fetch_sub(1);
@@ -1668,7 +1849,22 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMalloc((void **)&t->slots, (size_t)FV_NB_CLASSES * t->B * t->w * sizeof(fv_slot)));
   FV_HIP(hipMalloc((void **)&t->slot_count, (size_t)FV_NB_CLASSES * t->K * sizeof(uint32_t)));
   FV_HIP(hipMalloc((void **)&t->xx, (size_t)t->ldk * sizeof(float)));
-  FV_HIP(hipMalloc((void **)&t->bmax, ((size_t)t->dense_blocks + (size_t)FV_NB_CLASSES * t->K) * sizeof(float)));
+  // a neuron's four sparse block maxima are read as one 16-byte word: they start at a multiple of 4
+  t->sparse_base = (t->dense_blocks + 3u) & ~3u;
+  const size_t n_bmax = (size_t)t->sparse_base + (size_t)FV_NB_CLASSES * t->K;
+  FV_HIP(hipMalloc((void **)&t->bmax, n_bmax * sizeof(float)));
+  FV_HIP(hipMemsetAsync(t->bmax, 0, n_bmax * sizeof(float), t->stream));
+  FV_HIP(hipMalloc((void **)&t->row_hits, (size_t)FV_NB_CLASSES * t->K * sizeof(uint32_t)));
+  FV_HIP(hipMemsetAsync(t->row_hits, 0, (size_t)FV_NB_CLASSES * t->K * sizeof(uint32_t), t->stream));
+  FV_HIP(hipMalloc((void **)&t->row_top2, (size_t)t->K * sizeof(float2)));
+  FV_HIP(hipMemsetAsync(t->row_top2, 0, (size_t)t->K * sizeof(float2), t->stream));
+  FV_HIP(hipMalloc((void **)&t->path_count, 2 * sizeof(uint32_t)));
+  FV_HIP(hipMemsetAsync(t->path_count, 0, 2 * sizeof(uint32_t), t->stream));
+  if (t->onepass_unroll) {
+    const size_t n_part = (size_t)t->K * t->onepass_blocks;
+    FV_HIP(hipMalloc((void **)&t->top2_part, n_part * sizeof(float2)));
+    FV_HIP(hipMemsetAsync(t->top2_part, 0, n_part * sizeof(float2), t->stream));
+  }
   FV_HIP(hipMemsetAsync(t->win, 0, ((size_t)t->B + 16) * sizeof(int32_t), t->stream));
   FV_HIP(hipMalloc((void **)&t->win16, ((size_t)t->B + 64) * sizeof(uint16_t)));  // read in 16-byte pieces
   FV_HIP(hipMemsetAsync(t->win16, 0, ((size_t)t->B + 64) * sizeof(uint16_t), t->stream));
@@ -1695,27 +1891,30 @@ static int fv_trainer_alloc(fv_trainer *t) {
 
 // One launch for both dense passes when every compute unit can hold a block whose threads keep the
 // whole matrix in registers between them; otherwise (onepass_unroll = 0) the two launches.
-// a 16-byte word and two 4-byte words per thread, then one running total per block of the sparse launch
+// Dynamic LDS of that launch: xx and two words per neuron, the list of sentinels, four pairs per thread.
 static size_t fv_onepass_smem(const fv_trainer *t) {
-  return (size_t)FV_ONEPASS_THREADS * (sizeof(float4) + 2 * sizeof(uint32_t)) +
-         (size_t)t->K * FV_NB_CLASSES * sizeof(uint32_t);
+  return (size_t)t->ldk * 3 * sizeof(float) + (size_t)FV_ONEPASS_HIT_CAP * sizeof(uint2) +
+         (size_t)FV_ONEPASS_THREADS * 4 * sizeof(float2);
 }
 
 static void fv_choose_onepass(fv_trainer *t, uint64_t cu) {
-  t->onepass_blocks = t->onepass_unroll = 0;
+  t->onepass_blocks = t->onepass_unroll = t->onepass_active = 0;
   t->onepass_spin_limit = FV_ONEPASS_SPIN_LIMIT;
-  uint64_t blocks = ((uint64_t)t->total4 + FV_ONEPASS_THREADS - 1) / FV_ONEPASS_THREADS;
+  const uint32_t ldk4 = t->ldk / 4;
+  if (ldk4 > FV_ONEPASS_THREADS) return;
+  // a block takes whole rows: rows_per_round of them at a time, one 16-byte group per thread
+  const uint32_t rows_per_round = FV_ONEPASS_THREADS / ldk4;
+  uint64_t blocks = (t->N + rows_per_round - 1) / rows_per_round;
   if (blocks > cu * FV_ONEPASS_BLOCKS_PER_CU) blocks = cu * FV_ONEPASS_BLOCKS_PER_CU;
-  const uint64_t need = ((uint64_t)t->total4 + blocks * FV_ONEPASS_THREADS - 1) / (blocks * FV_ONEPASS_THREADS);
+  const uint64_t need = (t->N + blocks * rows_per_round - 1) / (blocks * rows_per_round);
   if (need > FV_ONEPASS_MAX_UNROLL) return;
   const unsigned unroll = need <= 8 ? 8 : 16;
   const size_t smem = fv_onepass_smem(t);
-  const bool narrow = (uint64_t)t->K * FV_NB_CLASSES <= 2 * FV_ONEPASS_THREADS;
-  const int fits = unroll == 8 ? (narrow ? fv_onepass_fits<8, 2>(smem) : fv_onepass_fits<8, 8>(smem))
-                               : (narrow ? fv_onepass_fits<16, 2>(smem) : fv_onepass_fits<16, 8>(smem));
+  const int fits = unroll == 8 ? fv_onepass_fits<8>(smem) : fv_onepass_fits<16>(smem);
   if (!fits) return;
   t->onepass_blocks = (unsigned)blocks;
   t->onepass_unroll = unroll;
+  t->onepass_active = rows_per_round * ldk4;
   t->onepass = true;
 }
 
@@ -1873,6 +2072,7 @@ extern "C" int fv_trainer_set_weights(fv_trainer *t, const float *W) {
   FV_REQUIRE(t && W, FV_ERR_INVALID, "null argument");
   FV_TRY(fv_upload_weights(W, t->Wt, t->K, t->N, t->ldk, t->stream));
   t->have_weights = true;
+  t->top2_valid = false;  // the first single dense launch on the new matrix makes the pass for max|ds|
   return FV_OK;
 }
 
@@ -1937,7 +2137,7 @@ extern "C" int fv_trainer_get_permutation(fv_trainer *t, uint64_t *out_perm, uin
 template <int NV>
 static void fv_launch_gather(const fv_gather_args &a, bool with_second, bool weighted, hipStream_t stream) {
   const uint32_t waves = (a.n + FV_GATHER_WINDOWS - 1) / FV_GATHER_WINDOWS;
-  const dim3 grid((waves + 3) / 4), block(256);
+  const dim3 grid((waves + 3) / 4 + a.merge_rows), block(256);
   if (weighted) {
     if (with_second)
       hipLaunchKernelGGL((fv_gather_winner_kernel<NV, true, true>), grid, block, 0, stream, a);
@@ -1990,7 +2190,20 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
                            unsigned which = 0x3f, bool repeated = false) {
   const bool anti = delta != 0.0f;  // the second neuron of every window takes part (flyvec/src/cuda_funcs.cu:726-734)
   if (anti) FV_TRY(fv_trainer_alloc_delta(t));
+  const bool whole = which == 0x3f;
+  // records the slot regions of this step hold; the single dense launch finds a record through the number in
+  // its sentinel, so it is only taken when every record number fits one
+  const uint64_t n_slots = (uint64_t)FV_NB_CLASSES * t->B * t->w * (anti ? 2 : 1);
+  const bool onepass = t->onepass && fv_trainers_alive.load() == 1 && n_slots + 1 < FV_SENTINEL_MAX;
+  // the rows' two largest weights are in hand if the last write of the matrix was a single dense launch
+  const bool top2_known = whole ? onepass && t->top2_valid : t->last_top2_known;
+  if (whole) t->last_top2_known = top2_known;
   fv_gather_args g;
+  g.merge_rows = (top2_known && (whole || (which & 1u))) ? t->K : 0u;
+  g.top2_part = t->top2_part;
+  g.part_stride = t->onepass_blocks;
+  g.n_part = t->onepass_blocks;
+  g.row_top2 = t->row_top2;
   g.Wt = t->Wt;
   g.corpus = t->corpus;
   g.pstart = t->pstart;
@@ -2033,7 +2246,6 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
     g.won = t->won[t->won_parity];
   }
   // a whole step whose windows the previous one has sampled ahead takes that buffer
-  const bool whole = which == 0x3f;
   g.sampled = 0;
   if (whole) {
     if (t->ahead_valid && t->ahead_first == first && t->ahead_n == n) {
@@ -2104,7 +2316,10 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.lbase = t->cfg.lbase;
   sp.xx = t->xx;
   sp.invf = t->invf;
-  sp.bmax_sparse = t->bmax + t->dense_blocks;
+  sp.bmax_sparse = t->bmax + t->sparse_base;
+  sp.row_top2 = t->row_top2;
+  sp.row_hits = t->row_hits;
+  sp.top2_known = top2_known ? 1u : 0u;
   sp.slot_count = t->slot_count;
   sp.pad_row = t->B;
   sp.stride = t->idx_stride;
@@ -2161,13 +2376,22 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.ldk = t->ldk;
   d.V = (uint32_t)t->V;
   d.K = t->K;
-  d.n_bmax = t->dense_blocks + t->K * FV_NB_CLASSES;
+  d.n_bmax = t->sparse_base + t->K * FV_NB_CLASSES;
   d.dense_blocks = t->dense_blocks;
+  d.sparse_base = t->sparse_base;
+  d.n_rows = (uint32_t)t->N;
+  d.active = t->onepass_active;
+  d.n_slots = (uint32_t)n_slots;
+  d.row_top2 = t->row_top2;
+  d.row_hits = t->row_hits;
+  d.top2_known = top2_known ? 1u : 0u;
+  d.top2_part = t->top2_part;
+  d.part_stride = t->onepass_blocks;
+  d.path_count = t->path_count;
   d.eps = eps;
   d.prec = t->cfg.prec;
   d.update_cut = t->update_cut;
   const size_t smem = (size_t)t->ldk * sizeof(float);
-  const bool onepass = t->onepass && fv_trainers_alive.load() == 1;
   if (onepass) {
     // both dense passes in the launch that takes the place of the first one
     if (which & 8u) {
@@ -2186,24 +2410,23 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
         t->ahead_first = next_first;
         t->ahead_n = d.ahead_n;
       }
-      const bool narrow = (uint64_t)t->K * FV_NB_CLASSES <= 2 * FV_ONEPASS_THREADS;
       const size_t smem1 = fv_onepass_smem(t);
-#define FV_CASE(U, P)                                                                     \
-  if (anti) fv_launch_onepass<U, P, true>(d, t->onepass_blocks, smem1, t->stream);        \
-  else fv_launch_onepass<U, P, false>(d, t->onepass_blocks, smem1, t->stream);
-      if (t->onepass_unroll == 8) {
-        if (narrow) { FV_CASE(8, 2) } else { FV_CASE(8, 8) }
-      } else {
-        if (narrow) { FV_CASE(16, 2) } else { FV_CASE(16, 8) }
-      }
+#define FV_CASE(U)                                                                     \
+  if (anti) fv_launch_onepass<U, true>(d, t->onepass_blocks, smem1, t->stream);        \
+  else fv_launch_onepass<U, false>(d, t->onepass_blocks, smem1, t->stream);
+      if (t->onepass_unroll == 8) { FV_CASE(8) } else { FV_CASE(16) }
 #undef FV_CASE
+      t->top2_valid = true;  // this launch leaves the shares of the matrix it writes
     }
     if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
   } else {
     if (which & 8u)
       hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
     if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
-    if (which & 16u) hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
+    if (which & 16u) {
+      hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
+      t->top2_valid = false;  // the matrix changes and nobody keeps the rows' largest weights
+    }
   }
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
   if ((which & 32u) && !onepass) {  // the single launch has finished the sparse elements as well
@@ -2309,7 +2532,18 @@ extern "C" int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separ
 
 extern "C" int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches) {
   FV_REQUIRE(t && out_launches, FV_ERR_INVALID, "null argument");
-  *out_launches = t->onepass && fv_trainers_alive.load() == 1 ? 1u : 2u;
+  const uint64_t n_slots = (uint64_t)FV_NB_CLASSES * t->B * t->w;  // of a step without the anti-Hebbian term
+  *out_launches = t->onepass && fv_trainers_alive.load() == 1 && n_slots + 1 < FV_SENTINEL_MAX ? 1u : 2u;
+  return FV_OK;
+}
+
+extern "C" int fv_trainer_get_dense_path_counts(fv_trainer *t, uint64_t *out_known, uint64_t *out_pass) {
+  FV_REQUIRE(t && out_known && out_pass, FV_ERR_INVALID, "null argument");
+  uint32_t c[2] = {0, 0};
+  FV_HIP(hipStreamSynchronize(t->stream));
+  FV_HIP(hipMemcpy(c, t->path_count, sizeof c, hipMemcpyDeviceToHost));
+  *out_known = c[0];
+  *out_pass = c[1];
   return FV_OK;
 }
 

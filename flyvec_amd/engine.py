@@ -166,6 +166,13 @@ class Trainer:
         check(self.lib.fv_trainer_get_dense_launches(self.handle, C.byref(out)))
         return out.value
 
+    @property
+    def dense_path_counts(self):
+        """(single dense launches that knew max|ds| when they started, launches that made the pass for it)."""
+        known, made = C.c_uint64(0), C.c_uint64(0)
+        check(self.lib.fv_trainer_get_dense_path_counts(self.handle, C.byref(known), C.byref(made)))
+        return known.value, made.value
+
     def _set_wait_limit(self, rounds):
         check(self.lib.fv_trainer_set_wait_limit(self.handle, int(rounds)))
 

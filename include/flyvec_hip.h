@@ -185,13 +185,19 @@ int fv_trainer_epoch_eps(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs, fl
 int fv_trainer_sync(fv_trainer *t);
 
 /* The two passes over the matrix of a step (max|ds|, flyvec/src/cu_special_reduction.cu:241, and
- * the update, flyvec/src/cuda_funcs.cu:1787-1806) run as ONE launch that keeps the matrix in
- * registers between them when it fits the device (64 MiB on 256 compute units), else as two.
+ * the update, flyvec/src/cuda_funcs.cu:1787-1806) run as ONE launch when the matrix fits the registers of
+ * the device (64 MiB on 256 compute units) and a step has fewer than 2^23 slot records, else as two.
  * launches = 1 or 2 forces the form (1 fails with FV_ERR_INVALID when the matrix does not fit),
  * 0 returns to the choice made at creation. Results are bit-identical either way. The single
  * launch needs the whole device for itself, so while a process holds more than one trainer every
  * step takes two launches whatever is set here. */
 int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches);
+/* The single launch carries the two largest |W| of every row from step to step; from them and from what
+ * the sparse-element launch reports it usually knows max|ds| (flyvec/src/cu_special_reduction.cu:241) before
+ * it reads the matrix and is then one streaming read-modify-write; otherwise it makes the pass for the
+ * maximum first, on registers. Counts of single launches so far that knew it / that made the pass (the
+ * first step on a new matrix always makes it). Same results either way. No counterpart in the reference. */
+int fv_trainer_get_dense_path_counts(fv_trainer *t, uint64_t *out_known, uint64_t *out_pass);
 int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches); /* 1 or 2: the form the next step takes */
 /* Grouping the windows of a step by winner (what flyvec/src/cuda_funcs.cu:1719-1721 leaves in
  * max_IDs and xx) runs inside the sparse-element launch when the trainer's batch is at most 16384

@@ -87,9 +87,9 @@ def test_shapes_bit_exact_with_two_dense_launches(gpu, oracle_lib, K, w, V, B):
     assert np.array_equal(Wg, Wo)
 
 
-@pytest.mark.parametrize("K,V", [(200, 20000), (300, 20000), (400, 20000), (400, 20970)])
+@pytest.mark.parametrize("K,V", [(200, 20000), (300, 20000), (400, 20000), (400, 20480)])
 def test_single_dense_launch_size_classes(gpu, oracle_lib, K, V):
-    # 32, 48, 64 and 67.1 MB of W: a thread of the single launch keeps 8, 12, 16 and 16 groups
+    # 32, 48, 64 and 65.5 MB of W: a thread of the single launch keeps 8, 12, 16 and 16 groups (40960 rows are the most: 256 blocks x 10 rows x 16)
     wg, wo, Wg, Wo = run_both(gpu, oracle_lib, V=V, K=K, w=11, B=3000, steps=4, n_tokens=120000, mean_chunk=40,
                               launches=1)
     assert np.array_equal(wg, wo)
@@ -825,3 +825,47 @@ def test_random_configurations_match_the_oracle(gpu, oracle_lib, case):
         Wg = t.get_weights()
         t.close()
         assert np.array_equal(Wg.view(np.uint32), Wo.view(np.uint32)), f"W, separate grouping {separate}, {c}"
+
+
+def test_dense_launch_knows_the_maximum_from_the_rows_largest_weights(gpu, oracle_lib):
+    """The single dense launch carries every row's two largest |W| and, with what the sparse launch reports on
+    them, knows max|ds| before it reads the matrix; where the largest weights of the deciding row are sparse
+    elements of the step it makes the pass instead. Both ways, step by step, against the checker: random weights
+    (the maximum is nearly always known), and weights whose largest entries sit on the most frequent tokens
+    (they are sparse elements of nearly every row in every step: the pass has to be made)."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    V, K, w, B = 800, 96, 9, 2000
+    tokens, offsets = small_corpus(80000, V, seed=2)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    perm = np.random.default_rng(3).permutation(len(starts)).astype(np.uint64)
+    hot = np.argsort(-np.bincount(tokens[tokens >= 0], minlength=V))[:6]
+    plain = synthetic.synapses(K, V, seed=9)
+    planted = plain.copy()
+    # the same largest value three times in every row, on tokens that nearly every window holds; being positive,
+    # the dense term of such an element (-xx * 7, xx > 0) is partly cancelled by its sparse term, so no sparse
+    # element reaches the bound |xx| * 7 that the row would have if one of the three were dense
+    planted[:, hot[:3]] = np.float32(7.0)
+    tied = plain.copy()
+    tied[:, hot[0]] = np.float32(6.0)                # one sparse element and one dense element hold the row's
+    tied[:, 5] = np.float32(-6.0) if 5 not in hot else tied[:, 5]   # largest value: the dense one decides
+    counts = {}
+    for name, W0 in (("plain", plain), ("planted", planted), ("tied", tied)):
+        t = Trainer(V, K, w, B, initial_learning_rate=1e-3)
+        t.set_dense_launches(1)
+        t.set_corpus(tokens, offsets)
+        t.set_permutation(perm)
+        t.set_weights(W0)
+        Wo = W0.copy()
+        for s in range(8):
+            t.step(s * B, B, 1e-3)
+            ref = to.train_step(Wo, to.inflate(tokens, starts, perm, s * B, B, w, V), invf, 1e-3)
+            xx, nc = t.step_stats()
+            assert np.array_equal(t.winners(B), ref["winners"]) and np.array_equal(xx, ref["xx"]), (name, s)
+            assert nc == ref["nc"], (name, s)
+        assert np.array_equal(t.get_weights().view(np.uint32), Wo.view(np.uint32)), name
+        counts[name] = t.dense_path_counts
+        t.close()
+    assert all(known + made == 8 and made >= 1 for known, made in counts.values())   # the first step makes the pass
+    assert counts["plain"][0] >= 5
+    assert counts["planted"][1] >= 4
