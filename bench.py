@@ -9,13 +9,20 @@ synthetic 10 M-token Zipf(1.07) corpus with geometric chunk lengths, fp32, every
 HBM before the timed region.  One JSON line is printed:
 
   value              training windows / s over the K timed steps
-  roofline           the dominant kernel of the step against the 8 TB/s HBM peak: achieved =
-                     algorithmic bytes of that kernel per launch / its mean duration, measured with
-                     HIP events on the trainer's stream
-  step_roofline_frac (algorithmic bytes of the whole step / 8 TB/s) / measured time per step
+  roofline           the dominant kernel of the step against the 8 TB/s HBM peak: achieved = the bytes
+                     that kernel has to move per launch / its mean duration, measured with HIP events
+                     on the trainer's stream; traffic = HBM-side bytes per launch from the rocprofv3
+                     counter runs summarised under profiles/ (read from that file, not from this run)
+  kernels            the same for every kernel of the step; the window gathers, whose bytes are largely
+                     served by the L2 caches, are held against measured HBM-side traffic and against the
+                     vector-ALU issue rate instead of against their algorithmic bytes
+  step_roofline_frac (byte model of the whole step / 8 TB/s) / measured time per step
   cpu_baseline       the CPU restatement of the same step (oracle/, C + OpenMP) timed on this host
-  hash               the batched top-k hash (1,048,576 windows, k = 32, bit-packed) the same way,
+  hash               the batched top-k hash (1,048,576 windows, k = 32, bit-packed), device-resident,
                      with the reference's numpy per-word path as its CPU baseline
+  hash_host          the same batch through the host-buffer entry point (copies included)
+  large_step         K = 1000, V = 50000, w = 15, B = 50000 on a 200 M-token corpus (400 MB matrix)
+  epoch              one full epoch over a 100 M-token corpus with device shuffle and one checkpoint
 """
 import argparse
 import json
@@ -29,71 +36,99 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # B/s, MI355X
+# vector-ALU issue rate: 256 compute units x 4 SIMDs, one wave64 instruction per SIMD every 4 cycles
+# (16 lanes per SIMD), at the 2.4 GHz peak engine clock
+VALU_ISSUE_PEAK = 256 * 4 * 2.4e9 / 4
 
 TRAIN = dict(K=400, V=20000, w=11, B=10000, n_tokens=10_000_000, lr0=2e-4, n_epochs=15, prec=1e-30,
              zipf_s=1.07, mean_chunk=25)
-# the 400 MB matrix that exceeds the 256 MB Infinity Cache; the corpus is shortened from 200 M to
-# 20 M tokens (the step does not depend on its length)
-LARGE = dict(K=1000, V=50000, w=15, B=50000, n_tokens=20_000_000, lr0=2e-4, n_epochs=15, prec=1e-30,
+LARGE = dict(K=1000, V=50000, w=15, B=50000, n_tokens=200_000_000, lr0=2e-4, n_epochs=15, prec=1e-30,
              zipf_s=1.0, mean_chunk=40)
 EPOCH = dict(K=400, V=20000, w=11, B=10000, n_tokens=100_000_000, lr0=2e-4, n_epochs=15, prec=1e-30,
              zipf_s=1.07, mean_chunk=25)
 HASH = dict(K=400, V=20000, w=11, k=32, n=1 << 20)
 
-
-# HBM-side bytes per launch at the headline configuration, from two rocprofv3 --pmc runs of this
-# script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same counter reads
-# for the plain copy kernel of --copy-calibration (FETCH_SIZE reads half the bytes copied: x2.0;
-# WRITE_SIZE reads them all: x1.0). Traffic below the algorithmic bytes means the rest was served
-# by the L2 caches.
-MEASURED_TRAFFIC = {
-    "dense_max_update": (33303.5 * 2.0 + 65249.7) * 1024,
-    "gather_winner": (28514.5 * 2.0 + 817.5) * 1024,
-    "sparse_owners": (5819.5 * 2.0 + 2993.3) * 1024,  # grouping by winner included
-    "hash": (2478239.7 * 2.0 + 82381.6) * 1024,
-    # the step as six launches (--dense-launches 2 --separate-grouping)
-    "update": (32309.5 * 2.0 + 62498.2) * 1024,
-    "absmax_ds": (31275.5 * 2.0 + 64.0) * 1024,
-    "slot_update": (621.9 * 2.0 + 1501.2) * 1024,
-    "group_xx": (312.9 * 2.0 + 87.2) * 1024,
-}
-
-# the same for --workload large-step (profiles/train_step_K1000_V50000_B50000.txt)
-MEASURED_TRAFFIC_LARGE = {
-    "gather_winner": (760768.6 * 2.0 + 5100.7) * 1024,
-    "group_xx": (1249.9 * 2.0 + 316.0) * 1024,
-    "sparse_owners": (30823.7 * 2.0 + 17905.1) * 1024,
-    "absmax_ds": (195347.6 * 2.0 + 67.9) * 1024,
-    "update": (195624.6 * 2.0 + 390612.4) * 1024,
-    "slot_update": (3550.7 * 2.0 + 11373.4) * 1024,
-}
-
-# the two passes over W of a step (and the sparse elements' update) as one launch: W stays in
-# registers between them, so the launch moves 8*K*N bytes of W while the byte model of the step
-# counts the two passes' 12*K*N
-DENSE_ONE = "dense_max_update"
+# rocprofv3 summaries of the command lines below them; their lines "@ <kernel> name=value ..." carry the
+# per-launch counter means this script quotes (HBM-side KiB fetched / written, wave-level VALU instructions)
+PROFILE = {"step": "profiles/train_step_and_hash_K400_V20000_B10000.txt",
+           "large": "profiles/train_step_K1000_V50000_B50000.txt"}
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0  # what the counters read for a plain copy kernel of known size
 
 
-def train_bytes(K, N, w, B):
-    """Algorithmic HBM bytes per step and per kernel: every window gathers w rows of K floats once;
-    W is read once for max|ds| and read + written once by the update; ds is never stored; token
-    ids, 1/f lookups and the sparse count updates are 16 bytes per window position."""
-    per = {
+def profile_counters(which):
+    """{kernel: {name: value}} from the '@' lines of a profiles/ summary ({} if the file is absent)."""
+    out = {}
+    try:
+        with open(os.path.join(ROOT, PROFILE[which])) as f:
+            for line in f:
+                if line.startswith("@ "):
+                    parts = line.split()
+                    out[parts[1]] = {k: float(v) for k, v in (p.split("=") for p in parts[2:])}
+    except OSError:
+        pass
+    return out
+
+
+def traffic_bytes(counters, kernel):
+    c = counters.get(kernel)
+    if not c or "fetch_kib" not in c or "write_kib" not in c:
+        return None
+    return (c["fetch_kib"] * FETCH_SCALE + c["write_kib"] * WRITE_SCALE) * 1024
+
+
+def kernel_bytes(K, N, w, B):
+    """Bytes every kernel of a step has to move. The window gather reads w rows of K floats per window
+    (largely from L2: the rows repeat); the dense passes read the matrix for max|ds| and read + write it
+    for the update -- the single launch keeps it in registers or knows max|ds| beforehand and so moves it
+    once each way; token ids, 1/f look-ups, slot records and sparse elements are 8 bytes per window
+    position and kernel."""
+    return {
         "gather_winner": 4 * B * w * K,
         "group_xx": 8 * B,
         "sparse_owners": 8 * B * w,
         "absmax_ds": 4 * K * N,
         "update": 8 * K * N,
         "slot_update": 8 * B * w,
+        "dense_update": 8 * K * N + 8 * B * w,
     }
-    return 4 * B * w * K + 12 * K * N + 16 * B * w, per
+
+
+def step_byte_model(K, N, w, B):
+    """The byte model the step is held to: gathers counted in full, the matrix read for max|ds| and read +
+    written for the update (12 K N), 16 bytes per window position. A scheme that skips one of those
+    passes scores above its share of this model; that is said where it applies."""
+    return 4 * B * w * K + 12 * K * N + 16 * B * w
 
 
 def hash_bytes_per_window(K, w):
     return 4 * w * K + 4 * w + 8 * ((K + 63) // 64)
 
 
-def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0, separate_grouping=False):
+def hbm_entry(kernel, nbytes, ms, traffic, source):
+    achieved = nbytes / (ms * 1e-3)
+    return {"bound": "hbm", "kernel": kernel, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK, "traffic": traffic, "traffic_source": source if traffic else None,
+            "algorithmic_bytes": nbytes}
+
+
+def gather_entry(kernel, nbytes, ms, counters, source):
+    """A window-gather kernel: its algorithmic bytes mostly hit in L2, so it is held against the HBM-side
+    traffic the counters saw and against the rate at which the vector ALUs can issue."""
+    traffic = traffic_bytes(counters, kernel)
+    out = {"kernel": kernel, "algorithmic_bytes": nbytes, "algorithmic_rate_GBps": nbytes / (ms * 1e-3) / 1e9,
+           "traffic": traffic, "traffic_source": source if traffic else None}
+    if traffic:
+        out["hbm"] = {"bound": "hbm", "achieved": traffic / (ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                      "frac": traffic / (ms * 1e-3) / HBM_PEAK, "basis": "measured HBM-side traffic / duration"}
+    insts = counters.get(kernel, {}).get("valu_insts")
+    if insts:
+        out["valu_issue"] = {"bound": "valu_issue", "achieved": insts / (ms * 1e-3) / 1e9, "peak": VALU_ISSUE_PEAK / 1e9,
+                             "unit": "G wave-instructions/s", "frac": insts / (ms * 1e-3) / VALU_ISSUE_PEAK,
+                             "insts_per_launch": insts, "insts_source": source}
+    return out
+
+
+def bench_train(steps, warmup, cpu_seconds, c=TRAIN, which="step", dense_launches=0, separate_grouping=False):
     from flyvec_amd import Trainer, synthetic
     tokens, offsets = synthetic.corpus(c["n_tokens"], c["V"], s=c["zipf_s"], mean_chunk=c["mean_chunk"])
     W0 = synthetic.synapses(c["K"], c["V"], seed=5)
@@ -113,12 +148,14 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0, separate_
     for s in range(warmup):
         t.step(s * c["B"], c["B"], eps)
     t.sync()
+    known0, made0 = t.dense_path_counts
     # timed region: exactly `steps` steps, device idle before and after
     t0 = time.perf_counter()
     for s in range(steps):
         t.step((warmup + s) * c["B"], c["B"], eps)
     t.sync()
     wall = time.perf_counter() - t0
+    known1, made1 = t.dense_path_counts
     # the same number of steps again, timed by two HIP events on the trainer's stream
     total_ms, _ = t.time_steps((warmup + steps) * c["B"], steps, eps, per_kernel=False)
     ev_ms_per_step = total_ms / steps
@@ -131,42 +168,53 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, dense_launches=0, separate_
     t.close()
 
     N = 2 * c["V"]
-    step_bytes, per_kernel = train_bytes(c["K"], N, c["w"], c["B"])
+    per_kernel = kernel_bytes(c["K"], N, c["w"], c["B"])
     if launches == 1:
-        # max|ds|, the update and the slot update ran as one launch (timed under the first name;
-        # the others are empty)
-        parts = ("absmax_ds", "update", "slot_update")
-        kern_ms[DENSE_ONE] = sum(kern_ms.pop(k) for k in parts)
-        per_kernel[DENSE_ONE] = sum(per_kernel.pop(k) for k in parts)
+        # max|ds|, the update and the slot update ran as one launch (timed under the first name; the others are empty)
+        kern_ms["dense_update"] = sum(kern_ms.pop(k) for k in ("absmax_ds", "update", "slot_update"))
+        for k in ("absmax_ds", "update", "slot_update"):
+            per_kernel.pop(k)
+    else:
+        per_kernel.pop("dense_update")
     if not grouping_separate:
         # the sparse launch has grouped the windows by winner itself: no grouping launch ran
         kern_ms["sparse_owners"] += kern_ms.pop("group_xx")
         per_kernel["sparse_owners"] += per_kernel.pop("group_xx")
+    counters = profile_counters(which)
+    source = PROFILE[which]
+    kernels = {}
+    for k, ms in kern_ms.items():
+        if k == "gather_winner":
+            kernels[k] = gather_entry(k, per_kernel[k], ms, counters, source)
+        else:
+            kernels[k] = hbm_entry(k, per_kernel[k], ms, traffic_bytes(counters, k), source)
+        kernels[k]["ms"] = ms
     dom = max(kern_ms, key=kern_ms.get)
-    achieved = per_kernel[dom] / (kern_ms[dom] * 1e-3)
+    if dom == "gather_winner":
+        g = kernels[dom]
+        roofline = dict(g.get("hbm") or {"bound": "hbm", "achieved": None, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": None})
+        roofline.update(kernel=dom, traffic=g["traffic"], traffic_source=g["traffic_source"],
+                        algorithmic_bytes=g["algorithmic_bytes"])
+    else:
+        roofline = {k: v for k, v in kernels[dom].items() if k != "ms"}
+    model = step_byte_model(c["K"], N, c["w"], c["B"])
     ms_per_step = wall / steps * 1e3
     out = {
         "value": steps * c["B"] / wall,
         "ms_per_step": ms_per_step,
         "event_ms_per_step": ev_ms_per_step,
-        "kernel_ms": kern_ms,
-        "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK,
-                     "traffic": (MEASURED_TRAFFIC if c is TRAIN else MEASURED_TRAFFIC_LARGE).get(dom),
-                     "algorithmic_bytes": per_kernel[dom]},
+        "roofline": roofline,
+        "kernels": kernels,
         "dense_launches": launches,
         "grouping_launch": "own" if grouping_separate else "in sparse_owners",
-        "step_roofline_frac": (step_bytes / HBM_PEAK) / (ms_per_step * 1e-3),
-        "step_algorithmic_bytes": step_bytes,
+        "step_roofline_frac": (model / HBM_PEAK) / (ms_per_step * 1e-3),
+        "step_byte_model": model,
         "n_windows": nwin,
     }
-
-    if dom == DENSE_ONE:
-        # what the launch has to move (W read once, written once) and the rate on that count
-        moved = 8 * c["K"] * N + 8 * c["B"] * c["w"]
-        out["roofline"]["moved_bytes"] = moved
-        out["roofline"]["frac_of_moved"] = moved / (kern_ms[dom] * 1e-3) / HBM_PEAK
-
+    if launches == 1:
+        out["dense_launch_paths"] = {"knew_max_ds": known1 - known0, "made_the_pass": made1 - made0,
+                                     "note": "timed steps whose single dense launch took max|ds| from the carried "
+                                             "row maxima / read the matrix for it first"}
     if cpu_seconds > 0:
         from oracle import train_oracle as to
         starts = to.window_starts(offsets, c["w"])
@@ -203,6 +251,7 @@ def bench_epoch(c=EPOCH):
     nwin = t.num_windows
     t.shuffle(1)
     t.run_epoch(0, c["n_epochs"])      # warm-up epoch: first-touch of every buffer
+    known0, made0 = t.dense_path_counts
     t0 = time.perf_counter()
     t.shuffle(2)
     t.sync()
@@ -216,18 +265,24 @@ def bench_epoch(c=EPOCH):
         np.save(os.path.join(d, "flyvec_model_1.npy"), W)
     t_ckpt = time.perf_counter() - t2
     total = time.perf_counter() - t0
+    known1, made1 = t.dense_path_counts
     t.close()
     n_steps = (nwin + c["B"] - 1) // c["B"]
-    step_bytes, _ = train_bytes(c["K"], 2 * c["V"], c["w"], c["B"])
-    return {"value": nwin / total, "seconds_per_epoch": total, "n_windows": nwin, "n_steps": n_steps,
+    model = step_byte_model(c["K"], 2 * c["V"], c["w"], c["B"])
+    return {"metric": "train windows/s over one full epoch", "value": nwin / total, "unit": "windows/s",
+            "config": {"workload": f"full training epoch: {c['n_tokens']} Zipf({c['zipf_s']}) tokens, K={c['K']} "
+                                   f"Nvoc={c['V']} w={c['w']} B={c['B']}, {nwin} windows, device shuffle before "
+                                   f"and one .npy checkpoint after (second epoch of a run)"},
+            "seconds_per_epoch": total, "n_windows": nwin, "n_steps": n_steps,
             "ms_per_step": t_steps / n_steps * 1e3,
             "breakdown_s": {"shuffle": t_shuffle, "minibatch_loop": t_steps, "checkpoint": t_ckpt,
                             "setup_once": t_setup, "synthetic_corpus_generation": t_gen},
-            "step_roofline_frac": (step_bytes * (nwin / c["B"]) / HBM_PEAK) / t_steps}
+            "step_roofline_frac": (model * (nwin / c["B"]) / HBM_PEAK) / t_steps,
+            "dense_launch_paths": {"knew_max_ds": known1 - known0, "made_the_pass": made1 - made0}}
 
 
-def bench_hash(reps, cpu_seconds):
-    from flyvec_amd import Hasher, synthetic
+def bench_hash(reps, cpu_seconds, host_reps=5, host=True):
+    from flyvec_amd import Hasher, synthetic, _lib
     from flyvec_amd._lib import DeviceBuffer
     c = HASH
     W = synthetic.synapses(c["K"], c["V"], seed=1)
@@ -239,14 +294,40 @@ def bench_hash(reps, cpu_seconds):
     ms = h.time_windows(d_idx, c["n"], c["w"], c["k"], bits_buf=d_bits, reps=reps)
     h.sync()
     bpw = hash_bytes_per_window(c["K"], c["w"])
-    achieved = bpw * c["n"] / (ms * 1e-3)
+    counters = profile_counters("step")
+    workload = (f"batched contextual hash: K={c['K']} V={c['V']} w={c['w']} k={c['k']} n={c['n']} windows, "
+                f"{h.words} uint64 words out")
     out = {"metric": "hash codes/s", "value": c["n"] / (ms * 1e-3), "unit": "codes/s", "ms_per_batch": ms,
-           "config": {"workload": f"batched contextual hash: K={c['K']} V={c['V']} w={c['w']} k={c['k']} "
-                                  f"n={c['n']} windows, 7 uint64 words out"},
-           "dtype": "f32",
-           "roofline": {"bound": "hbm", "kernel": "hash", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
-                        "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": MEASURED_TRAFFIC["hash"],
-                        "algorithmic_bytes": bpw * c["n"]}}
+           "config": {"workload": workload + ", indices and codes resident in HBM"}, "dtype": "f32",
+           "roofline": gather_entry("hash", bpw * c["n"], ms, counters, PROFILE["step"]),
+           "byte_model_frac": (bpw * c["n"] / HBM_PEAK) / (ms * 1e-3),
+           "byte_model_note": "time the algorithmic bytes would take at 8 TB/s / measured time; above 1 because the "
+                              "64 MB matrix is served by the L2 and Infinity caches"}
+    if not host:
+        h.close()
+        d_idx.free()
+        d_bits.free()
+        return out, None
+    # the same batch from host buffers through fv_hash_windows: copies included
+    host = {}
+    bits = np.empty((c["n"], h.words), dtype=np.uint64)
+    pin_idx = _lib.pinned_empty(idx.shape, np.int32)
+    pin_idx[:] = idx
+    pin_bits = _lib.pinned_empty(bits.shape, np.uint64)
+    pin_bits[:] = 0
+    for name, i, o in (("pageable", idx, bits), ("page_locked", pin_idx, pin_bits)):
+        h.hash_windows(i, c["k"], out_bits=o)
+        best = float("inf")
+        for _ in range(host_reps):
+            t0 = time.perf_counter()
+            h.hash_windows(i, c["k"], out_bits=o)
+            best = min(best, time.perf_counter() - t0)
+        host[name] = {"value": c["n"] / best, "unit": "codes/s", "ms_per_batch": best * 1e3}
+    moved = idx.nbytes + bits.nbytes
+    out_host = {"metric": "hash codes/s from host buffers (PCIe-inclusive)", "config": {"workload": workload + ", numpy "
+                "buffers in host memory through fv_hash_windows (chunks on two streams)"},
+                "bytes_over_the_link": moved, "buffers": host,
+                "link_GBps_page_locked": moved / (host["page_locked"]["ms_per_batch"] * 1e-3) / 1e9}
     if cpu_seconds > 0:
         from oracle import hash_oracle as ho
         ids = synthetic.zipf_ids(4096, c["V"], seed=2)
@@ -267,7 +348,24 @@ def bench_hash(reps, cpu_seconds):
     h.close()
     d_idx.free()
     d_bits.free()
-    return out
+    return out, out_host
+
+
+def train_line(c, tr, steps, warmup):
+    line = {
+        "metric": f"train windows/s at K={c['K']},Nvoc={c['V'] // 1000}k",
+        "value": tr["value"], "unit": "windows/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": tr["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"single training minibatch step: K={c['K']} Nvoc={c['V']} w={c['w']} B={c['B']}, "
+                               f"{c['n_tokens']} Zipf({c['zipf_s']}) tokens, geometric chunks (mean {c['mean_chunk']}), "
+                               f"{tr['n_windows']} windows, lr 2e-4, fp32"},
+    }
+    for k in ("roofline", "step_roofline_frac", "step_byte_model", "event_ms_per_step", "kernels", "dense_launches",
+              "grouping_launch", "dense_launch_paths", "cpu_baseline"):
+        if k in tr:
+            line[k] = tr[k]
+    return line
 
 
 def main():
@@ -277,14 +375,17 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample length (0 = skip)")
     ap.add_argument("--no-hash", action="store_true")
+    ap.add_argument("--no-hash-host", action="store_true", help="skip the host-buffer hash timings (profiling runs: "
+                    "their chunk launches would mix into the per-kernel means)")
+    ap.add_argument("--no-large", action="store_true", help="skip the K=1000, V=50000 step")
+    ap.add_argument("--no-epoch", action="store_true", help="skip the full epoch over 100 M tokens")
     ap.add_argument("--separate-grouping", action="store_true",
                     help="group the windows by winner in a launch of its own (the default does it inside the sparse launch)")
     ap.add_argument("--dense-launches", type=int, choices=[0, 1, 2], default=0,
                     help="the passes over W of a step as one launch (1), two (2), or as the library chooses (0)")
-    ap.add_argument("--workload", choices=["step", "large-step", "epoch"], default="step",
-                    help="step: the headline minibatch step (default); large-step: K=1000, V=50000, w=15, "
-                         "B=50000 (400 MB matrix); epoch: one full epoch over 100 M tokens with shuffle and "
-                         "checkpoint")
+    ap.add_argument("--workload", choices=["all", "step", "large-step", "epoch"], default="all",
+                    help="all: the headline step with the hash batch, the large step and the epoch as sub-objects "
+                         "(default); step / large-step / epoch: that workload alone as the line")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB copy kernel (yardstick for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -294,43 +395,33 @@ def main():
     from flyvec_amd import _lib
     info = _lib.device_info()
     if args.workload == "epoch":
-        c = EPOCH
-        ep = bench_epoch(c)
-        print(json.dumps({
-            "metric": "train windows/s over one full epoch", "value": ep["value"], "unit": "windows/s",
-            "n_gpus": 1, "steps": ep["n_steps"], "warmup": ep["n_steps"], "ms_per_step": ep["ms_per_step"],
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-            "config": {"workload": f"full training epoch: {c['n_tokens']} Zipf(1.07) tokens, K={c['K']} "
-                                   f"Nvoc={c['V']} w={c['w']} B={c['B']}, {ep['n_windows']} windows, device "
-                                   f"shuffle before and one .npy checkpoint after"},
-            "device": info["name"].strip(), "seconds_per_epoch": ep["seconds_per_epoch"],
-            "breakdown_s": ep["breakdown_s"], "step_roofline_frac": ep["step_roofline_frac"]}))
+        ep = bench_epoch(EPOCH)
+        ep.update({"n_gpus": 1, "steps": ep["n_steps"], "warmup": ep["n_steps"], "higher_is_better": True,
+                   "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                   "device": info["name"].strip()})
+        print(json.dumps(ep))
         return
-    c = LARGE if args.workload == "large-step" else TRAIN
     if args.workload == "large-step":
-        args.steps, args.warmup, args.no_hash = min(args.steps, 50), min(args.warmup, 5), True
-    tr = bench_train(args.steps, args.warmup, args.cpu_seconds, c, args.dense_launches, args.separate_grouping)
-    line = {
-        "metric": f"train windows/s at K={c['K']},Nvoc={c['V'] // 1000}k",
-        "value": tr["value"], "unit": "windows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": tr["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"single training minibatch step: K={c['K']} Nvoc={c['V']} w={c['w']} B={c['B']}, "
-                               f"{c['n_tokens']} Zipf({c['zipf_s']}) tokens, geometric chunks (mean {c['mean_chunk']}), "
-                               f"{tr['n_windows']} windows, lr 2e-4, fp32"},
-        "device": info["name"].strip(),
-        "roofline": tr["roofline"],
-        "step_roofline_frac": tr["step_roofline_frac"],
-        "step_algorithmic_bytes": tr["step_algorithmic_bytes"],
-        "event_ms_per_step": tr["event_ms_per_step"],
-        "kernel_ms": tr["kernel_ms"],
-        "dense_launches": tr["dense_launches"],
-        "grouping_launch": tr["grouping_launch"],
-    }
-    if "cpu_baseline" in tr:
-        line["cpu_baseline"] = tr["cpu_baseline"]
+        steps, warmup = min(args.steps, 50), min(args.warmup, 5)
+        tr = bench_train(steps, warmup, args.cpu_seconds, LARGE, "large", args.dense_launches, args.separate_grouping)
+        line = train_line(LARGE, tr, steps, warmup)
+        line["device"] = info["name"].strip()
+        print(json.dumps(line))
+        return
+    tr = bench_train(args.steps, args.warmup, args.cpu_seconds, TRAIN, "step", args.dense_launches,
+                     args.separate_grouping)
+    line = train_line(TRAIN, tr, args.steps, args.warmup)
+    line["device"] = info["name"].strip()
     if not args.no_hash:
-        line["hash"] = bench_hash(reps=10, cpu_seconds=min(args.cpu_seconds, 5.0))
+        line["hash"], line["hash_host"] = bench_hash(reps=10, cpu_seconds=min(args.cpu_seconds, 5.0),
+                                                     host=not args.no_hash_host)
+    if args.workload == "all":
+        if not args.no_large:
+            steps, warmup = min(args.steps, 30), min(args.warmup, 5)
+            lt = bench_train(steps, warmup, 0.0, LARGE, "large", args.dense_launches, args.separate_grouping)
+            line["large_step"] = train_line(LARGE, lt, steps, warmup)
+        if not args.no_epoch:
+            line["epoch"] = bench_epoch(EPOCH)
     if args.copy_calibration:
         nbytes = 1 << 30
         ms = _lib.calibration_copy(nbytes, reps=5)

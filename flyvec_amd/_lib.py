@@ -157,6 +157,35 @@ def calibration_copy(nbytes, reps=5):
     return ms.value
 
 
+class _PinnedBlock:
+    """Page-locked host memory from fv_host_alloc_pinned, returned with fv_host_free_pinned."""
+
+    def __init__(self, nbytes):
+        p = C.c_void_p()
+        check(load().fv_host_alloc_pinned(max(int(nbytes), 1), C.byref(p)))
+        self.ptr = p
+
+    def __del__(self):
+        try:
+            if self.ptr is not None and self.ptr.value:
+                load().fv_host_free_pinned(self.ptr)
+        except Exception:
+            pass
+        self.ptr = None
+
+
+def pinned_empty(shape, dtype):
+    """A numpy array over page-locked host memory: the device copies such buffers by DMA without
+    staging, which is what lets the host-buffer entry points (fv_hash_windows, fv_hash_targets) overlap their
+    copies with the kernel. The memory is returned when the array and its views are gone."""
+    dtype = np.dtype(dtype)
+    n = int(np.prod(shape))
+    block = _PinnedBlock(n * dtype.itemsize)
+    raw = (C.c_ubyte * max(n * dtype.itemsize, 1)).from_address(block.ptr.value)
+    raw._owner = block  # the ctypes view is the array's base and keeps the block alive
+    return np.frombuffer(raw, dtype=dtype, count=n).reshape(shape)
+
+
 class DeviceBuffer:
     """A block of HBM owned through fv_dev_alloc / fv_dev_free."""
 

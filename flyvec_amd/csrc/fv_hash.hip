@@ -19,6 +19,20 @@
 
 #include "fv_internal.h"
 
+// Host-buffer batches go through the device in chunks on two streams of equal priority, so that one
+// chunk's copies run while the other's kernel does: per stream a device buffer for the chunk's indices and
+// one for each kind of output, kept from call to call (grown when a call needs more).
+#define FV_HASH_LANES 2
+#define FV_HASH_CHUNK (1u << 17)  // windows per chunk
+
+struct fv_hash_lane {
+  hipStream_t stream;
+  int32_t *idx;
+  uint64_t *bits;
+  int8_t *codes;
+  size_t idx_cap, bits_cap, codes_cap;  // bytes
+};
+
 struct fv_hasher {
   uint32_t K, ldk;
   uint64_t N;
@@ -26,6 +40,7 @@ struct fv_hasher {
   float *Wt;
   uint32_t *err;  // device flag: a column index outside [-1, N) was met
   unsigned max_blocks;
+  fv_hash_lane lane[FV_HASH_LANES];  // lane 0 runs on `stream`
 };
 
 struct fv_hash_args {
@@ -110,8 +125,9 @@ static void fv_launch_hash(const fv_hash_args &a, unsigned blocks, hipStream_t s
 }
 
 static int fv_enqueue_hash(fv_hasher *h, const int32_t *idx_dev, uint64_t n, uint32_t w, uint32_t k,
-                           int32_t shift, uint64_t *bits_dev, int8_t *codes_dev) {
+                           int32_t shift, uint64_t *bits_dev, int8_t *codes_dev, hipStream_t stream = nullptr) {
   if (n == 0) return FV_OK;
+  if (!stream) stream = h->stream;
   fv_hash_args a;
   a.Wt = h->Wt;
   a.idx = idx_dev;
@@ -128,7 +144,7 @@ static int fv_enqueue_hash(fv_hasher *h, const int32_t *idx_dev, uint64_t n, uin
   uint64_t want = (n + 3) / 4;
   unsigned blocks = (unsigned)(want < h->max_blocks ? want : h->max_blocks);
   switch ((h->K + 63) / 64) {
-#define FV_CASE(NV) case NV: fv_launch_hash<NV>(a, blocks, h->stream); break;
+#define FV_CASE(NV) case NV: fv_launch_hash<NV>(a, blocks, stream); break;
     FV_CASE(1) FV_CASE(2) FV_CASE(3) FV_CASE(4) FV_CASE(5) FV_CASE(6) FV_CASE(7) FV_CASE(8)
     FV_CASE(9) FV_CASE(10) FV_CASE(11) FV_CASE(12) FV_CASE(13) FV_CASE(14) FV_CASE(15) FV_CASE(16)
     FV_CASE(17) FV_CASE(18) FV_CASE(19) FV_CASE(20) FV_CASE(21) FV_CASE(22) FV_CASE(23) FV_CASE(24)
@@ -154,6 +170,16 @@ static int fv_check_hash_args(fv_hasher *h, uint32_t w, uint32_t k) {
 extern "C" int fv_hasher_destroy(fv_hasher *h) {
   if (!h) return FV_OK;
   if (h->stream) (void)hipStreamSynchronize(h->stream);
+  for (int l = 0; l < FV_HASH_LANES; ++l) {
+    fv_hash_lane &ln = h->lane[l];
+    if (ln.stream && ln.stream != h->stream) {
+      (void)hipStreamSynchronize(ln.stream);
+      (void)hipStreamDestroy(ln.stream);
+    }
+    (void)hipFree(ln.idx);
+    (void)hipFree(ln.bits);
+    (void)hipFree(ln.codes);
+  }
   (void)hipFree(h->Wt);
   (void)hipFree(h->err);
   if (h->stream) (void)hipStreamDestroy(h->stream);
@@ -225,36 +251,69 @@ extern "C" int fv_hash_windows_dev(fv_hasher *h, const int32_t *idx_dev, uint64_
   return fv_enqueue_hash(h, idx_dev, n, w, k, 0, out_bits_dev, out_codes_dev);
 }
 
+// Makes a lane's buffer hold at least `bytes` (freed and allocated anew when it does not).
+template <typename P>
+static int fv_hash_reserve(P **buf, size_t *cap, size_t bytes) {
+  if (*cap >= bytes) return FV_OK;
+  (void)hipFree(*buf);
+  *buf = nullptr;
+  *cap = 0;
+  FV_HIP(hipMalloc((void **)buf, bytes));
+  *cap = bytes;
+  return FV_OK;
+}
+
+// A batch in host memory: chunks of FV_HASH_CHUNK windows alternate between the lanes; on its lane a
+// chunk is copied in, hashed and copied out in stream order, so the copies of one chunk overlap the kernel
+// of the other. Host buffers from fv_host_alloc_pinned are copied by DMA as they are; pageable ones go
+// through the runtime's staging. Nothing is allocated once the lanes' buffers have reached the chunk size.
 static int fv_hash_host(fv_hasher *h, const int32_t *idx, uint64_t n, uint32_t w, uint32_t k, int32_t shift,
                         uint64_t *out_bits, int8_t *out_codes) {
   if (n == 0) return FV_OK;
   FV_REQUIRE(idx, FV_ERR_INVALID, "null index buffer");
   const uint32_t words = (h->K + 63) / 64;
-  int32_t *d_idx = nullptr;
-  uint64_t *d_bits = nullptr;
-  int8_t *d_codes = nullptr;
+  const uint64_t chunk = n < FV_HASH_CHUNK ? n : FV_HASH_CHUNK;
+  const int lanes = n > chunk ? FV_HASH_LANES : 1;
+  FV_HIP(hipStreamSynchronize(h->stream));  // what the caller enqueued on the hasher's stream comes first
+  for (int l = 0; l < lanes; ++l) {
+    fv_hash_lane &ln = h->lane[l];
+    if (!ln.stream) {
+      if (l == 0)
+        ln.stream = h->stream;
+      else
+        FV_HIP(hipStreamCreate(&ln.stream));
+    }
+    FV_TRY(fv_hash_reserve(&ln.idx, &ln.idx_cap, chunk * w * sizeof(int32_t)));
+    if (out_bits) FV_TRY(fv_hash_reserve(&ln.bits, &ln.bits_cap, chunk * words * sizeof(uint64_t)));
+    if (out_codes) FV_TRY(fv_hash_reserve(&ln.codes, &ln.codes_cap, chunk * (size_t)h->K));
+  }
   int rc = FV_OK;
-  hipError_t e = hipMalloc((void **)&d_idx, n * w * sizeof(int32_t));
-  if (e == hipSuccess && out_bits) e = hipMalloc((void **)&d_bits, n * words * sizeof(uint64_t));
-  if (e == hipSuccess && out_codes) e = hipMalloc((void **)&d_codes, n * (uint64_t)h->K);
-  if (e == hipSuccess)
-    e = hipMemcpyAsync(d_idx, idx, n * w * sizeof(int32_t), hipMemcpyHostToDevice, h->stream);
-  if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "hash staging failed: %s", hipGetErrorString(e));
-  if (rc == FV_OK) rc = fv_enqueue_hash(h, d_idx, n, w, k, shift, d_bits, d_codes);
-  if (rc == FV_OK && out_bits) {
-    e = hipMemcpyAsync(out_bits, d_bits, n * words * sizeof(uint64_t), hipMemcpyDeviceToHost, h->stream);
-    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
+  uint64_t c = 0;
+  for (uint64_t first = 0; first < n && rc == FV_OK; first += chunk, ++c) {
+    fv_hash_lane &ln = h->lane[c % lanes];
+    const uint64_t m = n - first < chunk ? n - first : chunk;
+    hipError_t e = hipMemcpyAsync(ln.idx, idx + first * w, m * w * sizeof(int32_t), hipMemcpyHostToDevice, ln.stream);
+    if (e != hipSuccess) {
+      rc = fv_fail(FV_ERR_HIP, "hash upload failed: %s", hipGetErrorString(e));
+      break;
+    }
+    rc = fv_enqueue_hash(h, ln.idx, m, w, k, shift, out_bits ? ln.bits : nullptr, out_codes ? ln.codes : nullptr,
+                         ln.stream);
+    if (rc == FV_OK && out_bits) {
+      e = hipMemcpyAsync(out_bits + first * words, ln.bits, m * words * sizeof(uint64_t), hipMemcpyDeviceToHost, ln.stream);
+      if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
+    }
+    if (rc == FV_OK && out_codes) {
+      e = hipMemcpyAsync(out_codes + first * (uint64_t)h->K, ln.codes, m * (uint64_t)h->K, hipMemcpyDeviceToHost, ln.stream);
+      if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
+    }
   }
-  if (rc == FV_OK && out_codes) {
-    e = hipMemcpyAsync(out_codes, d_codes, n * (uint64_t)h->K, hipMemcpyDeviceToHost, h->stream);
-    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
+  for (int l = 1; l < lanes; ++l) {
+    const hipError_t e = hipStreamSynchronize(h->lane[l].stream);
+    if (e != hipSuccess && rc == FV_OK) rc = fv_fail(FV_ERR_HIP, "hash stream failed: %s", hipGetErrorString(e));
   }
-  int rs = fv_hasher_sync(h);
-  if (rc == FV_OK) rc = rs;
-  (void)hipFree(d_idx);
-  (void)hipFree(d_bits);
-  (void)hipFree(d_codes);
-  return rc;
+  const int rs = fv_hasher_sync(h);  // lane 0, and the flag for indices out of range
+  return rc == FV_OK ? rs : rc;
 }
 
 extern "C" int fv_hash_windows(fv_hasher *h, const int32_t *idx, uint64_t n, uint32_t w, uint32_t k,

@@ -771,7 +771,7 @@ __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uin
 // the block of class 0 leaves xx[h], the neuron's count and its base for the dense launch and clears
 // the neuron's row of the other bit-row buffer.
 template <bool DELTA, bool GROUPING>
-__global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6))) void fv_sparse_kernel(fv_sparse_args a) {
+__device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   static_assert(!(DELTA && GROUPING), "the anti-Hebbian form has its two lists grouped by launches of their own");
   __shared__ uint32_t cnt[FV_NB_CNT_WORDS];
   __shared__ uint32_t cnt2[DELTA ? FV_NB_CNT_WORDS : 4];
@@ -783,7 +783,6 @@ __global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6
   __shared__ ord_t ord[FV_SP_STAGE];
   __shared__ uint32_t sh_pos;
   __shared__ float sh_xx;
-  __shared__ float2 sh_top2;
   __shared__ uint32_t sh_hits[2];
   __shared__ float sc64[GROUPING ? 64 : 1];  // activations of a neuron with up to 64 windows, by rank
   __shared__ float wave_max[16];
@@ -875,12 +874,9 @@ __global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6
     }
     return;
   }
-  // the row's two largest weights wait in LDS for the elements (every path to them passes a barrier)
-  // and so do the counts of the block's elements that hold the largest / the second largest
-  if (tid == 0) {
-    sh_top2 = a.top2_known ? a.row_top2[h] : make_float2(0.0f, 0.0f);
-    sh_hits[0] = sh_hits[1] = 0;
-  }
+  // counts of the block's elements that hold the row's largest / second largest weight (every path to the
+  // elements passes a barrier)
+  if (tid == 0) sh_hits[0] = sh_hits[1] = 0;
   // The launch lasts as long as its few heaviest blocks: their waves go first wherever they share a
   // SIMD with the waves of light blocks.
   if (c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
@@ -1087,6 +1083,8 @@ __global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6
       // number of the round's first record, for the sentinels (saturated: a step with more records than a
       // sentinel can name is not finished by the launch that reads the numbers)
       const uint32_t record0 = (uint32_t)min(slot_first + emitted, (uint64_t)FV_SENTINEL_MAX);
+      // the row's two largest weights: the same address in the whole block, fetched where they are used
+      const float2 top2 = a.top2_known ? a.row_top2[h] : make_float2(0.0f, 0.0f);
       for (uint32_t eb = tid; eb < take; eb += 4 * T) {
         uint32_t pe[4], ne[4], n2e[4];
         float wv[4], fe[4], le[4];
@@ -1127,7 +1125,6 @@ __global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6
             if (DELTA) a.slot_n2[slot_first + emitted + eb + u * T] = n2e[u];
             a.Wt[pe[u]] = fv_sentinel(record0 + eb + u * T);
             const float aw = fabsf(wv[u]);
-            const float2 top2 = sh_top2;
             if (aw == top2.x) atomicAdd(&sh_hits[0], 1u);  // a few per step over the whole grid
             else if (aw == top2.y) atomicAdd(&sh_hits[1], 1u);
             if (x_h != 0.0f)
@@ -1145,6 +1142,18 @@ __global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6
     a.slot_count[blockIdx.x] = emitted;
     a.row_hits[blockIdx.x] = min(sh_hits[0], 3u) | (min(sh_hits[1], 3u) << 2);
   }
+}
+
+template <bool DELTA>
+__global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
+  fv_sparse_block<DELTA, false>(a);
+}
+
+// The form that groups for itself: with its 16-bit window ids six blocks fit a compute unit's LDS, and
+// the register count is held to what six waves per SIMD allow.
+__global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6))) void fv_sparse_grouping_kernel(
+    fv_sparse_args a) {
+  fv_sparse_block<false, true>(a);
 }
 
 // ---- kernel 4: dense passes over the matrix (one launch, or 4a + 5 + 6) ---------------------------
@@ -2339,11 +2348,11 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   if (which & 4u) {
     const dim3 sp_grid(t->K * FV_NB_CLASSES), sp_block(FV_SP_THREADS);
     if (anti)
-      hipLaunchKernelGGL((fv_sparse_kernel<true, false>), sp_grid, sp_block, 0, t->stream, sp);
+      hipLaunchKernelGGL(fv_sparse_kernel<true>, sp_grid, sp_block, 0, t->stream, sp);
     else if (grouping_in_sparse)
-      hipLaunchKernelGGL((fv_sparse_kernel<false, true>), sp_grid, sp_block, 0, t->stream, sp);
+      hipLaunchKernelGGL(fv_sparse_grouping_kernel, sp_grid, sp_block, 0, t->stream, sp);
     else
-      hipLaunchKernelGGL((fv_sparse_kernel<false, false>), sp_grid, sp_block, 0, t->stream, sp);
+      hipLaunchKernelGGL(fv_sparse_kernel<false>, sp_grid, sp_block, 0, t->stream, sp);
   }
   if (ev) FV_HIP(hipEventRecord(ev[3], t->stream));
   fv_dense_args d;

@@ -265,16 +265,21 @@ class Hasher:
         check(self.lib.fv_hash_targets(self.handle, ptr(ids), len(ids), k, ptr(out)))
         return out
 
-    def hash_windows(self, idx, k=50, packed=True, codes=False):
+    def hash_windows(self, idx, k=50, packed=True, codes=False, out_bits=None, out_codes=None):
         """idx (n, w) int32 column indices (-1 = masked). Returns packed uint64 words, int8 codes,
-        or both as a tuple."""
+        or both as a tuple. out_bits / out_codes: arrays to fill instead of new ones (page-locked ones
+        from flyvec_amd._lib.pinned_empty, like a page-locked idx, are copied without staging)."""
         self._check_k(k)
         idx = np.ascontiguousarray(idx, dtype=np.int32)
         if idx.ndim != 2:
             raise ValueError("idx must be (n, w)")
         n, w = idx.shape
-        bits = np.empty((n, self.words), dtype=np.uint64) if packed else None
-        cds = np.empty((n, self.hid), dtype=np.int8) if codes else None
+        for out, shape, dt in ((out_bits, (n, self.words), np.uint64), (out_codes, (n, self.hid), np.int8)):
+            if out is not None and (out.shape != shape or out.dtype != dt or not out.flags.c_contiguous):
+                raise ValueError(f"output must be a C-contiguous {np.dtype(dt).name} array of shape {shape}")
+        packed, codes = packed or out_bits is not None, codes or out_codes is not None
+        bits = (out_bits if out_bits is not None else np.empty((n, self.words), dtype=np.uint64)) if packed else None
+        cds = (out_codes if out_codes is not None else np.empty((n, self.hid), dtype=np.int8)) if codes else None
         check(self.lib.fv_hash_windows(self.handle, ptr(idx), n, w, k, ptr(bits), ptr(cds)))
         if packed and codes:
             return bits, cds

@@ -181,3 +181,51 @@ def test_flyvec_wrapper_stop_words_and_export(gpu, tmp_path):
     assert table["brain"] == ho.sparse_code(W[:, V + 4], 10).astype(int).tolist() and sum(table["brain"]) == 10
     with pytest.raises(NotImplementedError):
         FlyVec.load()
+
+
+def test_host_batches_in_chunks_on_two_streams(gpu):
+    """Host-buffer batches larger than one chunk (131072 windows) alternate between two streams: ragged sizes
+    around the chunk boundaries, pageable and page-locked buffers, both outputs, the device-resident entry point
+    as the reference, and an index out of range in a late chunk."""
+    from flyvec_amd import Hasher, _lib, synthetic
+    from flyvec_amd._lib import DeviceBuffer
+    from oracle import hash_oracle as ho
+    K, V, w, k = 200, 3000, 7, 24
+    W = synthetic.synapses(K, V, seed=3)
+    h = Hasher(W)
+    chunk = 1 << 17
+    for n in (chunk - 1, chunk, chunk + 1, 2 * chunk + 77, 3 * chunk + 5):
+        idx = synthetic.window_indices(n, w, V, seed=n % 97)
+        idx[::1001, 2] = -1
+        bits, codes = h.hash_windows(idx, k, packed=True, codes=True)
+        d_idx, d_bits = DeviceBuffer.from_numpy(idx), DeviceBuffer(n * h.words * 8)
+        h.hash_windows_dev(d_idx, n, w, k, bits_buf=d_bits)
+        h.sync()
+        assert np.array_equal(bits, d_bits.to_numpy(np.uint64, (n, h.words)))
+        assert np.array_equal(ho.pack_codes(codes), bits)
+        for sl in (slice(0, 3000), slice(chunk - 1500, chunk + 1500), slice(n - 3000, n)):
+            assert np.array_equal(codes[sl], ho.hash_windows(W, idx[sl], k))
+        d_idx.free()
+        d_bits.free()
+    # page-locked buffers in and out
+    n = 2 * chunk + 9
+    idx = synthetic.window_indices(n, w, V, seed=5)
+    pin_idx = _lib.pinned_empty(idx.shape, np.int32)
+    pin_idx[:] = idx
+    pin_bits = _lib.pinned_empty((n, h.words), np.uint64)
+    pin_bits[:] = 0
+    out = h.hash_windows(pin_idx, k, out_bits=pin_bits)
+    assert out is pin_bits and np.array_equal(pin_bits, h.hash_windows(idx, k))
+    # a smaller batch afterwards (the lanes' buffers are kept), and target ids beyond one chunk
+    assert np.array_equal(h.hash_windows(idx[:1000], k), pin_bits[:1000])
+    ids = synthetic.zipf_ids(chunk + 300, V, seed=8)
+    got = h.hash_targets(ids, k)
+    assert np.array_equal(got[-500:], ho.hash_targets_loop(W, ids[-500:], k))
+    # an index out of range in the last chunk is reported, the call returns, the hasher stays usable
+    bad = idx.copy()
+    bad[n - 3, 1] = 2 * V
+    with pytest.raises(_lib.FlyvecError) as e:
+        h.hash_windows(bad, k)
+    assert e.value.code == _lib.FV_ERR_DATA
+    assert np.array_equal(h.hash_windows(idx[:1000], k), pin_bits[:1000])
+    h.close()
