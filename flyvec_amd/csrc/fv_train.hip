@@ -877,6 +877,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   // counts of the block's elements that hold the row's largest / second largest weight (every path to the
   // elements passes a barrier)
   if (tid == 0) sh_hits[0] = sh_hits[1] = 0;
+  uint32_t hits1 = 0, hits2 = 0;  // the same in all lanes of a wave
   // The launch lasts as long as its few heaviest blocks: their waves go first wherever they share a
   // SIMD with the waves of light blocks.
   if (c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
@@ -1124,9 +1125,10 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
             slots[emitted + eb + u * T] = rec;
             if (DELTA) a.slot_n2[slot_first + emitted + eb + u * T] = n2e[u];
             a.Wt[pe[u]] = fv_sentinel(record0 + eb + u * T);
+            // counted per wave from lane masks: the counts stay in scalar registers
             const float aw = fabsf(wv[u]);
-            if (aw == top2.x) atomicAdd(&sh_hits[0], 1u);  // a few per step over the whole grid
-            else if (aw == top2.y) atomicAdd(&sh_hits[1], 1u);
+            hits1 += (uint32_t)__popcll(__ballot(aw == top2.x));
+            hits2 += (uint32_t)__popcll(__ballot(aw == top2.y && top2.y < top2.x));
             if (x_h != 0.0f)
               ds_max = fv_absmax_keep(ds_max, DELTA ? fv_sparse_ds2(x_h, wv[u], fe[u], ne[u], a.delta, n2e[u], le[u])
                                                     : fv_sparse_ds(x_h, wv[u], fe[u], ne[u], le[u]));
@@ -1136,7 +1138,11 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       fv_lds_barrier();
     } while (found > FV_SP_LIST_CAP);
   }
-  const float bm = fv_block_max_nonneg(ds_max, wave_max);  // behind its barriers every thread's hits are counted
+  if ((tid & 63u) == 0 && (hits1 | hits2)) {
+    atomicAdd(&sh_hits[0], hits1);
+    atomicAdd(&sh_hits[1], hits2);
+  }
+  const float bm = fv_block_max_nonneg(ds_max, wave_max);  // behind its barriers every wave's hits are counted
   if (tid == 0) {
     a.bmax_sparse[blockIdx.x] = bm;
     a.slot_count[blockIdx.x] = emitted;
