@@ -79,7 +79,9 @@ SIGNATURES = {
     "fv_trainer_get_second_winners": [_vp, _vp, _u32],
     "fv_trainer_run_epoch": [_vp, _u64, _u64],
     "fv_trainer_epoch_eps": [_vp, _u64, _u64, C.POINTER(_f32)],
+    "fv_trainer_set_stale_tail": [_vp, _u32],
     "fv_trainer_sync": [_vp],
+    "fv_trainer_get_giveups_recovered": [_vp, C.POINTER(_u64)],
     "fv_trainer_set_dense_launches": [_vp, _u32],
     "fv_trainer_get_dense_launches": [_vp, C.POINTER(_u32)],
     "fv_trainer_get_dense_path_counts": [_vp, C.POINTER(_u64), C.POINTER(_u64)],

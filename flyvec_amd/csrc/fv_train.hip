@@ -131,12 +131,15 @@ struct fv_trainer {
   uint32_t *path_count;  // device: launches that took max|ds| from them / that made the pass
   bool top2_valid, last_top2_known;
   unsigned sparse_base;  // index in bmax of the sparse launch's first block maximum
+  bool stale_tail;  // run_epoch trains a final partial minibatch with the previous one's rows behind its own
   bool separate_grouping;  // the grouping kernel always runs as a launch of its own (fv_trainer_set_grouping_launch)
   bool last_grouped_in_sparse;  // the form the last whole step took: a launch on its own repeats that form
   unsigned long long *arrive;
   uint32_t onepass_epoch;
   uint32_t onepass_spin_limit;
-  uint32_t *onepass_status;
+  uint32_t *onepass_status;  // pinned host word: 0, or the tag of the first launch that gave up
+  uint32_t step_tag;         // tag of the step being enqueued: run_epoch numbers its steps from 1, else 0
+  uint64_t giveups_recovered;  // epochs in which run_epoch took up again behind a launch that gave up
   float update_cut;  // largest fp32 <= 1e-10
 };
 
@@ -198,6 +201,7 @@ struct fv_gather_args {
   uint32_t n, K, ldk, w, V, tie_rule;
   uint32_t stride;   // entries per row of idx: w rounded up to 4, the ones past w hold -1
   uint32_t sampled;  // idx already holds this minibatch
+  uint32_t n_fresh;  // windows the sampler fills (not sampled): the rows from there on keep what idx holds
   uint32_t prune;    // in-window duplicate pruning while sampling
   float lmid, lbase; // weight of a window's centre position and of the others (WEIGHTED kernels)
   // the first merge_rows blocks of the launch merge the shares of the rows' two largest weights that the
@@ -257,8 +261,9 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
   for (int k = 0; k < FV_GATHER_WINDOWS; ++k) {
     const uint32_t r = g + k * per;
     idx[k] = -1;
+    const bool kept = a.sampled || r >= a.n_fresh;
     if (lane < (int)a.w && r < a.n) {
-      if (a.sampled) {
+      if (kept) {
         idx[k] = a.idx[(uint64_t)r * a.stride + lane];
       } else {
         const uint64_t s = a.pstart[a.first + r];
@@ -267,7 +272,7 @@ __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a)
         idx[k] = fv_column_index(tok, (uint32_t)lane, a.w, a.V);
       }
     }
-    if (!a.sampled && lane < (int)a.stride && r < a.n) a.idx[(uint64_t)r * a.stride + lane] = idx[k];
+    if (!kept && lane < (int)a.stride && r < a.n) a.idx[(uint64_t)r * a.stride + lane] = idx[k];
   }
 #pragma unroll
   for (int k = 0; k < FV_GATHER_WINDOWS; ++k) {
@@ -1180,9 +1185,10 @@ struct fv_dense_args {
   uint32_t total4, ldk4, ldk, V, K, w, n_bmax, dense_blocks;
   float eps, prec, update_cut;
   // single-launch form only
-  unsigned long long *arrive;
+  unsigned long long *arrive;  // one word per block, then the launch's decision word
   uint32_t *status;
   uint32_t epoch, spin_limit;
+  uint32_t step_tag;  // what a launch that gives up leaves in *status (not 0)
   float lmid, lbase;  // weight of a window's centre position (elements p >= V * ldk) and of the others
   // the minibatch sampled ahead (ahead_n = 0: none)
   const int32_t *corpus;
@@ -1429,6 +1435,22 @@ __device__ __forceinline__ void fv_sample_ahead(const fv_dense_args &a, bool sam
     }
 }
 
+// The one decision of a launch that makes the pass for max|ds|: whether all its blocks go on to the update,
+// and with which maximum. The word carries (launch number, value); whoever writes this launch's number
+// first -- block 0 with the maximum once every block has arrived, or any block that has run out of patience
+// with FV_ONEPASS_ABANDONED -- has decided for all, and everybody, the writer included, follows what the
+// word says. Returns the decision.
+__device__ __forceinline__ uint32_t fv_onepass_decide(unsigned long long *word, uint32_t epoch, uint32_t value) {
+  unsigned long long old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long mine = ((unsigned long long)epoch << 32) | value;
+  while ((uint32_t)(old >> 32) != epoch) {
+    if (__hip_atomic_compare_exchange_strong(word, &old, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT))
+      return value;
+  }
+  return (uint32_t)old;
+}
+
 static_assert(FV_MAX_HID <= 2 * FV_ONEPASS_THREADS, "two neurons per thread cover every row");
 static_assert(FV_NB_CLASSES == 4, "a neuron's block maxima and hit counts are read as one 16-byte word each");
 
@@ -1469,8 +1491,9 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
     hit4[j] = ((const uint4 *)a.row_hits)[h];
     smx[j] = ((const float4 *)(a.bmax + a.sparse_base))[h];
   }
-  // after one launch has given up, the launches already enqueued behind it do not wait at all
-  const uint32_t limit = a.scalars[1] != 0.0f ? 0u : a.spin_limit;
+  // after one launch has given up, the launches already enqueued behind it neither wait nor update
+  const bool dead = a.scalars[1] != 0.0f;
+  const uint32_t limit = dead ? 0u : a.spin_limit;
   float4 w[U];
   __builtin_amdgcn_sched_barrier(0);  // nothing that uses a small load moves up between the loads of W
 #pragma unroll
@@ -1538,7 +1561,8 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   if (fast) {
     const float nc = __uint_as_float(max(S, E));
     s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
-    if (blockIdx.x == 0 && tid == 0) {
+    ok = !dead;
+    if (blockIdx.x == 0 && tid == 0 && ok) {
       a.scalars[0] = nc;
       a.path_count[0] += 1;
     }
@@ -1566,31 +1590,42 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
       if (tid == 0)
         __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | __float_as_uint(bm),
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      uint32_t mx = 0;
-      bool done = false, abandoned = false;
-      for (uint32_t spin = 0; spin < limit && !done && !abandoned; ++spin) {
-        bool all = true, bad = false;
-        mx = 0;
-        for (uint32_t i = tid; i < gridDim.x; i += 64) {
-          const unsigned long long v = __hip_atomic_load(&a.arrive[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          all = all && (uint32_t)(v >> 32) == a.epoch;
-          bad = bad || ((uint32_t)(v >> 32) == a.epoch && (uint32_t)v == FV_ONEPASS_ABANDONED);
-          mx = max(mx, (uint32_t)v);  // non-negative floats order like their bit patterns
+      // Block 0 waits for every block's word and decides; the others wait for the decision. Both waits are
+      // bounded, and a block that gives up decides "abandoned" unless the decision has already been made.
+      unsigned long long *decision = a.arrive + gridDim.x;
+      uint32_t verdict = FV_ONEPASS_ABANDONED;
+      bool decided = false;
+      if (blockIdx.x == 0) {
+        uint32_t mx = 0;
+        bool done = false;
+        for (uint32_t spin = 0; spin < limit && !done; ++spin) {
+          bool all = true;
+          mx = 0;
+          for (uint32_t i = tid; i < gridDim.x; i += 64) {
+            const unsigned long long v = __hip_atomic_load(&a.arrive[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            all = all && (uint32_t)(v >> 32) == a.epoch;
+            mx = max(mx, (uint32_t)v);  // non-negative floats order like their bit patterns
+          }
+          done = __all(all);
+          if (!done) __builtin_amdgcn_s_sleep(2);
         }
-        abandoned = __any(bad);
-        done = !abandoned && __all(all);
-        if (!done && !abandoned) __builtin_amdgcn_s_sleep(2);
+        mx = fv_wave_max_u32(mx);
+        if (done) verdict = mx;
+      } else {
+        for (uint32_t spin = 0; spin < limit && !decided; ++spin) {
+          const unsigned long long v = __hip_atomic_load(decision, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          decided = (uint32_t)(v >> 32) == a.epoch;
+          if (decided) verdict = (uint32_t)v; else __builtin_amdgcn_s_sleep(2);
+        }
       }
-      mx = fv_wave_max_u32(mx);
       if (tid == 0) {
-        const float nc = __uint_as_float(mx);
+        if (!decided) verdict = fv_onepass_decide(decision, a.epoch, verdict);
+        const bool go = verdict != FV_ONEPASS_ABANDONED;
+        const float nc = __uint_as_float(verdict);
         sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
-        sh_ok = done;
-        if (!done) {
-          // blocks that arrive later must not update either
-          __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | FV_ONEPASS_ABANDONED,
-                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          *a.status = 1u;
+        sh_ok = go;
+        if (!go) {
+          if (!dead) *a.status = a.step_tag;  // the launches behind this one are dead and leave the word alone
           a.scalars[0] = __uint_as_float(0x7fc00000u);
           a.scalars[1] = 1.0f;
         } else if (blockIdx.x == 0) {
@@ -1796,16 +1831,30 @@ static void fv_trainer_free_corpus(fv_trainer *t) {
 // for the other half, so the form is only used while one trainer exists.
 static std::atomic<int> fv_trainers_alive{0};
 
-// Waits for the trainer's stream; reports a single-launch dense pass that gave up waiting for its
-// other blocks (the step it belonged to did not update the matrix).
+// After a single dense launch has given up: the trainer goes on with two launches per step, and the marks
+// the launch left (status word, "dead" flag for the launches behind it) are cleared. Returns the tag.
+static int fv_trainer_take_giveup(fv_trainer *t, uint32_t *out_tag) {
+  *out_tag = 0;
+  if (!t->onepass_status || !*(volatile uint32_t *)t->onepass_status) return FV_OK;
+  *out_tag = *(volatile uint32_t *)t->onepass_status;
+  *t->onepass_status = 0;
+  t->onepass = false;
+  t->top2_valid = false;
+  t->ahead_valid = false;
+  FV_HIP(hipMemsetAsync(t->scalars + 1, 0, sizeof(float), t->stream));
+  FV_HIP(hipStreamSynchronize(t->stream));
+  return FV_OK;
+}
+
+// Waits for the trainer's stream; reports a single dense launch that gave up waiting for its other blocks.
 static int fv_trainer_wait(fv_trainer *t) {
   FV_HIP(hipStreamSynchronize(t->stream));
-  if (t->onepass_status && *(volatile uint32_t *)t->onepass_status) {
-    *t->onepass_status = 0;
-    t->onepass = false;  // later steps take two launches
-    return fv_fail(FV_ERR_STATE, "a single-launch dense pass gave up waiting for its blocks (not resident together): "
-                                 "that step did not update the matrix; later steps use two launches");
-  }
+  uint32_t tag = 0;
+  FV_TRY(fv_trainer_take_giveup(t, &tag));
+  if (tag)
+    return fv_fail(FV_ERR_STATE, "a single dense launch gave up waiting for its blocks (not resident together): neither "
+                                 "that step nor the steps enqueued behind it have changed the matrix; later steps use "
+                                 "two launches");
   return FV_OK;
 }
 
@@ -1895,8 +1944,8 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMemsetAsync(t->xx, 0, (size_t)t->ldk * sizeof(float), t->stream));
   FV_HIP(hipMemsetAsync(t->scalars, 0, 16 * sizeof(float), t->stream));
   if (t->onepass_unroll) {
-    FV_HIP(hipMalloc((void **)&t->arrive, (size_t)t->onepass_blocks * sizeof(unsigned long long)));
-    FV_HIP(hipMemsetAsync(t->arrive, 0, (size_t)t->onepass_blocks * sizeof(unsigned long long), t->stream));
+    FV_HIP(hipMalloc((void **)&t->arrive, ((size_t)t->onepass_blocks + 1) * sizeof(unsigned long long)));
+    FV_HIP(hipMemsetAsync(t->arrive, 0, ((size_t)t->onepass_blocks + 1) * sizeof(unsigned long long), t->stream));
     FV_HIP(hipHostMalloc((void **)&t->onepass_status, sizeof(uint32_t), hipHostMallocDefault));
     *t->onepass_status = 0;
   }
@@ -2201,8 +2250,10 @@ static int fv_trainer_alloc_delta(fv_trainer *t) {
   return FV_OK;
 }
 
+// n_fresh < n: only the first n_fresh windows are sampled (from `first` on), the rows behind them are what
+// the index buffer of the previous step holds.
 static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps, float delta, hipEvent_t *ev,
-                           unsigned which = 0x3f, bool repeated = false) {
+                           unsigned which = 0x3f, bool repeated = false, uint32_t n_fresh = 0xffffffffu) {
   const bool anti = delta != 0.0f;  // the second neuron of every window takes part (flyvec/src/cuda_funcs.cu:726-734)
   if (anti) FV_TRY(fv_trainer_alloc_delta(t));
   const bool whole = which == 0x3f;
@@ -2233,6 +2284,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   g.sc2 = t->sc2;
   g.first = first;
   g.n = n;
+  g.n_fresh = n_fresh < n ? n_fresh : n;
   g.K = t->K;
   g.ldk = t->ldk;
   g.w = t->w;
@@ -2263,7 +2315,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   // a whole step whose windows the previous one has sampled ahead takes that buffer
   g.sampled = 0;
   if (whole) {
-    if (t->ahead_valid && t->ahead_first == first && t->ahead_n == n) {
+    if (t->ahead_valid && t->ahead_first == first && t->ahead_n == n && n_fresh >= n) {
       std::swap(t->idx, t->idx_ahead);
       g.idx = t->idx;
       g.sampled = 1;
@@ -2374,7 +2426,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.w = t->w;
   d.arrive = nullptr;
   d.status = nullptr;
-  d.epoch = d.spin_limit = 0;
+  d.epoch = d.spin_limit = d.step_tag = 0;
   d.lmid = t->cfg.lmid;
   d.lbase = t->cfg.lbase;
   d.corpus = t->corpus;
@@ -2415,6 +2467,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
       d.status = t->onepass_status;
       d.epoch = t->onepass_epoch;
       d.spin_limit = t->onepass_spin_limit;
+      d.step_tag = t->step_tag ? t->step_tag : 0xffffffffu;
       // the windows that follow this step's, a full batch or what is left of the order
       const uint64_t next_first = first + n;
       if (whole && next_first < t->n_windows && !t->cfg.prune_duplicates) {  // the ahead sampler does not prune
@@ -2514,11 +2567,47 @@ extern "C" int fv_trainer_run_epoch(fv_trainer *t, uint64_t epoch_id, uint64_t n
   float eps = 0.0f, delta = 0.0f;
   FV_TRY(fv_trainer_epoch_eps(t, epoch_id, n_epochs, &eps));
   FV_TRY(fv_trainer_epoch_delta(t, epoch_id, n_epochs, &delta));
-  for (uint64_t k = 0; k < t->n_windows; k += t->B) {
-    const uint64_t n = t->n_windows - k < t->B ? t->n_windows - k : t->B;
-    FV_TRY(fv_enqueue_step(t, k, (uint32_t)n, eps, delta, nullptr));
+  // The reference's loop never skips a minibatch (flyvec/src/cuda_funcs.cu:1662-1812). A single dense launch
+  // that gives up leaves the matrix as the step before it left it, and so do all launches behind it; the loop
+  // is then taken up again at that step, with two launches per step.
+  uint64_t k_first = 0;
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    int rc = FV_OK;
+    for (uint64_t k = k_first; k < t->n_windows && rc == FV_OK; k += t->B) {
+      const uint64_t n = t->n_windows - k < t->B ? t->n_windows - k : t->B;
+      t->step_tag = (uint32_t)(k / t->B) + 1u;
+      if (n < t->B && k > 0 && t->stale_tail)
+        // flyvec/src/cuda_funcs.cu:1679 against :1700-1732: only the sampler sees the remainder, the other
+        // kernels run on all Num rows, those behind the remainder being the previous minibatch's
+        rc = fv_enqueue_step(t, k, t->B, eps, delta, nullptr, 0x3f, false, (uint32_t)n);
+      else
+        rc = fv_enqueue_step(t, k, (uint32_t)n, eps, delta, nullptr);
+    }
+    t->step_tag = 0;
+    FV_TRY(rc);
+    FV_HIP(hipStreamSynchronize(t->stream));
+    uint32_t tag = 0;
+    FV_TRY(fv_trainer_take_giveup(t, &tag));
+    if (!tag) return FV_OK;
+    FV_REQUIRE(attempt == 0 && tag != 0xffffffffu, FV_ERR_STATE,
+               "a dense launch gave up although the epoch was already being redone with two launches per step");
+    k_first = (uint64_t)(tag - 1u) * t->B;
+    t->giveups_recovered++;
   }
-  return fv_trainer_wait(t);
+  return FV_OK;
+}
+
+extern "C" int fv_trainer_get_giveups_recovered(fv_trainer *t, uint64_t *out_count) {
+  FV_REQUIRE(t && out_count, FV_ERR_INVALID, "null argument");
+  *out_count = t->giveups_recovered;
+  return FV_OK;
+}
+
+extern "C" int fv_trainer_set_stale_tail(fv_trainer *t, uint32_t on) {
+  FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
+  FV_REQUIRE(on <= 1, FV_ERR_INVALID, "on must be 0 or 1");
+  t->stale_tail = on != 0;
+  return FV_OK;
 }
 
 extern "C" int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches) {

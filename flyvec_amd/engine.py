@@ -135,6 +135,12 @@ class Trainer:
     def run_epoch(self, epoch_id, n_epochs):
         check(self.lib.fv_trainer_run_epoch(self.handle, int(epoch_id), int(n_epochs)))
 
+    def set_stale_tail(self, on):
+        """True: run_epoch trains a final partial minibatch with the previous minibatch's rows behind its own,
+        as the reference does (flyvec/src/cuda_funcs.cu:1679 against :1700-1732); False (default): the
+        remainder only."""
+        check(self.lib.fv_trainer_set_stale_tail(self.handle, 1 if on else 0))
+
     def epoch_eps(self, epoch_id, n_epochs):
         out = C.c_float(0)
         check(self.lib.fv_trainer_epoch_eps(self.handle, int(epoch_id), int(n_epochs), C.byref(out)))
@@ -142,6 +148,13 @@ class Trainer:
 
     def sync(self):
         check(self.lib.fv_trainer_sync(self.handle))
+
+    @property
+    def giveups_recovered(self):
+        """Epochs in which run_epoch took up again behind a single dense launch that gave up."""
+        out = C.c_uint64(0)
+        check(self.lib.fv_trainer_get_giveups_recovered(self.handle, C.byref(out)))
+        return out.value
 
     def set_dense_launches(self, launches):
         """1: both passes over the matrix in one launch (it must fit the device's registers),

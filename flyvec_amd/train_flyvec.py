@@ -45,6 +45,7 @@ def build_parser():
     p.add_argument("--Lmid", default=1.0, type=float, help="Weight of a window's centre position (the reference holds 1.0 and has no flag for it; flyvec/src/cuda_funcs.cu:266-327, 675-697)")
     p.add_argument("--Lbase", default=1.0, type=float, help="Weight of the other window positions (likewise)")
     p.add_argument("--prune_duplicates", action="store_true", help="Drop a token that an earlier position of its window holds (the sampler variant the reference has switched off, flyvec/src/cuda_funcs.cu:938-979)")
+    p.add_argument("--stale_last_batch", action="store_true", help="Train an epoch's final partial minibatch with the previous minibatch's rows behind its own, as the reference's launch sizes do (flyvec/src/cuda_funcs.cu:1679 against :1700-1732); default: the remainder only")
     p.add_argument("--mu", default=0.0, type=float, help="Mean of the random normal initialisation")
     p.add_argument("--sigma", default=0.02, type=float, help="Stdev of the random normal initialisation")
     p.add_argument("--Nep", default=15, type=int, help="Maximum number of epochs, fewer if starting from a checkpoint")
@@ -81,6 +82,7 @@ def train(args, log=print):
                       initial_learning_rate=args.initial_learning_rate, delta=args.delta, prec=args.prec,
                       tie_rule=1 if args.tie_rule == "reference" else 0, lmid=args.Lmid, lbase=args.Lbase,
                       prune_duplicates=args.prune_duplicates)
+    trainer.set_stale_tail(args.stale_last_batch)
     log("Copying input...")
     trainer.set_corpus(tokens, offsets)
     log(f"Number of phrases:  {trainer.num_windows}")

@@ -174,15 +174,25 @@ int fv_trainer_epoch_delta(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs, 
 int fv_trainer_get_second_winners(fv_trainer *t, int32_t *out_seconds, uint32_t capacity);
 
 /* flyvec/src/cuda_funcs.cu:1220 launch_epoch_INPUT_AS_INT: eps = lr0 * (1 - epoch/n_epochs),
- * then every minibatch of the current permutation (the last one takes the remainder only).
+ * then every minibatch of the current permutation (the last one takes the remainder only, unless
+ * fv_trainer_set_stale_tail says otherwise).
  * Returns after the device has finished. */
 int fv_trainer_run_epoch(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs);
+/* The reference's treatment of a final partial minibatch: flyvec/src/cuda_funcs.cu:1679 launches only the
+ * sampler with the remainder, every other kernel with the full minibatch (:1700-1732), so the rows behind
+ * the remainder still hold the previous minibatch's windows and are trained on once more. on = 1 makes
+ * fv_trainer_run_epoch do the same (when a full minibatch precedes the partial one in the epoch);
+ * 0, the default, trains the remainder only. */
+int fv_trainer_set_stale_tail(fv_trainer *t, uint32_t on);
 /* eps of flyvec/src/cuda_funcs.cu:1229 for this trainer's learning rate. */
 int fv_trainer_epoch_eps(fv_trainer *t, uint64_t epoch_id, uint64_t n_epochs, float *out_eps);
 
-/* Waits for the trainer's stream. FV_ERR_STATE if a single-launch dense pass (below) gave up
- * waiting for its other blocks: the step it belonged to did not update the matrix. */
+/* Waits for the trainer's stream. FV_ERR_STATE if a single dense launch (below) gave up waiting for
+ * its other blocks: neither that step nor the steps enqueued behind it have changed the matrix.
+ * fv_trainer_run_epoch does not return that error: it takes the epoch up again at the step that gave up,
+ * with two launches per step, and counts the event (fv_trainer_get_giveups_recovered). */
 int fv_trainer_sync(fv_trainer *t);
+int fv_trainer_get_giveups_recovered(fv_trainer *t, uint64_t *out_count);
 
 /* The two passes over the matrix of a step (max|ds|, flyvec/src/cu_special_reduction.cu:241, and
  * the update, flyvec/src/cuda_funcs.cu:1787-1806) run as ONE launch when the matrix fits the registers of

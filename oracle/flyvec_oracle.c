@@ -23,6 +23,9 @@
  *       centre and context elect different winners).
  *   fvo_prune_windows : the reference's own prune_input_data (oracle/_ref).
  *   fvo_inflate_prune : a set-based first-occurrence formulation in Python.
+ *   fvo_train_steps_tail (the reference's re-use of the previous minibatch's
+ *       rows on a final partial minibatch) : the single step on an index
+ *       matrix assembled by hand from two inflate calls.
  *
  * Order-dependent fp32 sums (the reference uses atomics whose order is not
  * defined) are given a fixed order here.  The sparse term of ds: increasing
@@ -462,16 +465,30 @@ float fvo_epoch_delta(float delta, uint64_t epoch, uint64_t n_epochs) {
  * (the reference re-uses stale rows there; this restatement processes the
  * remainder only).  winners (if given) receives the winners of every step
  * back to back.  Returns the number of windows processed.
+ *
+ * stale_tail != 0 mirrors what the reference does on a final partial
+ * minibatch: only the sampler is launched with the remainder
+ * (flyvec/src/cuda_funcs.cu:1679 passes input_end - input_start), every other
+ * kernel with the full Num (:1700-1732), so the rows from the remainder on
+ * still hold the previous minibatch's windows and are trained on once more.
+ * The index matrix below is kept from step to step exactly like the
+ * reference's input_sparse_indx; a partial step that no full one precedes in
+ * this call takes its remainder only (the reference would read rows nobody
+ * has written).  The winners of re-used rows are not returned.
+ * Pinned in tests/test_oracle_train.py by building that index matrix by hand
+ * and running the (separately pinned) single step on it.
  */
-uint64_t fvo_train_steps_weighted(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
-                                  const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
-                                  uint64_t n_steps, int w, const float *invf, float eps, float prec,
-                                  int tie_rule, float delta, float lmid, float lbase, int prune,
-                                  int32_t *winners) {
+uint64_t fvo_train_steps_tail(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
+                              const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
+                              uint64_t n_steps, int w, const float *invf, float eps, float prec,
+                              int tie_rule, float delta, float lmid, float lbase, int prune, int stale_tail,
+                              int32_t *winners) {
   const uint64_t N = 2 * V;
   float *ds = (float *)malloc(sizeof(float) * (size_t)K * N);
   int32_t *idx = (int32_t *)malloc(sizeof(int32_t) * B * (uint64_t)w);
+  int32_t *win_all = (int32_t *)malloc(sizeof(int32_t) * B);
   uint64_t done = 0;
+  int full_before = 0;
   for (uint64_t j = 0; j < n_steps; ++j) {
     uint64_t k0 = first + j * B;
     if (k0 >= n_windows) break;
@@ -480,13 +497,26 @@ uint64_t fvo_train_steps_weighted(float *W, int K, uint64_t V, const int32_t *co
       fvo_inflate_prune(corpus, starts, perm, k0, n, w, V, idx);
     else
       fvo_inflate(corpus, starts, perm, k0, n, w, V, idx);
-    fvo_train_step_weighted(W, K, N, V, idx, n, w, invf, eps, prec, tie_rule, delta, lmid, lbase, ds,
-                            winners ? winners + done : NULL, NULL, NULL, NULL, NULL, NULL);
+    const uint64_t rows = (stale_tail && n < B && full_before) ? B : n;
+    fvo_train_step_weighted(W, K, N, V, idx, rows, w, invf, eps, prec, tie_rule, delta, lmid, lbase, ds, win_all,
+                            NULL, NULL, NULL, NULL, NULL);
+    if (winners) memcpy(winners + done, win_all, sizeof(int32_t) * n);
     done += n;
+    if (n == B) full_before = 1;
   }
   free(ds);
   free(idx);
+  free(win_all);
   return done;
+}
+
+uint64_t fvo_train_steps_weighted(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,
+                                  const uint64_t *perm, uint64_t n_windows, uint64_t first, uint64_t B,
+                                  uint64_t n_steps, int w, const float *invf, float eps, float prec,
+                                  int tie_rule, float delta, float lmid, float lbase, int prune,
+                                  int32_t *winners) {
+  return fvo_train_steps_tail(W, K, V, corpus, starts, perm, n_windows, first, B, n_steps, w, invf, eps, prec,
+                              tie_rule, delta, lmid, lbase, prune, 0, winners);
 }
 
 uint64_t fvo_train_steps_delta(float *W, int K, uint64_t V, const int32_t *corpus, const uint64_t *starts,

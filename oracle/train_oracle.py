@@ -78,6 +78,11 @@ def lib():
                                                C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_void_p,
                                                C.c_float, C.c_float, C.c_int, C.c_float, C.c_float, C.c_float,
                                                C.c_int, C.c_void_p]
+        L.fvo_train_steps_tail.restype = C.c_uint64
+        L.fvo_train_steps_tail.argtypes = [C.c_void_p, C.c_int, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                           C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_void_p,
+                                           C.c_float, C.c_float, C.c_int, C.c_float, C.c_float, C.c_float,
+                                           C.c_int, C.c_int, C.c_void_p]
         L.fvo_inflate_prune.restype = None
         L.fvo_inflate_prune.argtypes = L.fvo_inflate.argtypes
         L.fvo_prune_windows.restype = None
@@ -259,8 +264,9 @@ def train_step(W, idx, invf, eps, prec=1e-30, tie_rule=0, delta=0.0, lmid=1.0, l
 
 
 def train_steps(W, corpus, starts, perm, first, B, n_steps, w, invf, eps, prec=1e-30, tie_rule=0, delta=0.0,
-                lmid=1.0, lbase=1.0, prune=False):
-    """In-place n_steps minibatches; returns the winners of all processed windows."""
+                lmid=1.0, lbase=1.0, prune=False, stale_tail=False):
+    """In-place n_steps minibatches; returns the winners of all processed windows. stale_tail: a final partial
+    minibatch is trained with the previous minibatch's rows behind its own, as the reference does."""
     assert W.dtype == np.float32 and W.flags.c_contiguous
     corpus = np.ascontiguousarray(corpus, dtype=np.int32)
     starts = np.ascontiguousarray(starts, dtype=np.uint64)
@@ -271,7 +277,7 @@ def train_steps(W, corpus, starts, perm, first, B, n_steps, w, invf, eps, prec=1
     nwin = len(perm)
     cap = max(0, min(n_steps * B, nwin - first))
     win = np.empty(cap, dtype=np.int32)
-    done = lib().fvo_train_steps_weighted(_p(W), K, V, _p(corpus), _p(starts), _p(perm), nwin, first, B, n_steps,
-                                          w, _p(invf), eps, prec, tie_rule, delta, lmid, lbase, int(bool(prune)),
-                                          _p(win))
+    done = lib().fvo_train_steps_tail(_p(W), K, V, _p(corpus), _p(starts), _p(perm), nwin, first, B, n_steps,
+                                      w, _p(invf), eps, prec, tie_rule, delta, lmid, lbase, int(bool(prune)),
+                                      int(bool(stale_tail)), _p(win))
     return win[:done]

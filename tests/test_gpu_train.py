@@ -869,3 +869,72 @@ def test_dense_launch_knows_the_maximum_from_the_rows_largest_weights(gpu, oracl
     assert all(known + made == 8 and made >= 1 for known, made in counts.values())   # the first step makes the pass
     assert counts["plain"][0] >= 5
     assert counts["planted"][1] >= 4
+
+
+@pytest.mark.parametrize("launches,prune", [(1, False), (2, False), (1, True)])
+def test_stale_tail_of_the_last_minibatch(gpu, oracle_lib, launches, prune):
+    """The reference trains a final partial minibatch on all Num rows, the ones behind the remainder being the
+    previous minibatch's (flyvec/src/cuda_funcs.cu:1679 against :1700-1732). Switched on, run_epoch does the same,
+    over two epochs with a reshuffled order in between, bit for bit with the checker's mode; switched off it
+    trains the remainder only."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    V, K, w, B = 400, 70, 7, 900
+    tokens, offsets = small_corpus(9000, V if not prune else 30, seed=6)
+    tokens[-1] = V - 1
+    W0 = synthetic.synapses(K, V, seed=4)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    assert len(starts) % B not in (0,) and len(starts) > 3 * B
+    for stale in (True, False):
+        t = Trainer(V, K, w, B, initial_learning_rate=1e-3, prune_duplicates=prune)
+        t.set_dense_launches(launches)
+        t.set_stale_tail(stale)
+        t.set_corpus(tokens, offsets)
+        t.set_weights(W0)
+        Wo = W0.copy()
+        for ep in range(2):
+            t.shuffle(ep)
+            perm = t.get_permutation()
+            t.run_epoch(ep, 15)
+            to.train_steps(Wo, tokens, starts, perm, 0, B, len(starts) // B + 1, w, invf, to.epoch_eps(1e-3, ep, 15),
+                           prune=prune, stale_tail=stale)
+        assert np.array_equal(t.get_weights().view(np.uint32), Wo.view(np.uint32)), stale
+        t.close()
+
+
+@pytest.mark.parametrize("planted", [False, True])
+def test_run_epoch_takes_up_again_behind_a_launch_that_gave_up(gpu, oracle_lib, planted):
+    """The reference's minibatch loop never skips a step (flyvec/src/cuda_funcs.cu:1662-1812). With the wait of
+    the single dense launch forced to zero rounds (every kernel still runs to its end) the first launch that has
+    to make the pass for max|ds| gives up -- the epoch's first step on a fresh matrix, or, with the rows' largest
+    weights planted on the most frequent tokens, the first step whose deciding row has them among its sparse
+    elements although they are known from the epoch before -- and so do the launches behind it; run_epoch redoes the epoch from that step with two launches per step and the matrix
+    equals the checker's."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    V, K, w, B = 800, 96, 9, 2000
+    tokens, offsets = small_corpus(80000, V, seed=2)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    W0 = synthetic.synapses(K, V, seed=9)
+    if planted:
+        hot = np.argsort(-np.bincount(tokens[tokens >= 0], minlength=V))[:3]
+        W0[:, hot] = np.float32(7.0)
+    t = Trainer(V, K, w, B, initial_learning_rate=1e-3)
+    t.set_dense_launches(1)
+    t.set_corpus(tokens, offsets)
+    t.set_weights(W0)
+    Wo = W0.copy()
+    n_steps = len(starts) // B + 1
+    for ep in range(2):
+        t.shuffle(ep)
+        perm = t.get_permutation()
+        if ep == 1 or not planted:
+            t.set_dense_launches(1)
+            t._set_wait_limit(0)
+        t.run_epoch(ep, 15)
+        to.train_steps(Wo, tokens, starts, perm, 0, B, n_steps, w, invf, to.epoch_eps(1e-3, ep, 15))
+        assert np.array_equal(t.get_weights().view(np.uint32), Wo.view(np.uint32)), ep
+    assert t.giveups_recovered == (1 if planted else 2)
+    assert t.dense_launches == 2
+    t.sync()                   # nothing left to report
+    t.close()

@@ -51,11 +51,25 @@ def test_synthetic_corpus_contract():
 def test_byte_model_matches_the_baseline_figures():
     sys.path.insert(0, ROOT)
     import bench
-    total, per = bench.train_bytes(400, 40000, 11, 10000)
-    assert total == 369_760_000 and sum(per.values()) >= total - 200_000
-    total5, _ = bench.train_bytes(1000, 100000, 15, 50000)
-    assert total5 == 4_212_000_000
+    assert bench.step_byte_model(400, 40000, 11, 10000) == 369_760_000
+    assert bench.step_byte_model(1000, 100000, 15, 50000) == 4_212_000_000
     assert bench.hash_bytes_per_window(400, 11) == 17_700
+    per = bench.kernel_bytes(400, 40000, 11, 10000)
+    # the kernels of the step as six launches move the model's bytes; the single dense launch moves the matrix once each way
+    six = sum(per[k] for k in ("gather_winner", "group_xx", "sparse_owners", "absmax_ds", "update", "slot_update"))
+    assert 369_760_000 - 200_000 <= six <= 369_760_000 + 200_000
+    assert per["dense_update"] == 8 * 400 * 40000 + 8 * 10000 * 11
+
+
+def test_bench_reads_counters_from_the_profile_summaries():
+    sys.path.insert(0, ROOT)
+    import bench
+    for which in ("step", "large"):
+        c = bench.profile_counters(which)
+        assert {"gather_winner", "sparse_owners"} <= set(c), which
+        assert bench.traffic_bytes(c, "gather_winner") > 0
+        assert c["gather_winner"]["valu_insts"] > 0
+    assert bench.traffic_bytes({}, "gather_winner") is None
 
 
 def test_bench_refuses_more_than_one_gpu():

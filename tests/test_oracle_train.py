@@ -605,3 +605,43 @@ def test_inflate_prune_keeps_first_occurrences_and_the_centre():
     corpus2 = np.arange(50, dtype=np.int32) % 40
     st2 = np.arange(0, 30, dtype=np.uint64)
     assert np.array_equal(to.inflate_prune(corpus2, st2, st2, 0, 30, w, 40), to.inflate(corpus2, st2, st2, 0, 30, w, 40))
+
+
+@pytest.mark.parametrize("prune", [False, True])
+def test_stale_tail_reuses_the_previous_minibatch_rows(prune):
+    """flyvec/src/cuda_funcs.cu:1679 samples only the remainder of a final partial minibatch while :1700-1732
+    run on all Num rows: the rows behind the remainder are the previous minibatch's. The multi-step driver's
+    stale_tail mode must equal the single step run on that index matrix assembled by hand; without a full
+    minibatch before it, and with the mode off, the remainder alone is trained."""
+    from flyvec_amd import synthetic
+    V, K, w, B = 60, 9, 5, 64
+    tokens, offsets = synthetic.corpus(4000, V if not prune else 12, mean_chunk=14)
+    tokens[-1] = min(V, tokens.max() + 1) - 1
+    starts = to.window_starts(offsets, w)
+    invf = to.inverse_frequency(tokens, V)
+    perm = np.random.default_rng(2).permutation(len(starts)).astype(np.uint64)
+    n_win = 2 * B + 23                                   # two full minibatches and a remainder of 23
+    perm = perm[:n_win].copy()
+    W0 = synthetic.synapses(K, V, seed=3, sigma=0.3)
+    inflate = to.inflate_prune if prune else to.inflate
+    # by hand: two full steps, then the last on [23 new rows ; rows 23.. of the second minibatch]
+    Wh = W0.copy()
+    for j in range(2):
+        to.train_step(Wh, inflate(tokens, starts, perm, j * B, B, w, V), invf, 1e-2)
+    plain = Wh.copy()
+    idx = inflate(tokens, starts, perm, B, B, w, V).copy()
+    idx[:23] = inflate(tokens, starts, perm, 2 * B, 23, w, V)
+    ref = to.train_step(Wh, idx, invf, 1e-2)
+    to.train_step(plain, idx[:23], invf, 1e-2)
+    Ws = W0.copy()
+    win = to.train_steps(Ws, tokens, starts, perm, 0, B, 3, w, invf, 1e-2, prune=prune, stale_tail=True)
+    assert np.array_equal(Ws.view(np.uint32), Wh.view(np.uint32)) and not np.array_equal(Ws, plain)
+    assert len(win) == n_win and np.array_equal(win[2 * B:], ref["winners"][:23])
+    Wp = W0.copy()
+    to.train_steps(Wp, tokens, starts, perm, 0, B, 3, w, invf, 1e-2, prune=prune)
+    assert np.array_equal(Wp.view(np.uint32), plain.view(np.uint32))
+    # no full minibatch before the partial one: the remainder alone, in both modes
+    a, b = W0.copy(), W0.copy()
+    to.train_steps(a, tokens, starts, perm[:23].copy(), 0, B, 1, w, invf, 1e-2, prune=prune, stale_tail=True)
+    to.train_step(b, inflate(tokens, starts, perm, 0, 23, w, V), invf, 1e-2)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
