@@ -130,6 +130,8 @@ struct fv_trainer {
   uint32_t *row_hits;
   uint32_t *path_count;  // device: launches that took max|ds| from them / that made the pass
   bool top2_valid, last_top2_known;
+  uint32_t top2_n_part;  // shares per row that the last dense launches left (their number of blocks)
+  unsigned update_threads;  // 256, or 512 when a row has more than 256 groups of four neurons
   unsigned sparse_base;  // index in bmax of the sparse launch's first block maximum
   bool stale_tail;  // run_epoch trains a final partial minibatch with the previous one's rows behind its own
   bool separate_grouping;  // the grouping kernel always runs as a launch of its own (fv_trainer_set_grouping_launch)
@@ -157,25 +159,29 @@ __device__ __forceinline__ void fv_top2_merge(float &m1, float &m2, float b1, fl
   m2 = fmaxf(lo, fmaxf(m2, b2));
 }
 
-// The shares of every row's two largest weights that the blocks of the last single dense launch left,
-// merged: row_top2[h] for the step that begins. One block per neuron, run as the first blocks of the
-// winner kernel's launch.
+// The shares of every row's two largest weights that the blocks of the last dense launches left
+// (top2_part[block][neuron], a block's pairs side by side), merged: row_top2[h] for the step that begins.
+// One 256-thread block per 32 neurons, run as the first blocks of the winner kernel's launch: eight threads
+// per neuron share the blocks among them, eight loads in flight each.
+#define FV_MERGE_NEURONS 32
 __device__ __forceinline__ void fv_merge_row_top2(const float2 *__restrict__ part, uint32_t part_stride, uint32_t n_part,
-                                                  float2 *__restrict__ row_top2, uint32_t h) {
-  __shared__ float2 wave_pair[4];
+                                                  uint32_t K, float2 *__restrict__ row_top2, uint32_t group) {
+  __shared__ float2 sh_pair[8][FV_MERGE_NEURONS];
+  const uint32_t hh = threadIdx.x & (FV_MERGE_NEURONS - 1), bl = threadIdx.x / FV_MERGE_NEURONS;
+  const uint32_t h = min(group * FV_MERGE_NEURONS + hh, K - 1);  // past K: the last neuron once more, not stored
   float m1 = 0.0f, m2 = 0.0f;
-  for (uint32_t j = threadIdx.x; j < n_part; j += 256) {
-    const float2 b = part[(uint64_t)h * part_stride + j];
-    fv_top2_merge(m1, m2, b.x, b.y);
+  for (uint32_t b0 = bl; b0 < n_part; b0 += 64) {
+    float2 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = part[(uint64_t)min(b0 + 8u * u, n_part - 1) * part_stride + h];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (b0 + 8u * u < n_part) fv_top2_merge(m1, m2, v[u].x, v[u].y);
   }
-  for (int d = 32; d >= 1; d >>= 1) {  // the partner's pair covers other shares: no value is counted twice
-    const float b1 = __shfl_xor(m1, d, 64), b2 = __shfl_xor(m2, d, 64);
-    fv_top2_merge(m1, m2, b1, b2);
-  }
-  if ((threadIdx.x & 63) == 0) wave_pair[threadIdx.x >> 6] = make_float2(m1, m2);
+  sh_pair[bl][hh] = make_float2(m1, m2);
   __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int i = 1; i < 4; ++i) fv_top2_merge(m1, m2, wave_pair[i].x, wave_pair[i].y);
+  if (bl == 0 && group * FV_MERGE_NEURONS + hh < K) {
+    for (int i = 1; i < 8; ++i) fv_top2_merge(m1, m2, sh_pair[i][hh].x, sh_pair[i][hh].y);
     row_top2[h] = make_float2(m1, m2);
   }
 }
@@ -205,10 +211,10 @@ struct fv_gather_args {
   uint32_t prune;    // in-window duplicate pruning while sampling
   float lmid, lbase; // weight of a window's centre position and of the others (WEIGHTED kernels)
   // the first merge_rows blocks of the launch merge the shares of the rows' two largest weights that the
-  // last single dense launch left (fv_merge_row_top2); 0: none
+  // last dense launches left (fv_merge_row_top2: a block per 32 neurons); 0: none
   uint32_t merge_rows;
   const float2 *top2_part;
-  uint32_t part_stride, n_part;
+  uint32_t part_stride, n_part;  // pairs per share (ldk), shares
   float2 *row_top2;
 };
 
@@ -247,7 +253,7 @@ __device__ __forceinline__ int32_t fv_column_index(int32_t tok, uint32_t c, uint
 template <int NV, bool DELTA, bool WEIGHTED>
 __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a) {
   if (blockIdx.x < a.merge_rows) {
-    fv_merge_row_top2(a.top2_part, a.part_stride, a.n_part, a.row_top2, blockIdx.x);
+    fv_merge_row_top2(a.top2_part, a.part_stride, a.n_part, a.K, a.row_top2, blockIdx.x);
     return;
   }
   const int lane = threadIdx.x & 63;
@@ -1208,8 +1214,8 @@ struct fv_dense_args {
   const float2 *row_top2;
   const uint32_t *row_hits;
   uint32_t top2_known;
-  float2 *top2_part;     // out: the same of the matrix this launch leaves, over each block's share: [neuron][block]
-  uint32_t part_stride;  // blocks of a row of top2_part
+  float2 *top2_part;     // out: the same of the matrix this launch leaves, over each block's share: [block][ldk]
+  uint32_t part_base;    // separate launches: the update launch's blocks come first, then the slot launch's four
   uint32_t *path_count;  // [0] launches that knew max|ds| when they started, [1] launches that made the pass for it
 };
 
@@ -1268,11 +1274,66 @@ __device__ __forceinline__ void fv_dense_load(const fv_dense_args &a, uint32_t p
   for (int u = 0; u < U; ++u) w[u] = a.Wt4[p4 + u * stride < a.total4 ? p4 + u * stride : inside];
 }
 
+// |w| for the bookkeeping of a row's largest weights; a NaN (a sentinel) counts as 0
+__device__ __forceinline__ float fv_abs_or_zero(float w) { return w == w ? fabsf(w) : 0.0f; }
+
+// What one row adds to what is known of max|ds| before the matrix is seen (all three as bit patterns of
+// non-negative floats): S, the largest |ds| of a sparse element; E, the largest, over the rows whose largest
+// dense weight is known, of fl(|xx| * that weight); F, the same over the other rows with an upper bound of
+// that weight. x is the row's xx, top2 its two largest |W| (v1 >= v2), hit4 the counts of the row's sparse
+// elements that hold them, one word per block of the sparse launch, smx those blocks' largest |ds|.
+__device__ __forceinline__ void fv_row_candidate(float x, float2 top2, uint4 hit4, float4 smx, uint32_t &S, uint32_t &E,
+                                                 uint32_t &F) {
+  const uint32_t n1 = (hit4.x & 3u) + (hit4.y & 3u) + (hit4.z & 3u) + (hit4.w & 3u);
+  const uint32_t n2 = ((hit4.x >> 2) & 3u) + ((hit4.y >> 2) & 3u) + ((hit4.z >> 2) & 3u) + ((hit4.w >> 2) & 3u);
+  const float v1 = top2.x, v2 = top2.y;
+  // v1 == v2: two elements hold the largest value, one of them is dense unless two sparse ones hold it.
+  // v1 > v2: one element holds v1; if it is sparse, v2 bounds the rest, and is reached unless a
+  // sparse element holds it.
+  const bool first = v1 == v2 ? n1 <= 1 : n1 == 0;
+  const bool exact = first || (v1 != v2 && n2 == 0);
+  const uint32_t cand = __float_as_uint(__fmul_rn(fabsf(x), first ? v1 : v2));
+  if (exact) E = max(E, cand); else F = max(F, cand);
+  S = max(S, __float_as_uint(fmaxf(fmaxf(smx.x, smx.y), fmaxf(smx.z, smx.w))));
+}
+
+// Before the separate dense launches: one block looks at what is known of max|ds| (fv_row_candidate) and
+// leaves scalars[2] != 0 and max|ds| in scalars[3] when that settles it; the launch for the maximum then
+// ends at once and the update takes the figure from there.
+__global__ __launch_bounds__(1024) void fv_decide_kernel(fv_dense_args a) {
+  __shared__ uint32_t red3[16][3];
+  const uint32_t tid = threadIdx.x;
+  uint32_t S = 0, E = 0, F = 0;
+  for (uint32_t h = tid; h < a.K; h += 1024)
+    fv_row_candidate(a.xx[h], a.row_top2[h], ((const uint4 *)a.row_hits)[h],
+                     ((const float4 *)(a.bmax + a.sparse_base))[h], S, E, F);
+  const uint32_t ws = fv_wave_max_u32(S), we = fv_wave_max_u32(E), wf = fv_wave_max_u32(F);
+  if ((tid & 63) == 0) {
+    red3[tid >> 6][0] = ws;
+    red3[tid >> 6][1] = we;
+    red3[tid >> 6][2] = wf;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    S = E = F = 0;
+    for (int i = 0; i < 16; ++i) {
+      S = max(S, red3[i][0]);
+      E = max(E, red3[i][1]);
+      F = max(F, red3[i][2]);
+    }
+    const bool known = a.top2_known && F <= max(S, E);
+    a.scalars[2] = known ? 1.0f : 0.0f;
+    a.scalars[3] = __uint_as_float(max(S, E));
+    a.path_count[known ? 0 : 1] += 1;
+  }
+}
+
 // Kernel 4a: block maxima of |ds| over the dense elements. A thread's first loads of W
 // are issued before the block stages xx in LDS.
 __global__ __launch_bounds__(256) void fv_absmax_kernel(fv_dense_args a) {
   extern __shared__ float4 xs4[];  // xx, ldk4 float4
   __shared__ float smem4[4];
+  if (a.scalars[2] != 0.0f) return;  // max|ds| is known without the pass (fv_decide_kernel)
   const uint32_t stride = gridDim.x * 256;
   const uint32_t dq = stride % a.ldk4;
   uint32_t p4 = blockIdx.x * 256 + threadIdx.x;
@@ -1298,48 +1359,92 @@ __global__ __launch_bounds__(256) void fv_absmax_kernel(fv_dense_args a) {
   if (threadIdx.x == 0) a.bmax[blockIdx.x] = bm;
 }
 
-// Kernel 5: max|ds| from the block maxima, then W += (eps / max|ds|) * ds over the dense elements.
-// The first loads of W are in flight while the block reduces the maxima.
-__global__ __launch_bounds__(256) void fv_update_kernel(fv_dense_args a) {
-  extern __shared__ float4 xs4[];
-  __shared__ float smem4[4];
+// Kernel 5: max|ds| -- from fv_decide_kernel, else from the block maxima -- then W += (eps / max|ds|) * ds over
+// the dense elements. The first loads of W are in flight while the block finds the maximum. A block takes
+// whole rows of the token-major matrix, TB / ldk4 at a time, so that a thread keeps the same four neurons
+// throughout and can keep the two largest |W| it leaves behind for each of them; the block's share of every
+// row's two largest weights goes to top2_part[neuron][block] (the slot launch adds the sparse elements').
+template <int TB>
+__global__ __launch_bounds__(TB) void fv_update_kernel(fv_dense_args a) {
+  extern __shared__ float4 dyn4[];  // xx (ldk4 groups), then the threads' pairs (4 x TB)
+  float4 *xs4 = dyn4;
+  float2 *pairs = (float2 *)(dyn4 + a.ldk4);
+  __shared__ float smem16[16];
   __shared__ float sh_s;
-  const uint32_t stride = gridDim.x * 256;
-  const uint32_t dq = stride % a.ldk4;
-  uint32_t p4 = blockIdx.x * 256 + threadIdx.x;
-  uint32_t q = p4 % a.ldk4;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t rows_per_round = TB / a.ldk4;  // the launch is sized so that this is at least 1
+  const bool active = tid < rows_per_round * a.ldk4;
+  const uint32_t q = tid % a.ldk4, r = tid / a.ldk4;
+  const uint32_t row_step = gridDim.x * rows_per_round;
+  const uint32_t row0 = blockIdx.x * rows_per_round + r;
+  const uint32_t row_inside = min(row0, a.n_rows - 1);  // read again, and not used, by a load past the end
+  uint32_t row = active ? row0 : a.n_rows;
   float4 w[FV_UPDATE_UNROLL];
-  fv_dense_load(a, p4, stride, w);
-  for (uint32_t i = threadIdx.x; i < a.ldk4; i += 256) xs4[i] = ((const float4 *)a.xx)[i];
+#define FV_UPDATE_LOADS                                                              \
+  _Pragma("unroll") for (int u = 0; u < FV_UPDATE_UNROLL; ++u) {                     \
+    const uint32_t rr = row + u * row_step;                                          \
+    w[u] = a.Wt4[(rr < a.n_rows ? rr : row_inside) * a.ldk4 + q];                    \
+  }
+  FV_UPDATE_LOADS
+  for (uint32_t i = tid; i < a.ldk4; i += TB) xs4[i] = ((const float4 *)a.xx)[i];
   float nc = 0.0f;
-  {
+  const bool known = a.scalars[2] != 0.0f;
+  if (known) {
+    nc = a.scalars[3];
+  } else {
     const uint32_t n4 = a.n_bmax / 4;
     const float4 *b4 = (const float4 *)a.bmax;
-    for (uint32_t i = threadIdx.x; i < n4; i += 4 * 256) {  // four 16-byte loads together
+    for (uint32_t i = tid; i < n4; i += 4 * TB) {  // four 16-byte loads together
       float4 v[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = b4[min(i + u * 256, n4 - 1)];
+      for (int u = 0; u < 4; ++u) v[u] = b4[min(i + u * TB, n4 - 1)];
 #pragma unroll
       for (int u = 0; u < 4; ++u) nc = fmaxf(nc, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
     }
-    for (uint32_t i = 4 * n4 + threadIdx.x; i < a.n_bmax; i += 256) nc = fmaxf(nc, a.bmax[i]);
+    for (uint32_t i = 4 * n4 + tid; i < a.n_bmax; i += TB) nc = fmaxf(nc, a.bmax[i]);
   }
-  nc = fv_block_max_nonneg(nc, smem4);
-  if (threadIdx.x == 0) {
+  nc = fv_block_max_nonneg(nc, smem16);
+  if (tid == 0) {
     sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
     if (blockIdx.x == 0) a.scalars[0] = nc;
   }
   __syncthreads();
   const float s = sh_s;
-  while (p4 < a.total4) {
+  const float4 xq = xs4[q];
+  float t1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, t2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  while (row < a.n_rows) {
 #pragma unroll
     for (int u = 0; u < FV_UPDATE_UNROLL; ++u) {
-      if (p4 + u * stride < a.total4) fv_update_four(a, p4 + u * stride, w[u], xs4[q], s);
-      q += dq;
-      if (q >= a.ldk4) q -= a.ldk4;
+      const uint32_t rr = row + u * row_step;
+      if (rr < a.n_rows) {
+        float4 v = w[u];
+        // a sentinel goes back as it came; the slot launch replaces it
+        if (fv_apply_four(v, xq, s, a.update_cut)) a.Wt4[rr * a.ldk4 + q] = v;
+        fv_top2_insert(t1[0], t2[0], fv_abs_or_zero(v.x));
+        fv_top2_insert(t1[1], t2[1], fv_abs_or_zero(v.y));
+        fv_top2_insert(t1[2], t2[2], fv_abs_or_zero(v.z));
+        fv_top2_insert(t1[3], t2[3], fv_abs_or_zero(v.w));
+      }
     }
-    p4 += FV_UPDATE_UNROLL * stride;
-    if (p4 < a.total4) fv_dense_load(a, p4, stride, w);
+    row += FV_UPDATE_UNROLL * row_step;
+    if (row < a.n_rows) {
+      FV_UPDATE_LOADS
+    }
+  }
+#undef FV_UPDATE_LOADS
+  if (active) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pairs[(e * rows_per_round + r) * a.ldk4 + q] = make_float2(t1[e], t2[e]);
+  }
+  __syncthreads();
+  for (uint32_t h = tid; h < a.K; h += TB) {
+    const uint32_t e = h & 3u, qq = h >> 2;
+    float m1 = 0.0f, m2 = 0.0f;
+    for (uint32_t rr = 0; rr < rows_per_round; ++rr) {
+      const float2 b = pairs[(e * rows_per_round + rr) * a.ldk4 + qq];
+      fv_top2_merge(m1, m2, b.x, b.y);
+    }
+    a.top2_part[(uint64_t)blockIdx.x * a.ldk + h] = make_float2(m1, m2);
   }
 }
 
@@ -1393,8 +1498,6 @@ __device__ __forceinline__ void fv_top2_insert_lds(uint32_t *s1, uint32_t *s2, u
   const uint32_t old = atomicMax(&s1[h], b);
   atomicMax(&s2[h], min(old, b));
 }
-// |w| for that bookkeeping; a NaN (a sentinel) counts as 0
-__device__ __forceinline__ float fv_abs_or_zero(float w) { return w == w ? fabsf(w) : 0.0f; }
 
 // The element p holds the sentinel `bits`: its final value from the record the sentinel names. The saved
 // weight goes back where the row is not updated (xx == 0) or the launch gave up, else the updated one.
@@ -1510,9 +1613,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   const uint32_t er0 = samples0 ? e0 / a.idx_stride : 0u;
   const uint64_t start0 = a.ahead_n ? a.pstart[a.ahead_first + er0] : 0ull;
 
-  // What is known of max|ds| before the matrix is seen: S, the largest |ds| of a sparse element; E, the
-  // largest over the rows whose largest dense weight is known of fl(|xx| * that weight); F, the same over
-  // the other rows with an upper bound of that weight.
+  // what is known of max|ds| before the matrix is seen (fv_row_candidate)
   uint32_t S = 0, E = 0, F = 0;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -1522,19 +1623,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
       sp1[h] = 0;
       sp2[h] = 0;
     }
-    if (h < a.K) {
-      const uint32_t n1 = (hit4[j].x & 3u) + (hit4[j].y & 3u) + (hit4[j].z & 3u) + (hit4[j].w & 3u);
-      const uint32_t n2 = ((hit4[j].x >> 2) & 3u) + ((hit4[j].y >> 2) & 3u) + ((hit4[j].z >> 2) & 3u) + ((hit4[j].w >> 2) & 3u);
-      const float v1 = rm[j].x, v2 = rm[j].y;
-      // v1 == v2: two elements hold the largest value, one of them is dense unless two sparse ones hold it.
-      // v1 > v2: one element holds v1; if it is sparse, v2 bounds the rest, and is reached unless a
-      // sparse element holds it.
-      const bool first = v1 == v2 ? n1 <= 1 : n1 == 0;
-      const bool exact = first || (v1 != v2 && n2 == 0);
-      const uint32_t cand = __float_as_uint(__fmul_rn(fabsf(xh[j]), first ? v1 : v2));
-      if (exact) E = max(E, cand); else F = max(F, cand);
-      S = max(S, __float_as_uint(fmaxf(fmaxf(smx[j].x, smx[j].y), fmaxf(smx[j].z, smx[j].w))));
-    }
+    if (h < a.K) fv_row_candidate(xh[j], rm[j], hit4[j], smx[j], S, E, F);
   }
   if (tid == 0) sh_hits = 0;
   {
@@ -1703,7 +1792,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
       const float2 b = pairs[(e * rows_per_round + rr) * a.ldk4 + qq];
       fv_top2_merge(m1, m2, b.x, b.y);
     }
-    a.top2_part[(uint64_t)h * a.part_stride + blockIdx.x] = make_float2(m1, m2);
+    a.top2_part[(uint64_t)blockIdx.x * a.ldk + h] = make_float2(m1, m2);
   }
 }
 
@@ -1730,9 +1819,17 @@ static int fv_onepass_fits(size_t smem) {
 template <bool DELTA>
 __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
   // block (h, q) of the sparse launch wrote slot_count records at the start of its part of region q
+  __shared__ float2 wave_pair[4];
   const uint32_t count = a.slot_count[blockIdx.x];
-  if (count == 0) return;
   const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT, q = blockIdx.x & (FV_NB_CLASSES - 1);
+  // the two largest of what the block writes: its share of the row's two largest weights, behind the
+  // update launch's shares
+  float2 *share = a.top2_part + (uint64_t)(a.part_base + q) * a.ldk + h;
+  if (count == 0) {
+    if (threadIdx.x == 0) *share = make_float2(0.0f, 0.0f);
+    return;
+  }
+  float m1 = 0.0f, m2 = 0.0f;
   const uint64_t slot_first =
       (uint64_t)q * a.slot_stride + (uint64_t)(a.group_base[h] + (DELTA ? a.group_base2[h] : 0u)) * a.w;
   const fv_slot *slots = a.slots + slot_first;
@@ -1759,7 +1856,18 @@ __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
         if (fabsf(d) > a.update_cut) out = __fadd_rn(sl[u].wv, d);
       }
       ((float *)a.Wt4)[sl[u].p] = out;
+      fv_top2_insert(m1, m2, fv_abs_or_zero(out));
     }
+  }
+  for (int d = 32; d >= 1; d >>= 1) {  // the partner's pair covers other elements: no value is counted twice
+    const float b1 = __shfl_xor(m1, d, 64), b2 = __shfl_xor(m2, d, 64);
+    fv_top2_merge(m1, m2, b1, b2);
+  }
+  if ((threadIdx.x & 63) == 0) wave_pair[threadIdx.x >> 6] = make_float2(m1, m2);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int i = 1; i < 4; ++i) fv_top2_merge(m1, m2, wave_pair[i].x, wave_pair[i].y);
+    *share = make_float2(m1, m2);
   }
 }
 
@@ -1924,10 +2032,12 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMemsetAsync(t->row_top2, 0, (size_t)t->K * sizeof(float2), t->stream));
   FV_HIP(hipMalloc((void **)&t->path_count, 2 * sizeof(uint32_t)));
   FV_HIP(hipMemsetAsync(t->path_count, 0, 2 * sizeof(uint32_t), t->stream));
-  if (t->onepass_unroll) {
-    const size_t n_part = (size_t)t->K * t->onepass_blocks;
-    FV_HIP(hipMalloc((void **)&t->top2_part, n_part * sizeof(float2)));
-    FV_HIP(hipMemsetAsync(t->top2_part, 0, n_part * sizeof(float2), t->stream));
+  {
+    // shares per row: the single launch's blocks, or the update launch's blocks and the slot launch's four
+    const size_t per_row = t->onepass_blocks > t->update_blocks + FV_NB_CLASSES ? t->onepass_blocks
+                                                                                : t->update_blocks + FV_NB_CLASSES;
+    FV_HIP(hipMalloc((void **)&t->top2_part, (size_t)t->ldk * per_row * sizeof(float2)));
+    FV_HIP(hipMemsetAsync(t->top2_part, 0, (size_t)t->ldk * per_row * sizeof(float2), t->stream));
   }
   FV_HIP(hipMemsetAsync(t->win, 0, ((size_t)t->B + 16) * sizeof(int32_t), t->stream));
   FV_HIP(hipMalloc((void **)&t->win16, ((size_t)t->B + 64) * sizeof(uint16_t)));  // read in 16-byte pieces
@@ -2030,7 +2140,15 @@ extern "C" int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_tr
     if (want == 0) want = 1;
     const uint64_t cu = (uint64_t)(cus > 0 ? cus : 256);
     t->dense_blocks = (unsigned)(want < cu * FV_ABSMAX_BLOCKS_PER_CU ? want : cu * FV_ABSMAX_BLOCKS_PER_CU);
-    t->update_blocks = (unsigned)(want < cu * FV_UPDATE_BLOCKS_PER_CU ? want : cu * FV_UPDATE_BLOCKS_PER_CU);
+    {
+      // the update launch takes whole rows: 256-thread blocks, 512 when a row has more groups than that
+      const uint32_t ldk4 = t->ldk / 4;
+      t->update_threads = ldk4 <= 256 ? 256 : 512;
+      const uint64_t rows_per_round = t->update_threads / ldk4;
+      const uint64_t want_rows = (t->N + rows_per_round - 1) / rows_per_round;
+      const uint64_t cap = cu * FV_UPDATE_BLOCKS_PER_CU * 256 / t->update_threads;
+      t->update_blocks = (unsigned)(want_rows < cap ? want_rows : cap);
+    }
     fv_choose_onepass(t, cu);
     rc = fv_trainer_alloc(t);
   }
@@ -2262,13 +2380,13 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   const uint64_t n_slots = (uint64_t)FV_NB_CLASSES * t->B * t->w * (anti ? 2 : 1);
   const bool onepass = t->onepass && fv_trainers_alive.load() == 1 && n_slots + 1 < FV_SENTINEL_MAX;
   // the rows' two largest weights are in hand if the last write of the matrix was a single dense launch
-  const bool top2_known = whole ? onepass && t->top2_valid : t->last_top2_known;
+  const bool top2_known = whole ? t->top2_valid : t->last_top2_known;
   if (whole) t->last_top2_known = top2_known;
   fv_gather_args g;
-  g.merge_rows = (top2_known && (whole || (which & 1u))) ? t->K : 0u;
+  g.merge_rows = (top2_known && (whole || (which & 1u))) ? (t->K + FV_MERGE_NEURONS - 1) / FV_MERGE_NEURONS : 0u;
   g.top2_part = t->top2_part;
-  g.part_stride = t->onepass_blocks;
-  g.n_part = t->onepass_blocks;
+  g.part_stride = t->ldk;
+  g.n_part = t->top2_n_part;  // the shares the last dense launches left
   g.row_top2 = t->row_top2;
   g.Wt = t->Wt;
   g.corpus = t->corpus;
@@ -2453,7 +2571,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.row_hits = t->row_hits;
   d.top2_known = top2_known ? 1u : 0u;
   d.top2_part = t->top2_part;
-  d.part_stride = t->onepass_blocks;
+  d.part_base = onepass ? 0u : t->update_blocks;
   d.path_count = t->path_count;
   d.eps = eps;
   d.prec = t->cfg.prec;
@@ -2485,15 +2603,25 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
       if (t->onepass_unroll == 8) { FV_CASE(8) } else { FV_CASE(16) }
 #undef FV_CASE
       t->top2_valid = true;  // this launch leaves the shares of the matrix it writes
+      t->top2_n_part = t->onepass_blocks;
     }
     if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
   } else {
-    if (which & 8u)
+    if (which & 8u) {
+      // one block settles whether max|ds| is known from the rows' largest weights; the pass ends at once if so
+      hipLaunchKernelGGL(fv_decide_kernel, dim3(1), dim3(1024), 0, t->stream, d);
       hipLaunchKernelGGL(fv_absmax_kernel, dim3(t->dense_blocks), dim3(256), smem, t->stream, d);
+    }
     if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
     if (which & 16u) {
-      hipLaunchKernelGGL(fv_update_kernel, dim3(t->update_blocks), dim3(256), smem, t->stream, d);
-      t->top2_valid = false;  // the matrix changes and nobody keeps the rows' largest weights
+      const size_t smem_u = smem + (size_t)t->update_threads * 4 * sizeof(float2);
+      if (t->update_threads == 256)
+        hipLaunchKernelGGL(fv_update_kernel<256>, dim3(t->update_blocks), dim3(256), smem_u, t->stream, d);
+      else
+        hipLaunchKernelGGL(fv_update_kernel<512>, dim3(t->update_blocks), dim3(512), smem_u, t->stream, d);
+      // with the slot launch behind it, the two leave the shares of the matrix they write
+      t->top2_valid = whole;
+      t->top2_n_part = t->update_blocks + FV_NB_CLASSES;
     }
   }
   if (ev) FV_HIP(hipEventRecord(ev[5], t->stream));
