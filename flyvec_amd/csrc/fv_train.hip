@@ -127,6 +127,8 @@ struct fv_trainer {
   // describes the matrix as it is (top2_valid: set by a single dense launch, cleared by every other
   // write of the matrix), and whether the last whole step used them.
   float2 *row_top2, *top2_part;
+  float2 *top2_stage;  // inside row_top2's allocation
+  bool top2_merged;    // row_top2 already holds the merged pairs (separate dense launches merge behind themselves)
   uint32_t *row_hits;
   uint32_t *path_count;  // device: launches that took max|ds| from them / that made the pass
   bool top2_valid, last_top2_known;
@@ -160,30 +162,62 @@ __device__ __forceinline__ void fv_top2_merge(float &m1, float &m2, float b1, fl
 }
 
 // The shares of every row's two largest weights that the blocks of the last dense launches left
-// (top2_part[block][neuron], a block's pairs side by side), merged: row_top2[h] for the step that begins.
-// One 256-thread block per 32 neurons, run as the first blocks of the winner kernel's launch: eight threads
-// per neuron share the blocks among them, eight loads in flight each.
+// (top2_part[block][neuron], a block's pairs side by side) are merged into row_top2[neuron] for the step that
+// begins: one 256-thread block per 32 neurons and per chunk of FV_MERGE_CHUNK shares, eight threads per
+// neuron sharing the chunk's blocks among them, eight loads in flight each. A single dense launch leaves
+// one chunk, which the first blocks of the next winner kernel's launch merge. Separate dense launches
+// leave a share per block of a large grid: two small launches behind them merge first every chunk into a
+// staging array, then the staged pairs (fv_merge_shares_kernel, fv_merge_stage_kernel).
 #define FV_MERGE_NEURONS 32
-__device__ __forceinline__ void fv_merge_row_top2(const float2 *__restrict__ part, uint32_t part_stride, uint32_t n_part,
-                                                  uint32_t K, float2 *__restrict__ row_top2, uint32_t group) {
+#define FV_MERGE_CHUNK 256
+struct fv_merge_args {
+  const float2 *part;  // top2_part
+  uint32_t stride;     // pairs per share (ldk)
+  uint32_t n_part;     // shares
+  uint32_t K;
+  float2 *row_top2;    // out
+  float2 *stage;       // [chunk][ldk], used with more than one chunk
+};
+
+__device__ __forceinline__ void fv_merge_row_top2(const fv_merge_args &a, uint32_t block) {
   __shared__ float2 sh_pair[8][FV_MERGE_NEURONS];
+  const uint32_t groups = (a.K + FV_MERGE_NEURONS - 1) / FV_MERGE_NEURONS;
+  const uint32_t chunks = (a.n_part + FV_MERGE_CHUNK - 1) / FV_MERGE_CHUNK;
+  const uint32_t group = block % groups, chunk = block / groups;
+  const uint32_t first = chunk * FV_MERGE_CHUNK, last = min(first + FV_MERGE_CHUNK, a.n_part);  // shares [first, last)
   const uint32_t hh = threadIdx.x & (FV_MERGE_NEURONS - 1), bl = threadIdx.x / FV_MERGE_NEURONS;
-  const uint32_t h = min(group * FV_MERGE_NEURONS + hh, K - 1);  // past K: the last neuron once more, not stored
+  const bool real = group * FV_MERGE_NEURONS + hh < a.K;
+  const uint32_t h = min(group * FV_MERGE_NEURONS + hh, a.K - 1);  // past K: the last neuron once more, not stored
   float m1 = 0.0f, m2 = 0.0f;
-  for (uint32_t b0 = bl; b0 < n_part; b0 += 64) {
+  for (uint32_t b0 = first + bl; b0 < last; b0 += 64) {
     float2 v[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = part[(uint64_t)min(b0 + 8u * u, n_part - 1) * part_stride + h];
+    for (int u = 0; u < 8; ++u) v[u] = a.part[(uint64_t)min(b0 + 8u * u, last - 1) * a.stride + h];
 #pragma unroll
     for (int u = 0; u < 8; ++u)
-      if (b0 + 8u * u < n_part) fv_top2_merge(m1, m2, v[u].x, v[u].y);
+      if (b0 + 8u * u < last) fv_top2_merge(m1, m2, v[u].x, v[u].y);
   }
   sh_pair[bl][hh] = make_float2(m1, m2);
   __syncthreads();
-  if (bl == 0 && group * FV_MERGE_NEURONS + hh < K) {
+  if (bl == 0 && real) {
     for (int i = 1; i < 8; ++i) fv_top2_merge(m1, m2, sh_pair[i][hh].x, sh_pair[i][hh].y);
-    row_top2[h] = make_float2(m1, m2);
+    float2 *out = chunks == 1 ? a.row_top2 : a.stage + (uint64_t)chunk * a.stride;
+    out[h] = make_float2(m1, m2);
   }
+}
+
+__global__ __launch_bounds__(256) void fv_merge_shares_kernel(fv_merge_args a) { fv_merge_row_top2(a, blockIdx.x); }
+
+__global__ __launch_bounds__(256) void fv_merge_stage_kernel(fv_merge_args a) {
+  const uint32_t h = blockIdx.x * 256 + threadIdx.x;
+  if (h >= a.K) return;
+  const uint32_t chunks = (a.n_part + FV_MERGE_CHUNK - 1) / FV_MERGE_CHUNK;
+  float m1 = 0.0f, m2 = 0.0f;
+  for (uint32_t c = 0; c < chunks; ++c) {
+    const float2 b = a.stage[(uint64_t)c * a.stride + h];
+    fv_top2_merge(m1, m2, b.x, b.y);
+  }
+  a.row_top2[h] = make_float2(m1, m2);
 }
 
 // ---- kernel 1: sampler + gather-sum + winner ----------------------------------------------------
@@ -211,11 +245,9 @@ struct fv_gather_args {
   uint32_t prune;    // in-window duplicate pruning while sampling
   float lmid, lbase; // weight of a window's centre position and of the others (WEIGHTED kernels)
   // the first merge_rows blocks of the launch merge the shares of the rows' two largest weights that the
-  // last dense launches left (fv_merge_row_top2: a block per 32 neurons); 0: none
+  // last dense launches left (fv_merge_row_top2: a block per 32 neurons and chunk of shares); 0: none
   uint32_t merge_rows;
-  const float2 *top2_part;
-  uint32_t part_stride, n_part;  // pairs per share (ldk), shares
-  float2 *row_top2;
+  fv_merge_args merge;
 };
 
 // FV_GATHER_WINDOWS windows per wavefront, one after the other: the grid then fits the machine in
@@ -253,7 +285,7 @@ __device__ __forceinline__ int32_t fv_column_index(int32_t tok, uint32_t c, uint
 template <int NV, bool DELTA, bool WEIGHTED>
 __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a) {
   if (blockIdx.x < a.merge_rows) {
-    fv_merge_row_top2(a.top2_part, a.part_stride, a.n_part, a.K, a.row_top2, blockIdx.x);
+    fv_merge_row_top2(a.merge, blockIdx.x);
     return;
   }
   const int lane = threadIdx.x & 63;
@@ -2028,8 +2060,16 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMemsetAsync(t->bmax, 0, n_bmax * sizeof(float), t->stream));
   FV_HIP(hipMalloc((void **)&t->row_hits, (size_t)FV_NB_CLASSES * t->K * sizeof(uint32_t)));
   FV_HIP(hipMemsetAsync(t->row_hits, 0, (size_t)FV_NB_CLASSES * t->K * sizeof(uint32_t), t->stream));
-  FV_HIP(hipMalloc((void **)&t->row_top2, (size_t)t->K * sizeof(float2)));
-  FV_HIP(hipMemsetAsync(t->row_top2, 0, (size_t)t->K * sizeof(float2), t->stream));
+  {
+    const size_t shares = t->onepass_blocks > t->update_blocks + FV_NB_CLASSES ? t->onepass_blocks
+                                                                               : t->update_blocks + FV_NB_CLASSES;
+    const size_t chunks = (shares + FV_MERGE_CHUNK - 1) / FV_MERGE_CHUNK;
+    // row_top2, then the staging array of the merge
+    const size_t bytes = (1 + chunks) * t->ldk * sizeof(float2);
+    FV_HIP(hipMalloc((void **)&t->row_top2, bytes));
+    FV_HIP(hipMemsetAsync(t->row_top2, 0, bytes, t->stream));
+    t->top2_stage = t->row_top2 + t->ldk;
+  }
   FV_HIP(hipMalloc((void **)&t->path_count, 2 * sizeof(uint32_t)));
   FV_HIP(hipMemsetAsync(t->path_count, 0, 2 * sizeof(uint32_t), t->stream));
   {
@@ -2383,11 +2423,14 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   const bool top2_known = whole ? t->top2_valid : t->last_top2_known;
   if (whole) t->last_top2_known = top2_known;
   fv_gather_args g;
-  g.merge_rows = (top2_known && (whole || (which & 1u))) ? (t->K + FV_MERGE_NEURONS - 1) / FV_MERGE_NEURONS : 0u;
-  g.top2_part = t->top2_part;
-  g.part_stride = t->ldk;
-  g.n_part = t->top2_n_part;  // the shares the last dense launches left
-  g.row_top2 = t->row_top2;
+  const uint32_t merge_groups = (t->K + FV_MERGE_NEURONS - 1) / FV_MERGE_NEURONS;
+  g.merge_rows = (top2_known && !t->top2_merged && (whole || (which & 1u))) ? merge_groups : 0u;  // one chunk
+  g.merge.part = t->top2_part;
+  g.merge.stride = t->ldk;
+  g.merge.n_part = t->top2_n_part;  // the shares the last dense launches left
+  g.merge.K = t->K;
+  g.merge.row_top2 = t->row_top2;
+  g.merge.stage = t->top2_stage;
   g.Wt = t->Wt;
   g.corpus = t->corpus;
   g.pstart = t->pstart;
@@ -2604,6 +2647,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
 #undef FV_CASE
       t->top2_valid = true;  // this launch leaves the shares of the matrix it writes
       t->top2_n_part = t->onepass_blocks;
+      t->top2_merged = false;  // the next winner kernel's first blocks merge them
+      static_assert(FV_ONEPASS_BLOCKS_PER_CU == 1, "a single dense launch leaves no more shares than one chunk holds");
     }
     if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
   } else {
@@ -2630,6 +2675,17 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
       hipLaunchKernelGGL(fv_slot_update_kernel<true>, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, d);
     else
       hipLaunchKernelGGL(fv_slot_update_kernel<false>, dim3(t->K * FV_NB_CLASSES), dim3(256), 0, t->stream, d);
+    if (whole) {
+      // the shares the update and slot launches have left, merged here: a share per block of a large grid is
+      // more than the next winner kernel's first blocks should be kept busy with
+      fv_merge_args m = g.merge;
+      m.n_part = t->top2_n_part;
+      const uint32_t chunks = (m.n_part + FV_MERGE_CHUNK - 1) / FV_MERGE_CHUNK;
+      hipLaunchKernelGGL(fv_merge_shares_kernel, dim3(merge_groups * chunks), dim3(256), 0, t->stream, m);
+      if (chunks > 1)
+        hipLaunchKernelGGL(fv_merge_stage_kernel, dim3((t->K + 255) / 256), dim3(256), 0, t->stream, m);
+      t->top2_merged = true;
+    }
   }
   if (ev) FV_HIP(hipEventRecord(ev[6], t->stream));
   FV_HIP(hipGetLastError());
