@@ -15,6 +15,9 @@
 #include <math.h>
 #include <string.h>
 
+#include <atomic>
+#include <memory>
+#include <thread>
 #include <vector>
 
 #include "fv_internal.h"
@@ -31,6 +34,10 @@ struct fv_hash_lane {
   uint64_t *bits;
   int8_t *codes;
   size_t idx_cap, bits_cap, codes_cap;  // bytes
+  // page-locked staging for outputs that go to pageable host memory, and the event behind a chunk's copies
+  char *stage_bits, *stage_codes;
+  size_t stage_bits_cap, stage_codes_cap;
+  hipEvent_t done;
 };
 
 struct fv_hasher {
@@ -179,6 +186,9 @@ extern "C" int fv_hasher_destroy(fv_hasher *h) {
     (void)hipFree(ln.idx);
     (void)hipFree(ln.bits);
     (void)hipFree(ln.codes);
+    if (ln.stage_bits) (void)hipHostFree(ln.stage_bits);
+    if (ln.stage_codes) (void)hipHostFree(ln.stage_codes);
+    if (ln.done) (void)hipEventDestroy(ln.done);
   }
   (void)hipFree(h->Wt);
   (void)hipFree(h->err);
@@ -263,10 +273,81 @@ static int fv_hash_reserve(P **buf, size_t *cap, size_t bytes) {
   return FV_OK;
 }
 
+static int fv_hash_reserve_pinned(char **buf, size_t *cap, size_t bytes) {
+  if (*cap >= bytes) return FV_OK;
+  if (*buf) (void)hipHostFree(*buf);
+  *buf = nullptr;
+  *cap = 0;
+  FV_HIP(hipHostMalloc((void **)buf, bytes, hipHostMallocDefault));
+  *cap = bytes;
+  return FV_OK;
+}
+
+// Ordinary (pageable) host memory, which the device cannot write by DMA?
+static bool fv_is_pageable(const void *p) {
+  hipPointerAttribute_t at;
+  if (hipPointerGetAttributes(&at, p) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;
+  }
+  return at.type == hipMemoryTypeUnregistered;
+}
+
+// Copies from page-locked staging to the caller's pageable buffers, done by a few host threads while the
+// device works on the next chunks: one thread copies ~10 GB/s, less than the link delivers. Items are
+// published in order; every worker copies its slice of every item.
+#define FV_HASH_COPY_THREADS 4
+struct fv_copy_ring {
+  struct item {
+    const char *src;
+    char *dst;
+    size_t bytes;
+  };
+  std::vector<item> items;
+  std::unique_ptr<std::atomic<uint32_t>[]> finished;  // workers done with item i
+  std::atomic<uint32_t> published{0};
+  std::atomic<bool> quit{false};
+  std::vector<std::thread> workers;
+
+  explicit fv_copy_ring(size_t max_items) : items(max_items), finished(new std::atomic<uint32_t>[max_items]) {
+    for (size_t i = 0; i < max_items; ++i) finished[i].store(0);
+    for (int p = 0; p < FV_HASH_COPY_THREADS; ++p) workers.emplace_back([this, p] { run(p); });
+  }
+  void run(int p) {
+    for (uint32_t i = 0;; ++i) {
+      while (published.load(std::memory_order_acquire) <= i) {
+        if (quit.load(std::memory_order_acquire)) return;
+        std::this_thread::yield();
+      }
+      const item &it = items[i];
+      const size_t per = (it.bytes + FV_HASH_COPY_THREADS - 1) / FV_HASH_COPY_THREADS;
+      const size_t lo = per * p < it.bytes ? per * p : it.bytes, hi = lo + per < it.bytes ? lo + per : it.bytes;
+      if (hi > lo) memcpy(it.dst + lo, it.src + lo, hi - lo);
+      finished[i].fetch_add(1, std::memory_order_release);
+    }
+  }
+  uint32_t publish(const char *src, char *dst, size_t bytes) {
+    const uint32_t i = published.load(std::memory_order_relaxed);
+    items[i] = {src, dst, bytes};
+    published.store(i + 1, std::memory_order_release);
+    return i;
+  }
+  void wait(uint32_t i) {
+    while (finished[i].load(std::memory_order_acquire) < FV_HASH_COPY_THREADS) std::this_thread::yield();
+  }
+  ~fv_copy_ring() {
+    for (uint32_t i = 0; i < published.load(); ++i) wait(i);
+    quit.store(true, std::memory_order_release);
+    for (auto &t : workers) t.join();
+  }
+};
+
 // A batch in host memory: chunks of FV_HASH_CHUNK windows alternate between the lanes; on its lane a
 // chunk is copied in, hashed and copied out in stream order, so the copies of one chunk overlap the kernel
-// of the other. Host buffers from fv_host_alloc_pinned are copied by DMA as they are; pageable ones go
-// through the runtime's staging. Nothing is allocated once the lanes' buffers have reached the chunk size.
+// of the other. Host buffers from fv_host_alloc_pinned are copied by DMA as they are. Outputs that go to
+// pageable memory are copied by DMA into the lane's page-locked staging and from there by host threads
+// (fv_copy_ring) while the device goes on; pageable inputs go through the runtime's staging. Nothing is
+// allocated once the lanes' buffers have reached the chunk size.
 static int fv_hash_host(fv_hasher *h, const int32_t *idx, uint64_t n, uint32_t w, uint32_t k, int32_t shift,
                         uint64_t *out_bits, int8_t *out_codes) {
   if (n == 0) return FV_OK;
@@ -274,6 +355,10 @@ static int fv_hash_host(fv_hasher *h, const int32_t *idx, uint64_t n, uint32_t w
   const uint32_t words = (h->K + 63) / 64;
   const uint64_t chunk = n < FV_HASH_CHUNK ? n : FV_HASH_CHUNK;
   const int lanes = n > chunk ? FV_HASH_LANES : 1;
+  const size_t bits_row = words * sizeof(uint64_t), codes_row = h->K;
+  // staging pays off for outputs of some size that the device cannot reach by DMA
+  const bool stage_bits = out_bits && lanes > 1 && fv_is_pageable(out_bits);
+  const bool stage_codes = out_codes && lanes > 1 && fv_is_pageable(out_codes);
   FV_HIP(hipStreamSynchronize(h->stream));  // what the caller enqueued on the hasher's stream comes first
   for (int l = 0; l < lanes; ++l) {
     fv_hash_lane &ln = h->lane[l];
@@ -283,15 +368,32 @@ static int fv_hash_host(fv_hasher *h, const int32_t *idx, uint64_t n, uint32_t w
       else
         FV_HIP(hipStreamCreate(&ln.stream));
     }
+    if (!ln.done) FV_HIP(hipEventCreateWithFlags(&ln.done, hipEventDisableTiming));
     FV_TRY(fv_hash_reserve(&ln.idx, &ln.idx_cap, chunk * w * sizeof(int32_t)));
-    if (out_bits) FV_TRY(fv_hash_reserve(&ln.bits, &ln.bits_cap, chunk * words * sizeof(uint64_t)));
-    if (out_codes) FV_TRY(fv_hash_reserve(&ln.codes, &ln.codes_cap, chunk * (size_t)h->K));
+    if (out_bits) FV_TRY(fv_hash_reserve(&ln.bits, &ln.bits_cap, chunk * bits_row));
+    if (out_codes) FV_TRY(fv_hash_reserve(&ln.codes, &ln.codes_cap, chunk * codes_row));
+    if (stage_bits) FV_TRY(fv_hash_reserve_pinned(&ln.stage_bits, &ln.stage_bits_cap, chunk * bits_row));
+    if (stage_codes) FV_TRY(fv_hash_reserve_pinned(&ln.stage_codes, &ln.stage_codes_cap, chunk * codes_row));
   }
+  const uint64_t n_chunks = (n + chunk - 1) / chunk;
+  std::unique_ptr<fv_copy_ring> ring;
+  if (stage_bits || stage_codes) ring.reset(new fv_copy_ring(2 * n_chunks));
+  std::vector<uint32_t> last_item(n_chunks, 0xffffffffu);  // the last copy item of every chunk
   int rc = FV_OK;
-  uint64_t c = 0;
-  for (uint64_t first = 0; first < n && rc == FV_OK; first += chunk, ++c) {
+  // chunk c's staged outputs are handed to the host threads once its copies have landed (one iteration later,
+  // while the device works on chunk c + 1), and have left the staging before chunk c + 2 is copied into it
+  auto hand_over = [&](uint64_t c) -> int {
     fv_hash_lane &ln = h->lane[c % lanes];
-    const uint64_t m = n - first < chunk ? n - first : chunk;
+    FV_HIP(hipEventSynchronize(ln.done));
+    const uint64_t first = c * chunk, m = n - first < chunk ? n - first : chunk;
+    if (stage_bits) last_item[c] = ring->publish(ln.stage_bits, (char *)out_bits + first * bits_row, m * bits_row);
+    if (stage_codes) last_item[c] = ring->publish(ln.stage_codes, (char *)out_codes + first * codes_row, m * codes_row);
+    return FV_OK;
+  };
+  for (uint64_t c = 0; c < n_chunks && rc == FV_OK; ++c) {
+    fv_hash_lane &ln = h->lane[c % lanes];
+    const uint64_t first = c * chunk, m = n - first < chunk ? n - first : chunk;
+    if (ring && c >= (uint64_t)lanes && last_item[c - lanes] != 0xffffffffu) ring->wait(last_item[c - lanes]);
     hipError_t e = hipMemcpyAsync(ln.idx, idx + first * w, m * w * sizeof(int32_t), hipMemcpyHostToDevice, ln.stream);
     if (e != hipSuccess) {
       rc = fv_fail(FV_ERR_HIP, "hash upload failed: %s", hipGetErrorString(e));
@@ -300,14 +402,23 @@ static int fv_hash_host(fv_hasher *h, const int32_t *idx, uint64_t n, uint32_t w
     rc = fv_enqueue_hash(h, ln.idx, m, w, k, shift, out_bits ? ln.bits : nullptr, out_codes ? ln.codes : nullptr,
                          ln.stream);
     if (rc == FV_OK && out_bits) {
-      e = hipMemcpyAsync(out_bits + first * words, ln.bits, m * words * sizeof(uint64_t), hipMemcpyDeviceToHost, ln.stream);
+      void *dst = stage_bits ? (void *)ln.stage_bits : (void *)((char *)out_bits + first * bits_row);
+      e = hipMemcpyAsync(dst, ln.bits, m * bits_row, hipMemcpyDeviceToHost, ln.stream);
       if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
     }
     if (rc == FV_OK && out_codes) {
-      e = hipMemcpyAsync(out_codes + first * (uint64_t)h->K, ln.codes, m * (uint64_t)h->K, hipMemcpyDeviceToHost, ln.stream);
+      void *dst = stage_codes ? (void *)ln.stage_codes : (void *)((char *)out_codes + first * codes_row);
+      e = hipMemcpyAsync(dst, ln.codes, m * codes_row, hipMemcpyDeviceToHost, ln.stream);
       if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "download failed: %s", hipGetErrorString(e));
     }
+    if (rc == FV_OK && ring) {
+      e = hipEventRecord(ln.done, ln.stream);
+      if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "event record failed: %s", hipGetErrorString(e));
+      if (rc == FV_OK && c >= 1) rc = hand_over(c - 1);
+    }
   }
+  if (rc == FV_OK && ring) rc = hand_over(n_chunks - 1);
+  ring.reset();  // waits for the host threads' copies
   for (int l = 1; l < lanes; ++l) {
     const hipError_t e = hipStreamSynchronize(h->lane[l].stream);
     if (e != hipSuccess && rc == FV_OK) rc = fv_fail(FV_ERR_HIP, "hash stream failed: %s", hipGetErrorString(e));
