@@ -65,6 +65,7 @@ SIGNATURES = {
     "fv_trainer_create": [C.POINTER(TrainConfig), _pp],
     "fv_trainer_destroy": [_vp],
     "fv_trainer_set_corpus": [_vp, _vp, _u64, _vp, _u64],
+    "fv_trainer_set_corpus_starts": [_vp, _vp, _u64, _vp, _u64],
     "fv_trainer_num_windows": [_vp, C.POINTER(_u64)],
     "fv_trainer_get_window_starts": [_vp, _vp, _u64],
     "fv_trainer_get_inverse_frequency": [_vp, _vp],

@@ -14,7 +14,9 @@ CSRC = PKG / "csrc"
 INCLUDE = PKG.parent / "include"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libflyvec_hip.so"
-SOURCES = ["fv_runtime.hip", "fv_corpus.hip", "fv_train.hip", "fv_hash.hip"]
+SOURCES = ["fv_runtime.hip", "fv_corpus.hip", "fv_train.hip", "fv_hash.hip", "fv_legacy.hip"]
+# the five shared objects the reference's driver opens (flyvec/train_flyvec.py:62-66)
+LEGACY_NAMES = ["model_descriptor.so", "model_arrays.so", "cuda_helpers.so", "cuda_funcs.so", "prune_input.so"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared",
@@ -48,9 +50,29 @@ def build(verbose=False, extra_flags=()):
     return LIB_PATH
 
 
+def install_legacy_names(directory):
+    """Links the reference's five library names in `directory` to libflyvec_hip.so, which exports their
+    symbols as well (include/flyvec_legacy.h): the reference's driver then runs on this library."""
+    directory = Path(directory)
+    directory.mkdir(parents=True, exist_ok=True)
+    for name in LEGACY_NAMES:
+        link = directory / name
+        if link.is_symlink() or link.exists():
+            link.unlink()
+        link.symlink_to(LIB_PATH)
+    return [directory / n for n in LEGACY_NAMES]
+
+
 def main():
+    import argparse
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--legacy-names", metavar="DIR", help="also link the reference's five library names in DIR")
+    args = ap.parse_args()
     path = build(verbose=True)
     print(f"built {path}")
+    if args.legacy_names:
+        for link in install_legacy_names(args.legacy_names):
+            print(f"linked {link}")
 
 
 if __name__ == "__main__":

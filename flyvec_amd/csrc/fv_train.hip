@@ -2262,6 +2262,56 @@ extern "C" int fv_trainer_set_corpus(fv_trainer *t, const int32_t *tokens, uint6
   return FV_OK;
 }
 
+// The same with the window table given instead of built: what the reference's driver hands over
+// (flyvec/src/model_arrays.cu:358 set_up_INPUT_pointer takes the corpus and the table that
+// compute_offset_phrases wrote; :396 compute_inverse_word_frequency the corpus length).
+extern "C" int fv_trainer_set_corpus_starts(fv_trainer *t, const int32_t *tokens, uint64_t n_tokens,
+                                            const uint64_t *starts, uint64_t n_windows) {
+  FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
+  FV_REQUIRE(tokens && n_tokens > 0, FV_ERR_INVALID, "empty corpus");
+  FV_REQUIRE(starts || n_windows == 0, FV_ERR_INVALID, "null window table");
+  for (uint64_t i = 0; i < n_windows; ++i)
+    FV_REQUIRE(starts[i] <= n_tokens && t->w <= n_tokens - starts[i], FV_ERR_DATA,
+               "window %llu starts at token %llu: it does not fit the corpus of %llu", (unsigned long long)i,
+               (unsigned long long)starts[i], (unsigned long long)n_tokens);
+  FV_HIP(hipStreamSynchronize(t->stream));
+  fv_trainer_free_corpus(t);
+  int rc = FV_OK;
+  hipError_t e = hipMalloc((void **)&t->corpus, n_tokens * sizeof(int32_t));
+  if (e == hipSuccess) e = hipMalloc((void **)&t->invf, t->V * sizeof(float));
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(t->corpus, tokens, n_tokens * sizeof(int32_t), hipMemcpyHostToDevice, t->stream);
+  if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "corpus upload failed: %s", hipGetErrorString(e));
+  int32_t lo = 0, hi = 0;
+  if (rc == FV_OK) rc = fv_dev_inverse_frequency(t->corpus, n_tokens, t->V, t->invf, &lo, &hi, t->stream);
+  if (rc == FV_OK && (lo < -1 || (hi >= 0 && (uint64_t)hi >= t->V)))
+    rc = fv_fail(FV_ERR_DATA, "token ids span [%d, %d]; allowed are -1 (masked) and 0..%llu", lo, hi,
+                 (unsigned long long)(t->V - 1));
+  if (rc == FV_OK && n_windows) {
+    e = hipMalloc((void **)&t->starts, n_windows * sizeof(uint64_t));
+    if (e == hipSuccess) e = hipMalloc((void **)&t->perm, n_windows * sizeof(uint64_t));
+    if (e == hipSuccess) e = hipMalloc((void **)&t->pstart, n_windows * sizeof(uint64_t));
+    if (e == hipSuccess)
+      e = hipMemcpyAsync(t->starts, starts, n_windows * sizeof(uint64_t), hipMemcpyHostToDevice, t->stream);
+    if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "window table upload failed: %s", hipGetErrorString(e));
+    if (rc == FV_OK) {
+      hipLaunchKernelGGL(fv_identity_kernel, dim3(fv_perm_blocks(n_windows)), dim3(256), 0, t->stream, t->perm, n_windows);
+      hipLaunchKernelGGL(fv_order_starts_kernel, dim3(fv_perm_blocks(n_windows)), dim3(256), 0, t->stream, t->perm,
+                         t->starts, t->pstart, n_windows);
+      e = hipStreamSynchronize(t->stream);
+      if (e != hipSuccess) rc = fv_fail(FV_ERR_HIP, "permutation fill failed: %s", hipGetErrorString(e));
+    }
+  }
+  if (rc != FV_OK) {
+    fv_trainer_free_corpus(t);
+    return rc;
+  }
+  t->n_tokens = n_tokens;
+  t->n_windows = n_windows;
+  t->have_corpus = true;
+  return FV_OK;
+}
+
 extern "C" int fv_trainer_num_windows(fv_trainer *t, uint64_t *out_count) {
   FV_REQUIRE(t && out_count, FV_ERR_INVALID, "null argument");
   FV_REQUIRE(t->have_corpus, FV_ERR_STATE, "no corpus set");

@@ -74,6 +74,12 @@ class Trainer:
         offsets = np.ascontiguousarray(offsets, dtype=np.uint64)
         check(self.lib.fv_trainer_set_corpus(self.handle, ptr(tokens), len(tokens), ptr(offsets), len(offsets)))
 
+    def set_corpus_starts(self, tokens, starts):
+        """The corpus with a window-start table built elsewhere (what the reference's driver passes)."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        starts = np.ascontiguousarray(starts, dtype=np.uint64)
+        check(self.lib.fv_trainer_set_corpus_starts(self.handle, ptr(tokens), len(tokens), ptr(starts), len(starts)))
+
     @property
     def num_windows(self):
         out = C.c_uint64(0)

@@ -139,6 +139,11 @@ int fv_trainer_destroy(fv_trainer *t);
  * n_offsets entries (n_offsets-1 chunks). Fails with FV_ERR_DATA on ids outside [-1, V). */
 int fv_trainer_set_corpus(fv_trainer *t, const int32_t *tokens, uint64_t n_tokens,
                           const uint64_t *offsets, uint64_t n_offsets);
+/* flyvec/src/model_arrays.cu:358 set_up_INPUT_pointer as the reference's driver calls it: the corpus and
+ * the window-start table that compute_offset_phrases wrote (every start + window <= n_tokens, else
+ * FV_ERR_DATA); builds 1/frequency and the identity permutation like fv_trainer_set_corpus. */
+int fv_trainer_set_corpus_starts(fv_trainer *t, const int32_t *tokens, uint64_t n_tokens,
+                                 const uint64_t *starts, uint64_t n_windows);
 int fv_trainer_num_windows(fv_trainer *t, uint64_t *out_count);
 /* Read-back of what set_corpus built (parity hooks). */
 int fv_trainer_get_window_starts(fv_trainer *t, uint64_t *out_starts, uint64_t capacity);

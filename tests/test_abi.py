@@ -87,3 +87,36 @@ def test_without_a_gpu_the_product_raises_instead_of_falling_back():
         pytest.skip("a GPU is present")
     with pytest.raises(_lib.FlyvecError):
         Trainer(vocab=100, hid=16, window=3, batch=8)
+
+
+LEGACY_HEADER = os.path.join(ROOT, "include", "flyvec_legacy.h")
+LEGACY_SYMBOLS = ["do_gpu_cudaMallocManaged", "do_cpu_malloc", "do_gpu_cudaHostAlloc", "get_cuda_num_devices",
+                  "prune_input_data", "getnum_samples", "compute_offset_phrases", "model_create_descriptor",
+                  "set_model_param_int", "set_model_param_float", "compute_model_derived_parameters",
+                  "copy_model_params", "print_model_params", "model_create_arrays", "model_arrays_allocate_memory",
+                  "push_INPUT_memory_to_GPU", "get_data_pointer", "set_data_pointer", "set_up_INPUT_pointer",
+                  "compute_inverse_word_frequency", "do_reshuffle_indices", "launch_epoch_INPUT_AS_INT",
+                  "launch_epoch_INPUT_AS_IMAGE", "launch_epoch_INPUT_AS_FLOAT"]
+
+
+def test_legacy_surface_is_declared_and_exported(tmp_path):
+    """The 24 symbols the reference's driver binds from its five shared objects (flyvec/train_flyvec.py:62-139)."""
+    from flyvec_amd import _lib, build
+    text = re.sub(r"/\*.*?\*/", "", open(LEGACY_HEADER).read(), flags=re.S)
+    declared = set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\(", text))
+    assert set(LEGACY_SYMBOLS) <= declared
+    lib = C.CDLL(str(_lib.LIB_PATH))
+    assert not [s for s in LEGACY_SYMBOLS if not hasattr(lib, s)]
+    assert hasattr(lib, "flyvec_legacy_release") and "flyvec_legacy_release" in declared   # the one addition
+    links = build.install_legacy_names(tmp_path / "bin")
+    assert sorted(p.name for p in links) == sorted(build.LEGACY_NAMES)
+    for p in links:                                    # each name opens the one library
+        assert hasattr(C.CDLL(str(p)), "launch_epoch_INPUT_AS_INT")
+    # the descriptor needs no device
+    lib.model_create_descriptor.restype = C.c_void_p
+    d = lib.model_create_descriptor(C.c_int32(1))
+    lib.set_model_param_int(C.c_uint64(123), b"vocabulary_size", C.c_void_p(d))
+    lib.set_model_param_int(C.c_uint64(1), b"sparse_input", C.c_void_p(d))
+    lib.set_model_param_float(C.c_float(0.5), b"delta", C.c_void_p(d))
+    lib.compute_model_derived_parameters(C.c_void_p(d))
+    lib.print_model_params(C.c_void_p(d))
