@@ -35,6 +35,14 @@
  * is the plain sum in window order).  fvo_xx_sums is pinned by a numpy
  * restatement of that order and by its agreement with plain window order (to
  * rounding) in tests/test_oracle_train.py.
+ *
+ * Parity unpinned against the reference BINARY in one rounding: the update
+ * W += (eps / max|ds|) * ds is written as a multiply and then an add in
+ * flyvec/src/cu_special_reduction.cu:341-344, and that is what this file does.
+ * The reference is built with plain nvcc -O3, which is allowed to contract the
+ * two into one fused multiply-add; without nvcc its choice cannot be read
+ * off, so the binary's W may differ from this file's by one ulp per updated
+ * element and step.  No fixture of the reference settles it.
  */
 #include <math.h>
 #include <stdint.h>
