@@ -128,7 +128,8 @@ def gather_entry(kernel, nbytes, ms, counters, source):
     return out
 
 
-def bench_train(steps, warmup, cpu_seconds, c=TRAIN, which="step", dense_launches=0, separate_grouping=False):
+def bench_train(steps, warmup, cpu_seconds, c=TRAIN, which="step", dense_launches=0, separate_grouping=False,
+                graphs=False):
     from flyvec_amd import Trainer, synthetic
     tokens, offsets = synthetic.corpus(c["n_tokens"], c["V"], s=c["zipf_s"], mean_chunk=c["mean_chunk"])
     W0 = synthetic.synapses(c["K"], c["V"], seed=5)
@@ -159,6 +160,17 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, which="step", dense_launche
     # the same number of steps again, timed by two HIP events on the trainer's stream
     total_ms, _ = t.time_steps((warmup + steps) * c["B"], steps, eps, per_kernel=False)
     ev_ms_per_step = total_ms / steps
+    # and as HIP graphs (a graph per step, then one graph for all), on the windows that are left
+    graph = None
+    g_steps = min(steps, (nwin // c["B"] - warmup - 2 * steps) // 2)
+    if graphs and g_steps >= 5:
+        g0 = warmup + 2 * steps
+        per_step_ms = t.time_steps_graph(g0 * c["B"], g_steps, eps, 1) / g_steps
+        whole_ms = t.time_steps_graph((g0 + g_steps) * c["B"], g_steps, eps, g_steps) / g_steps
+        graph = {"steps": g_steps, "stream_launches_ms_per_step": ev_ms_per_step,
+                 "graph_per_step_ms_per_step": per_step_ms, "one_graph_ms_per_step": whole_ms,
+                 "note": "the same kernels with the same arguments captured into HIP graphs, instantiated before "
+                         "the clock starts; HIP events on the trainer's stream"}
     # per-kernel durations: each kernel of the last step launched back to back between two HIP
     # events on that stream (bracketing every kernel inside a step would add ~3 us of event
     # overhead to each); this destroys W, so it comes last
@@ -211,6 +223,8 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, which="step", dense_launche
         "step_byte_model": model,
         "n_windows": nwin,
     }
+    if graph:
+        out["hip_graph"] = graph
     if launches == 1:
         out["dense_launch_paths"] = {"knew_max_ds": known1 - known0, "made_the_pass": made1 - made0,
                                      "note": "timed steps whose single dense launch took max|ds| from the carried "
@@ -362,7 +376,7 @@ def train_line(c, tr, steps, warmup):
                                f"{tr['n_windows']} windows, lr 2e-4, fp32"},
     }
     for k in ("roofline", "step_roofline_frac", "step_byte_model", "event_ms_per_step", "kernels", "dense_launches",
-              "grouping_launch", "dense_launch_paths", "cpu_baseline"):
+              "grouping_launch", "dense_launch_paths", "hip_graph", "cpu_baseline"):
         if k in tr:
             line[k] = tr[k]
     return line
@@ -377,6 +391,7 @@ def main():
     ap.add_argument("--no-hash", action="store_true")
     ap.add_argument("--no-hash-host", action="store_true", help="skip the host-buffer hash timings (profiling runs: "
                     "their chunk launches would mix into the per-kernel means)")
+    ap.add_argument("--no-graph", action="store_true", help="skip the steps enqueued as HIP graphs")
     ap.add_argument("--no-large", action="store_true", help="skip the K=1000, V=50000 step")
     ap.add_argument("--no-epoch", action="store_true", help="skip the full epoch over 100 M tokens")
     ap.add_argument("--separate-grouping", action="store_true",
@@ -409,7 +424,7 @@ def main():
         print(json.dumps(line))
         return
     tr = bench_train(args.steps, args.warmup, args.cpu_seconds, TRAIN, "step", args.dense_launches,
-                     args.separate_grouping)
+                     args.separate_grouping, graphs=not args.no_graph)
     line = train_line(TRAIN, tr, args.steps, args.warmup)
     line["device"] = info["name"].strip()
     if not args.no_hash:

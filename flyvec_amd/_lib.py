@@ -93,6 +93,7 @@ SIGNATURES = {
     "fv_trainer_get_step_stats": [_vp, _vp, C.POINTER(_f32)],
     "fv_trainer_row_norms": [_vp, _u32, _vp],
     "fv_trainer_time_steps": [_vp, _u64, _u32, _f32, C.POINTER(_f32), C.POINTER(_f32)],
+    "fv_trainer_time_steps_graph": [_vp, _u64, _u32, _f32, _u32, C.POINTER(_f32)],
     "fv_trainer_time_kernel": [_vp, _u32, _u32, C.POINTER(_f32)],
     "fv_hasher_create": [_vp, _u32, _u64, _pp],
     "fv_hasher_destroy": [_vp],

@@ -2974,6 +2974,55 @@ extern "C" int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint3
   return rc;
 }
 
+// The same steps as fv_trainer_time_steps, enqueued as HIP graphs: the launches of steps_per_graph consecutive
+// steps are captured from the trainer's stream into one graph (every launch with the arguments it would have
+// had), all graphs are instantiated first, and the timed region holds their launches only. The steps train
+// like any others. No launch of a whole step is a memset, so the graphs hold kernel nodes only.
+extern "C" int fv_trainer_time_steps_graph(fv_trainer *t, uint64_t first_window, uint32_t n_steps, float eps,
+                                           uint32_t steps_per_graph, float *out_total_ms) {
+  FV_REQUIRE(t && out_total_ms, FV_ERR_INVALID, "null argument");
+  FV_REQUIRE(n_steps >= 1 && steps_per_graph >= 1, FV_ERR_INVALID, "n_steps and steps_per_graph must be >= 1");
+  FV_TRY(fv_check_step(t, first_window, t->B));
+  FV_REQUIRE(first_window + (uint64_t)n_steps * t->B <= t->n_windows, FV_ERR_INVALID,
+             "%u steps of %u windows from %llu exceed the %llu available", n_steps, t->B,
+             (unsigned long long)first_window, (unsigned long long)t->n_windows);
+  FV_HIP(hipStreamSynchronize(t->stream));
+  std::vector<hipGraphExec_t> execs;
+  int rc = FV_OK;
+  hipError_t e = hipSuccess;
+  for (uint32_t s = 0; s < n_steps && rc == FV_OK && e == hipSuccess; s += steps_per_graph) {
+    const uint32_t last = s + steps_per_graph < n_steps ? s + steps_per_graph : n_steps;
+    hipGraph_t graph = nullptr;
+    e = hipStreamBeginCapture(t->stream, hipStreamCaptureModeRelaxed);
+    if (e != hipSuccess) break;
+    for (uint32_t i = s; i < last && rc == FV_OK; ++i)
+      rc = fv_enqueue_step(t, first_window + (uint64_t)i * t->B, t->B, eps, 0.0f, nullptr);
+    e = hipStreamEndCapture(t->stream, &graph);
+    if (e == hipSuccess && rc == FV_OK) {
+      hipGraphExec_t exec = nullptr;
+      e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+      if (e == hipSuccess) execs.push_back(exec);
+    }
+    if (graph) (void)hipGraphDestroy(graph);
+  }
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (rc == FV_OK && e == hipSuccess) e = hipEventCreate(&e0);
+  if (rc == FV_OK && e == hipSuccess) e = hipEventCreate(&e1);
+  if (rc == FV_OK && e == hipSuccess) {
+    e = hipEventRecord(e0, t->stream);
+    for (size_t i = 0; i < execs.size() && e == hipSuccess; ++i) e = hipGraphLaunch(execs[i], t->stream);
+    if (e == hipSuccess) e = hipEventRecord(e1, t->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(t->stream);
+    if (e == hipSuccess) e = hipEventElapsedTime(out_total_ms, e0, e1);
+  }
+  for (hipGraphExec_t x : execs) (void)hipGraphExecDestroy(x);
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  if (rc != FV_OK) return rc;
+  if (e != hipSuccess) return fv_fail(FV_ERR_HIP, "steps as graphs failed: %s", hipGetErrorString(e));
+  return FV_OK;
+}
+
 extern "C" int fv_trainer_time_kernel(fv_trainer *t, uint32_t kernel_index, uint32_t reps, float *out_mean_ms) {
   FV_REQUIRE(t && out_mean_ms, FV_ERR_INVALID, "null argument");
   FV_REQUIRE(kernel_index < FV_TRAIN_KERNELS && reps >= 1, FV_ERR_INVALID, "bad kernel index or repetition count");

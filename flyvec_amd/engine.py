@@ -219,6 +219,12 @@ class Trainer:
                                              C.byref(total), kern if per_kernel else None))
         return total.value, dict(zip(_lib.TRAIN_KERNEL_NAMES, list(kern))) if per_kernel else None
 
+    def time_steps_graph(self, first_window, n_steps, eps, steps_per_graph=1):
+        """The same steps enqueued as HIP graphs of `steps_per_graph` steps each; milliseconds for all."""
+        total = C.c_float(0)
+        check(self.lib.fv_trainer_time_steps_graph(self.handle, int(first_window), int(n_steps), float(eps),
+                                                   int(steps_per_graph), C.byref(total)))
+        return total.value
 
     def _time_kernel(self, index, reps):
         ms = C.c_float(0)

@@ -244,6 +244,13 @@ int fv_trainer_row_norms(fv_trainer *t, uint32_t n_rows, double *out_norms);
 int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint32_t n_steps, float eps,
                           float *out_total_ms, float *out_kernel_ms);
 
+/* Measurement: the same n_steps minibatches enqueued as HIP graphs. The launches of steps_per_graph
+ * consecutive steps are captured from the trainer's stream into one graph, each with the arguments an
+ * ordinary step would give it; all graphs are instantiated before the clock starts, and out_total_ms covers
+ * their launches. The steps train like any others (same bits in W). No counterpart in the reference. */
+int fv_trainer_time_steps_graph(fv_trainer *t, uint64_t first_window, uint32_t n_steps, float eps,
+                                uint32_t steps_per_graph, float *out_total_ms);
+
 /* Measurement: launches kernel `kernel_index` (0 .. FV_TRAIN_KERNELS-1) of the last step `reps`
  * times back to back on its buffers and returns the mean duration between two HIP events on the
  * trainer's stream. The kernels that write W are not idempotent: the matrix is left in a state

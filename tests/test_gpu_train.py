@@ -225,6 +225,30 @@ def test_timing_hooks(gpu, launches):
     t.close()
 
 
+@pytest.mark.parametrize("launches,per_graph", [(1, 1), (1, 4), (2, 3)])
+def test_steps_enqueued_as_graphs_train_like_any_others(gpu, launches, per_graph):
+    """Seven steps from HIP graphs (the last graph shorter than the others), steps launched the ordinary way
+    before and after them: the matrix is the one that ordinary steps alone leave."""
+    from flyvec_amd import synthetic
+    V, K, w, B = 300, 64, 11, 256
+    tokens, offsets = small_corpus(30000, V)
+    W0 = synthetic.synapses(K, V, sigma=0.02)
+    t, _ = make_trainer(tokens, offsets, V, K, w, B, W0, launches=launches)
+    for s in range(12):
+        t.step(s * B, B, 1e-3)
+    want = t.get_weights()
+    t.set_weights(W0)
+    for s in range(2):
+        t.step(s * B, B, 1e-3)
+    assert t.time_steps_graph(2 * B, 7, 1e-3, per_graph) > 0
+    for s in range(9, 12):
+        t.step(s * B, B, 1e-3)
+    got = t.get_weights()
+    assert t.dense_launches == launches
+    t.close()
+    assert np.array_equal(got, want)
+
+
 def test_partial_last_batch_and_epoch_driver(gpu, oracle_lib):
     from flyvec_amd import synthetic
     to = oracle_lib
