@@ -104,6 +104,11 @@ struct fv_trainer {
   uint32_t *order;  // B window ids grouped by winner, ascending inside a group
   uint32_t *group_base, *group_count;  // K each
   fv_slot *slots;   // FV_NB_CLASSES regions of B x w slot records
+  // a region of slot_region records for every block of the sparse launch that groups for itself (0: none, the
+  // blocks share the class regions of slots[])
+  fv_slot *slots_blocks;
+  uint32_t slot_region;
+  bool no_block_regions;  // fv_trainer_set_slot_regions(0): the class regions are used all the same
   uint32_t *slot_count;  // K * FV_NB_CLASSES
   float *xx;        // ldk
   float *bmax;      // max|ds| of each block of the absmax launch, then of each block of the sparse launch
@@ -706,6 +711,10 @@ struct fv_sparse_args {
   float *Wt;
   fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records
   uint64_t slot_stride;
+  // Not 0 (grouping form only): every block has a region of slot_region records of its own in slots[], at
+  // blockIdx * slot_region, and a sentinel names a record by its place in the block's region. A block has no
+  // more records than its class has columns, so no block needs to know what the others write.
+  uint32_t slot_region;
   const float *xx;
   const float *invf;
   float *bmax_sparse;    // one maximum of |ds| per block
@@ -748,6 +757,7 @@ struct fv_sparse_args {
 // class in the top bits and the column of the class below, one subtraction and one comparison tell
 // whether an entry is this block's: of class q, inside [lo, lo + span), not masked, not padding.
 #define FV_SP_WPS (FV_SP_THREADS / 4)  // windows the block takes per step
+#define FV_SLOT_REGIONS_MAX_BYTES (1ull << 30)  // most memory spent on slot regions per block
 template <bool NARROW>
 __device__ __forceinline__ void fv_sparse_count_entry(uint32_t *cnt, int32_t iv, uint32_t drop, uint32_t origin,
                                                       uint32_t span) {
@@ -834,6 +844,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT;
   const uint32_t q = blockIdx.x & (FV_NB_CLASSES - 1);
   const uint32_t tid = threadIdx.x;
+  __shared__ uint32_t red2[GROUPING ? 17 : 1];
   uint32_t c_h, base, my_off = 0, r0 = 0;
   bool sc_complete = true;  // every thread's matches have their activations in pf[]
   uint64_t mask = 0;
@@ -845,26 +856,6 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     r0 = 64 * tid;
     uint2 mw = make_uint2(0u, 0u);
     if (2 * tid < a.won_words) mw = *(const uint2 *)(a.won + (uint64_t)h * a.won_words + 2 * tid);
-    // Windows won by lower neurons: 16-byte pieces of the 16-bit winner array dealt over the threads,
-    // two winners compared per operation (winner - h is negative in a 16-bit half exactly where the
-    // winner is lower; both are below 2^15). The entries behind the step's last window, up to the
-    // end of its piece, hold 0x7fff.
-    const uint32_t n8 = (n + 7) / 8;
-    const fv_short2 hh = {(short)h, (short)h};
-    fv_short2 below = {0, 0};
-#pragma unroll
-    for (int g = 0; g < 8; ++g) {  // n <= 8 * 8 * T
-      if (g * T < n8) {            // the same answer in the whole block
-        const uint32_t i4 = tid + g * T;
-        int4 v = ((const int4 *)a.win)[min(i4, n8 - 1)];
-        if (i4 >= n8) v = make_int4(0x7fff7fff, 0x7fff7fff, 0x7fff7fff, 0x7fff7fff);
-        below += (__builtin_bit_cast(fv_short2, v.x) - hh) >> 15;
-        below += (__builtin_bit_cast(fv_short2, v.y) - hh) >> 15;
-        below += (__builtin_bit_cast(fv_short2, v.z) - hh) >> 15;
-        below += (__builtin_bit_cast(fv_short2, v.w) - hh) >> 15;
-      }
-    }
-    const uint32_t lt = (uint32_t)(-((int)below.x + (int)below.y));
     mask = (uint64_t)mw.x | ((uint64_t)mw.y << 32);
     const uint32_t eq = (uint32_t)__popcll(mask);
     if (q == 0) {
@@ -878,11 +869,10 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       pf[e] = a.sc[min(r, n - 1)];
       mm &= mm - 1;
     }
-    // one block scan carries both counts as the halves of a word, and tells whether any thread has
-    // more matches than it has fetched activations for
+    // one block scan gives the ranks and the neuron's count, and tells whether any thread has more matches
+    // than it has fetched activations for
     const bool wave_more = __ballot(eq > (uint32_t)PF) != 0ull;
-    const uint32_t v = lt | (eq << 16);
-    const uint32_t incl = fv_wave_inclusive_scan_u32(v);
+    const uint32_t incl = fv_wave_inclusive_scan_u32(eq);
     if ((tid & 63u) == 63u) red[tid >> 6] = incl, red[8 + (tid >> 6)] = wave_more;
     fv_lds_barrier();
     uint32_t before = 0, total = 0;
@@ -894,14 +884,37 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       total += t;
       more = more || red[8 + i] != 0;
     }
-    before += incl - v;
-    base = total & 0xffffu;
-    c_h = total >> 16;
-    my_off = before >> 16;
+    c_h = total;
+    my_off = before + incl - eq;
     sc_complete = !more;
+    base = 0;
+    if (c_h != 0 && (a.slot_region == 0 || c_h > FV_SP_STAGE)) {
+      // The number of windows won by lower neurons is the neuron's place in order[] (more windows than LDS
+      // stages go through there) and in a class's slot region (where the blocks have no regions of their
+      // own). It is counted in the 16-bit winner array: 16-byte pieces dealt over the threads, two winners
+      // compared per operation (winner - h is negative in a 16-bit half exactly where the winner is lower;
+      // both are below 2^15). The entries behind the step's last window, up to the end of its piece, hold
+      // 0x7fff.
+      const uint32_t n8 = (n + 7) / 8;
+      const fv_short2 hh = {(short)h, (short)h};
+      fv_short2 below = {0, 0};
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {  // n <= 8 * 8 * T
+        if (g * T < n8) {            // the same answer in the whole block
+          const uint32_t i4 = tid + g * T;
+          int4 v = ((const int4 *)a.win)[min(i4, n8 - 1)];
+          if (i4 >= n8) v = make_int4(0x7fff7fff, 0x7fff7fff, 0x7fff7fff, 0x7fff7fff);
+          below += (__builtin_bit_cast(fv_short2, v.x) - hh) >> 15;
+          below += (__builtin_bit_cast(fv_short2, v.y) - hh) >> 15;
+          below += (__builtin_bit_cast(fv_short2, v.z) - hh) >> 15;
+          below += (__builtin_bit_cast(fv_short2, v.w) - hh) >> 15;
+        }
+      }
+      base = fv_block_sum_u32((uint32_t)(-((int)below.x + (int)below.y)), red2);
+    }
     for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
     if (q == 0 && tid == 0) {
-      a.group_base_out[h] = base;
+      a.group_base_out[h] = base;  // used where it was counted
       a.group_count_out[h] = c_h;
       if (c_h == 0) a.xx_out[h] = 0.0f;
     }
@@ -932,7 +945,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   const uint32_t n_cols = 2 * a.V;
   const uint32_t m_ent = max(c_h, c2_h) * a.w;
   // the block's records: no more than (c_h + c2_h) * w of them, behind those of the lower neurons
-  const uint64_t slot_first = (uint64_t)q * a.slot_stride + (uint64_t)(base + base2) * a.w;
+  const bool regions = GROUPING && a.slot_region != 0;
+  const uint64_t slot_first = regions ? (uint64_t)blockIdx.x * a.slot_region
+                                      : (uint64_t)q * a.slot_stride + (uint64_t)(base + base2) * a.w;
   fv_slot *slots = a.slots + slot_first;
 
   const bool staged_once = !DELTA && c_h <= FV_SP_STAGE;  // the usual case: the neuron's window ids are staged here
@@ -1126,7 +1141,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       // xx == 0 has ds == 0)
       // number of the round's first record, for the sentinels (saturated: a step with more records than a
       // sentinel can name is not finished by the launch that reads the numbers)
-      const uint32_t record0 = (uint32_t)min(slot_first + emitted, (uint64_t)FV_SENTINEL_MAX);
+      const uint32_t record0 = (uint32_t)min((regions ? 0ull : slot_first) + emitted, (uint64_t)FV_SENTINEL_MAX);
       // the row's two largest weights: the same address in the whole block, fetched where they are used
       const float2 top2 = a.top2_known ? a.row_top2[h] : make_float2(0.0f, 0.0f);
       for (uint32_t eb = tid; eb < take; eb += 4 * T) {
@@ -1241,6 +1256,7 @@ struct fv_dense_args {
   // thread keeps the same four neurons in every round
   uint32_t n_rows, active;
   uint32_t n_slots;  // records the slot regions hold (what a sentinel can name)
+  uint32_t slot_region;  // not 0: records per block of the sparse launch, which has a region of its own (fv_sparse_args)
   // the two largest |W[h][i]| of every row before this step (v1 >= v2), when known, and for every block of
   // the sparse launch how many of its elements hold them (fv_sparse_args.row_hits)
   const float2 *row_top2;
@@ -1536,11 +1552,16 @@ __device__ __forceinline__ void fv_top2_insert_lds(uint32_t *s1, uint32_t *s2, u
 template <bool DELTA>
 __device__ __forceinline__ void fv_finish_sparse_element(const fv_dense_args &a, uint32_t bits, uint32_t p, float s,
                                                          bool ok, const float *xs, uint32_t *sp1, uint32_t *sp2) {
-  const uint32_t at = (bits & FV_SENTINEL_MAX) - 1u;
-  if (at >= a.n_slots) return;  // a NaN of another origin stays what it is
+  const uint32_t number = (bits & FV_SENTINEL_MAX) - 1u;
+  if (number >= a.n_slots) return;  // a NaN of another origin stays what it is
+  const uint32_t col = p / a.ldk, h = p - col * a.ldk;
+  // the sentinel's number counts from the start of the slots, or of the region of the sparse launch's block
+  // that owns the element
+  const uint64_t at = a.slot_region
+                          ? (uint64_t)((h << FV_NB_CLASS_SHIFT) | (col & (FV_NB_CLASSES - 1))) * a.slot_region + number
+                          : number;
   const fv_slot sl = a.slots[at];
   if (sl.p != p) return;
-  const uint32_t h = p % a.ldk;
   const float x = xs[h];
   float out = sl.wv;
   if (ok && x != 0.0f) {
@@ -1863,7 +1884,8 @@ __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
   }
   float m1 = 0.0f, m2 = 0.0f;
   const uint64_t slot_first =
-      (uint64_t)q * a.slot_stride + (uint64_t)(a.group_base[h] + (DELTA ? a.group_base2[h] : 0u)) * a.w;
+      a.slot_region ? (uint64_t)blockIdx.x * a.slot_region
+                    : (uint64_t)q * a.slot_stride + (uint64_t)(a.group_base[h] + (DELTA ? a.group_base2[h] : 0u)) * a.w;
   const fv_slot *slots = a.slots + slot_first;
   const float x = a.xx[h];
   const float nc = a.scalars[0];
@@ -2006,6 +2028,7 @@ extern "C" int fv_trainer_destroy(fv_trainer *t) {
   (void)hipFree(t->idx);
   (void)hipFree(t->idx_ahead);
   (void)hipFree(t->slots);
+  (void)hipFree(t->slots_blocks);
   (void)hipFree(t->slot_count);
   (void)hipFree(t->order);
   (void)hipFree(t->group_base);
@@ -2088,6 +2111,15 @@ static int fv_trainer_alloc(fv_trainer *t) {
     FV_HIP(hipMalloc((void **)&t->won[0], 2 * row_words * sizeof(uint32_t)));
     t->won[1] = t->won[0] + row_words;
     FV_HIP(hipMemsetAsync(t->won[0], 0, 2 * row_words * sizeof(uint32_t), t->stream));
+    // A block of that launch writes no more records than its class has columns, nor more than the step has
+    // window positions: with that much room of its own per block, no block has to count the windows of the
+    // neurons before it to find its place. Left out where the regions would take more than a gigabyte.
+    const uint64_t class_cols = (t->N + FV_NB_CLASSES - 1) / FV_NB_CLASSES, positions = (uint64_t)t->B * t->w;
+    const uint64_t region = class_cols < positions ? class_cols : positions;
+    if (region * t->K * FV_NB_CLASSES * sizeof(fv_slot) <= FV_SLOT_REGIONS_MAX_BYTES && region + 1 < FV_SENTINEL_MAX) {
+      t->slot_region = (uint32_t)region;
+      FV_HIP(hipMalloc((void **)&t->slots_blocks, region * t->K * FV_NB_CLASSES * sizeof(fv_slot)));
+    }
   }
   FV_HIP(hipMalloc((void **)&t->scalars, 16 * sizeof(float)));
   FV_HIP(hipMemsetAsync(t->Wt, 0, elems * sizeof(float), t->stream));
@@ -2467,8 +2499,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   const bool whole = which == 0x3f;
   // records the slot regions of this step hold; the single dense launch finds a record through the number in
   // its sentinel, so it is only taken when every record number fits one
-  const uint64_t n_slots = (uint64_t)FV_NB_CLASSES * t->B * t->w * (anti ? 2 : 1);
-  const bool onepass = t->onepass && fv_trainers_alive.load() == 1 && n_slots + 1 < FV_SENTINEL_MAX;
+  uint64_t n_slots = (uint64_t)FV_NB_CLASSES * t->B * t->w * (anti ? 2 : 1);
   // the rows' two largest weights are in hand if the last write of the matrix was a single dense launch
   const bool top2_known = whole ? t->top2_valid : t->last_top2_known;
   if (whole) t->last_top2_known = top2_known;
@@ -2513,6 +2544,11 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   const bool grouping_in_sparse =
       which == 0x3f ? !anti && t->won[0] && !t->separate_grouping : t->last_grouped_in_sparse;
   if (which == 0x3f) t->last_grouped_in_sparse = grouping_in_sparse;
+  // the blocks of a sparse launch that groups for itself write their records to regions of their own, where
+  // the trainer has them, and a sentinel names a record inside its block's region
+  const uint32_t slot_region = grouping_in_sparse && !t->no_block_regions ? t->slot_region : 0u;
+  if (slot_region) n_slots = slot_region;
+  const bool onepass = t->onepass && fv_trainers_alive.load() == 1 && n_slots + 1 < FV_SENTINEL_MAX;
   g.won = nullptr;
   g.won_words = t->won_words;
   if (grouping_in_sparse) {
@@ -2583,7 +2619,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.group_count = t->group_count;
   sp.idx = t->idx;
   sp.Wt = t->Wt;
-  sp.slots = anti ? t->slots2 : t->slots;
+  sp.slots = anti ? t->slots2 : slot_region ? t->slots_blocks : t->slots;
+  sp.slot_region = slot_region;
   sp.slot_stride = (uint64_t)t->B * t->w * (anti ? 2 : 1);
   sp.order2 = t->order2;
   sp.group_base2 = t->group_base2;
@@ -2628,7 +2665,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.Wt4 = (float4 *)t->Wt;
   d.xx = t->xx;
   d.invf = t->invf;
-  d.slots = anti ? t->slots2 : t->slots;
+  d.slots = anti ? t->slots2 : slot_region ? t->slots_blocks : t->slots;
+  d.slot_region = slot_region;
   d.slot_count = t->slot_count;
   d.group_base = t->group_base;
   d.group_base2 = t->group_base2;
@@ -2862,6 +2900,12 @@ extern "C" int fv_trainer_set_grouping_launch(fv_trainer *t, uint32_t separate) 
   return FV_OK;
 }
 
+extern "C" int fv_trainer_set_slot_regions(fv_trainer *t, uint32_t per_block) {
+  FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
+  t->no_block_regions = per_block == 0;
+  return FV_OK;
+}
+
 extern "C" int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate) {
   FV_REQUIRE(t && out_separate, FV_ERR_INVALID, "null argument");
   *out_separate = (t->won[0] && !t->separate_grouping) ? 0u : 1u;
@@ -2870,7 +2914,9 @@ extern "C" int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separ
 
 extern "C" int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches) {
   FV_REQUIRE(t && out_launches, FV_ERR_INVALID, "null argument");
-  const uint64_t n_slots = (uint64_t)FV_NB_CLASSES * t->B * t->w;  // of a step without the anti-Hebbian term
+  // what a sentinel has to number in a step without the anti-Hebbian term
+  const bool regions = t->won[0] && !t->separate_grouping && t->slot_region && !t->no_block_regions;
+  const uint64_t n_slots = regions ? t->slot_region : (uint64_t)FV_NB_CLASSES * t->B * t->w;
   *out_launches = t->onepass && fv_trainers_alive.load() == 1 && n_slots + 1 < FV_SENTINEL_MAX ? 1u : 2u;
   return FV_OK;
 }

@@ -172,6 +172,12 @@ class Trainer:
         sparse-element launch where the step allows it.  Same results either way."""
         check(self.lib.fv_trainer_set_grouping_launch(self.handle, 1 if separate else 0))
 
+    def set_slot_regions(self, per_block):
+        """True (the default): every block of the sparse-element launch that groups for itself keeps its
+        records in room of its own; False: in its class's region, behind the lower neurons' records.
+        Same results either way."""
+        check(self.lib.fv_trainer_set_slot_regions(self.handle, 1 if per_block else 0))
+
     @property
     def grouping_launch(self):
         """True when a step without the anti-Hebbian term groups in a launch of its own."""

@@ -219,7 +219,15 @@ int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches); /* 1 o
  * windows and the step has no anti-Hebbian term, as a launch of its own otherwise. separate = 1 forces the launch of its
  * own, 0 returns to that rule. Results are bit-identical either way. */
 int fv_trainer_set_grouping_launch(fv_trainer *t, uint32_t separate);
-int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate); /* the form a step without the anti-Hebbian term takes */
+int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate);
+/* Where the sparse-element launch that groups for itself keeps a step's records of sparse elements (the
+ * weight, count and 1/frequency of each element the minibatch touches: the sparse operand of
+ * flyvec/src/cuda_funcs.cu:657-672). per_block = 1, the default: every block of that launch has room of its own
+ * for as many records as its class has columns (or the minibatch positions, if fewer), where that takes no more
+ * than a gigabyte in all, so no block has to count the windows of the neurons before it; per_block = 0: the
+ * blocks share one region per class, each behind the records of the neurons before it, as the other launch
+ * forms do. Results are bit-identical either way. No counterpart in the reference. */
+int fv_trainer_set_slot_regions(fv_trainer *t, uint32_t per_block); /* the form a step without the anti-Hebbian term takes */
 /* Test hook: between its two passes a single-launch dense pass waits for all its blocks, at most
  * `rounds` polling rounds (2^14 by default, tens of milliseconds); 0 makes every block give up at once, which
  * is how the error path of fv_trainer_sync is exercised. No counterpart in the reference. */

@@ -836,6 +836,7 @@ def test_random_configurations_match_the_oracle(gpu, oracle_lib, case):
                     prune_duplicates=c["prune"])
         t.set_dense_launches(c["launches"])
         t.set_grouping_launch(separate)
+        t.set_slot_regions(case % 2 == 0)  # odd cases: the blocks of the launch that groups for itself share class regions
         t.set_corpus(tokens, offsets)
         t.set_permutation(perm)
         t.set_weights(W0)
@@ -849,6 +850,39 @@ def test_random_configurations_match_the_oracle(gpu, oracle_lib, case):
         Wg = t.get_weights()
         t.close()
         assert np.array_equal(Wg.view(np.uint32), Wo.view(np.uint32)), f"W, separate grouping {separate}, {c}"
+
+
+@pytest.mark.parametrize("launches", [1, 2])
+@pytest.mark.parametrize("per_block", [True, False])
+def test_slot_records_per_block_or_per_class(gpu, oracle_lib, launches, per_block):
+    """The records of a step's sparse elements in a region per block of the sparse launch, or in one region per
+    class behind the lower neurons' records: three steps against the checker, with one neuron winning most windows
+    (its records are many) and most neurons winning none."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    V, K, w, B = 500, 70, 7, 3000
+    tokens, offsets = small_corpus(60000, V, seed=4)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    perm = np.random.default_rng(5).permutation(len(starts)).astype(np.uint64)
+    W0 = synthetic.synapses(K, V, seed=3, sigma=0.02)
+    W0[11] += 0.05  # neuron 11 wins nearly everything
+    Wo = W0.copy()
+    t = Trainer(V, K, w, B, initial_learning_rate=1e-3)
+    t.set_dense_launches(launches)
+    t.set_slot_regions(per_block)
+    t.set_corpus(tokens, offsets)
+    t.set_permutation(perm)
+    t.set_weights(W0)
+    for s in range(3):
+        ref = to.train_step(Wo, to.inflate(tokens, starts, perm, s * B, B, w, V), invf, 1e-3)
+        t.step(s * B, B, 1e-3)
+        assert np.array_equal(t.winners(B), ref["winners"])
+        assert np.bincount(ref["winners"], minlength=K)[11] > B // 2
+        xx, nc = t.step_stats()
+        assert np.array_equal(xx, ref["xx"]) and nc == ref["nc"]
+    Wg = t.get_weights()
+    t.close()
+    assert np.array_equal(Wg.view(np.uint32), Wo.view(np.uint32))
 
 
 @pytest.mark.parametrize("launches", [1, 2])
