@@ -396,8 +396,9 @@ def main():
     ap.add_argument("--no-epoch", action="store_true", help="skip the full epoch over 100 M tokens")
     ap.add_argument("--separate-grouping", action="store_true",
                     help="group the windows by winner in a launch of its own (the default does it inside the sparse launch)")
-    ap.add_argument("--dense-launches", type=int, choices=[0, 1, 2], default=0,
-                    help="the passes over W of a step as one launch (1), two (2), or as the library chooses (0)")
+    ap.add_argument("--dense-launches", type=int, choices=[0, 1, 2, 3], default=0,
+                    help="the passes over W of a step as one launch (1; 3: its streaming form), separate launches (2), or as the "
+                         "library chooses (0)")
     ap.add_argument("--workload", choices=["all", "step", "large-step", "epoch"], default="all",
                     help="all: the headline step with the hash batch, the large step and the epoch as sub-objects "
                          "(default); step / large-step / epoch: that workload alone as the line")

@@ -126,6 +126,8 @@ struct fv_trainer {
   unsigned onepass_blocks, onepass_unroll;
   unsigned onepass_active;  // threads of a block of that launch that own elements (a multiple of ldk / 4)
   bool onepass;  // in use (fv_trainer_set_dense_launches)
+  // the same launch with the rows streamed through the registers (any matrix size): available, in use
+  bool stream_ok, onepass_stream;
   // The two largest |W| of every row, kept by the single dense launch so that it knows max|ds| without
   // a pass over the matrix: each block's share after a launch (top2_part), merged by the next step's
   // winner kernel (row_top2); what the sparse launch reports on them (row_hits); whether top2_part
@@ -1607,6 +1609,73 @@ __device__ __forceinline__ uint32_t fv_onepass_decide(unsigned long long *word, 
   return (uint32_t)old;
 }
 
+// Between the pass for the maximum and the update of a single dense launch: the block publishes its maximum m
+// of |ds|, its first wave waits (bounded) for the launch's decision, and its first thread leaves the step's scale
+// in *sh_s and whether the update goes ahead in *sh_ok (read behind the caller's next barrier).
+__device__ __forceinline__ void fv_onepass_exchange(const fv_dense_args &a, float m, uint32_t limit, bool dead,
+                                                    float *smem16, float *sh_s_out, uint32_t *sh_ok_out) {
+  constexpr uint32_t T = FV_ONEPASS_THREADS;
+  const uint32_t tid = threadIdx.x;
+  float &sh_s = *sh_s_out;
+  uint32_t &sh_ok = *sh_ok_out;
+  // the block's maximum, needed by its first wave only: one barrier
+  {
+    const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
+    if ((tid & 63) == 0) smem16[tid >> 6] = __uint_as_float(wm);
+  }
+  __syncthreads();
+  if (tid < 64) {
+    float bm = tid < T / 64 ? smem16[tid] : 0.0f;
+    bm = __uint_as_float(fv_wave_max_u32(__float_as_uint(bm)));
+    if (tid == 0)
+      __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | __float_as_uint(bm),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // Block 0 waits for every block's word and decides; the others wait for the decision. Both waits are
+    // bounded, and a block that gives up decides "abandoned" unless the decision has already been made.
+    unsigned long long *decision = a.arrive + gridDim.x;
+    uint32_t verdict = FV_ONEPASS_ABANDONED;
+    bool decided = false;
+    if (blockIdx.x == 0) {
+      uint32_t mx = 0;
+      bool done = false;
+      for (uint32_t spin = 0; spin < limit && !done; ++spin) {
+        bool all = true;
+        mx = 0;
+        for (uint32_t i = tid; i < gridDim.x; i += 64) {
+          const unsigned long long v = __hip_atomic_load(&a.arrive[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          all = all && (uint32_t)(v >> 32) == a.epoch;
+          mx = max(mx, (uint32_t)v);  // non-negative floats order like their bit patterns
+        }
+        done = __all(all);
+        if (!done) __builtin_amdgcn_s_sleep(2);
+      }
+      mx = fv_wave_max_u32(mx);
+      if (done) verdict = mx;
+    } else {
+      for (uint32_t spin = 0; spin < limit && !decided; ++spin) {
+        const unsigned long long v = __hip_atomic_load(decision, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        decided = (uint32_t)(v >> 32) == a.epoch;
+        if (decided) verdict = (uint32_t)v; else __builtin_amdgcn_s_sleep(2);
+      }
+    }
+    if (tid == 0) {
+      if (!decided) verdict = fv_onepass_decide(decision, a.epoch, verdict);
+      const bool go = verdict != FV_ONEPASS_ABANDONED;
+      const float nc = __uint_as_float(verdict);
+      sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
+      sh_ok = go;
+      if (!go) {
+        if (!dead) *a.status = a.step_tag;  // the launches behind this one are dead and leave the word alone
+        a.scalars[0] = __uint_as_float(0x7fc00000u);
+        a.scalars[1] = 1.0f;
+      } else if (blockIdx.x == 0) {
+        a.scalars[0] = nc;
+        a.path_count[1] += 1;
+      }
+    }
+  }
+}
+
 static_assert(FV_MAX_HID <= 2 * FV_ONEPASS_THREADS, "two neurons per thread cover every row");
 static_assert(FV_NB_CLASSES == 4, "a neuron's block maxima and hit counts are read as one 16-byte word each");
 
@@ -1720,62 +1789,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
         w[u + DEPTH] = a.Wt4[(rown < a.n_rows ? rown : row_inside) * a.ldk4 + q];
       }
     }
-    // the block's maximum, needed by its first wave only: one barrier
-    {
-      const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
-      if ((tid & 63) == 0) smem16[tid >> 6] = __uint_as_float(wm);
-    }
-    __syncthreads();
-    if (tid < 64) {
-      float bm = tid < T / 64 ? smem16[tid] : 0.0f;
-      bm = __uint_as_float(fv_wave_max_u32(__float_as_uint(bm)));
-      if (tid == 0)
-        __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | __float_as_uint(bm),
-                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      // Block 0 waits for every block's word and decides; the others wait for the decision. Both waits are
-      // bounded, and a block that gives up decides "abandoned" unless the decision has already been made.
-      unsigned long long *decision = a.arrive + gridDim.x;
-      uint32_t verdict = FV_ONEPASS_ABANDONED;
-      bool decided = false;
-      if (blockIdx.x == 0) {
-        uint32_t mx = 0;
-        bool done = false;
-        for (uint32_t spin = 0; spin < limit && !done; ++spin) {
-          bool all = true;
-          mx = 0;
-          for (uint32_t i = tid; i < gridDim.x; i += 64) {
-            const unsigned long long v = __hip_atomic_load(&a.arrive[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            all = all && (uint32_t)(v >> 32) == a.epoch;
-            mx = max(mx, (uint32_t)v);  // non-negative floats order like their bit patterns
-          }
-          done = __all(all);
-          if (!done) __builtin_amdgcn_s_sleep(2);
-        }
-        mx = fv_wave_max_u32(mx);
-        if (done) verdict = mx;
-      } else {
-        for (uint32_t spin = 0; spin < limit && !decided; ++spin) {
-          const unsigned long long v = __hip_atomic_load(decision, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          decided = (uint32_t)(v >> 32) == a.epoch;
-          if (decided) verdict = (uint32_t)v; else __builtin_amdgcn_s_sleep(2);
-        }
-      }
-      if (tid == 0) {
-        if (!decided) verdict = fv_onepass_decide(decision, a.epoch, verdict);
-        const bool go = verdict != FV_ONEPASS_ABANDONED;
-        const float nc = __uint_as_float(verdict);
-        sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
-        sh_ok = go;
-        if (!go) {
-          if (!dead) *a.status = a.step_tag;  // the launches behind this one are dead and leave the word alone
-          a.scalars[0] = __uint_as_float(0x7fc00000u);
-          a.scalars[1] = 1.0f;
-        } else if (blockIdx.x == 0) {
-          a.scalars[0] = nc;
-          a.path_count[1] += 1;
-        }
-      }
-    }
+    fv_onepass_exchange(a, m, limit, dead, smem16, &sh_s, &sh_ok);
     fv_sample_ahead(a, samples0, e0, er0, start0, ahead_entries, TS);  // while the first wave waits
     __syncthreads();
     ok = sh_ok != 0;
@@ -1847,6 +1861,197 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
     }
     a.top2_part[(uint64_t)blockIdx.x * a.ldk + h] = make_float2(m1, m2);
   }
+}
+
+// The same launch for a matrix of any size: nothing is kept in registers between the passes, the block's rows
+// go through FV_STREAM_DEPTH 16-byte groups per thread in rounds. When max|ds| is known from the rows' largest
+// weights (the usual case) it is one streaming read-modify-write; otherwise the rows are streamed once for the
+// maximum, the blocks exchange their maxima as above, and the rows are streamed again for the update: the
+// traffic of the separate launches, without their launches. Rows, ownership of the sparse elements, the shares of
+// the rows' largest weights and the minibatch sampled ahead are those of fv_dense_onepass_kernel.
+#ifndef FV_STREAM_DEPTH
+#define FV_STREAM_DEPTH 2
+#endif
+#define FV_STREAM_HIT_CAP 8192  // sentinels a block notes in LDS (64 KB)
+
+template <bool DELTA>
+__global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_dense_args a) {
+  constexpr uint32_t T = FV_ONEPASS_THREADS;
+  constexpr int D = FV_STREAM_DEPTH;
+  extern __shared__ float4 dyn4[];
+  float *xs = (float *)dyn4;
+  uint32_t *sp1 = (uint32_t *)(xs + a.ldk);
+  uint32_t *sp2 = sp1 + a.ldk;
+  uint2 *hit_list = (uint2 *)(sp2 + a.ldk);
+  float2 *pairs = (float2 *)(hit_list + FV_STREAM_HIT_CAP);
+  __shared__ uint32_t red3[T / 64][3];
+  __shared__ float smem16[16];
+  __shared__ float sh_s;
+  __shared__ uint32_t sh_ok, sh_hits;
+  const uint32_t tid = threadIdx.x;
+  const bool active = tid < a.active;
+  const uint32_t q = tid % a.ldk4, r = tid / a.ldk4;
+  const uint32_t rows_per_round = a.active / a.ldk4;
+  const uint32_t row0 = blockIdx.x + gridDim.x * r;
+  const uint32_t row_step = gridDim.x * rows_per_round;
+  const uint32_t rounds = (a.n_rows + row_step - 1) / row_step;
+  const uint32_t row_inside = min(row0, a.n_rows - 1);
+  float xh[2];
+  float2 rm[2];
+  uint4 hit4[2];
+  float4 smx[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t h = min(tid + T * j, a.K - 1);
+    xh[j] = a.xx[min(tid + T * j, a.ldk - 1)];
+    rm[j] = a.row_top2[h];
+    hit4[j] = ((const uint4 *)a.row_hits)[h];
+    smx[j] = ((const float4 *)(a.bmax + a.sparse_base))[h];
+  }
+  const bool dead = a.scalars[1] != 0.0f;
+  const uint32_t limit = dead ? 0u : a.spin_limit;
+  float4 w[D];
+  auto group_of = [&](uint32_t row) { return (row < a.n_rows ? row : row_inside) * a.ldk4 + q; };
+#pragma unroll
+  for (int u = 0; u < D; ++u) w[u] = a.Wt4[group_of(row0 + u * row_step)];
+  constexpr uint32_t TS = T - 64;
+  const uint32_t ahead_entries = a.ahead_n * a.idx_stride;
+  const uint32_t e0 = blockIdx.x * TS + (tid - 64);
+  const bool samples0 = tid >= 64 && e0 < ahead_entries;
+  const uint32_t er0 = samples0 ? e0 / a.idx_stride : 0u;
+  const uint64_t start0 = a.ahead_n ? a.pstart[a.ahead_first + er0] : 0ull;
+
+  uint32_t S = 0, E = 0, F = 0;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint32_t h = tid + T * j;
+    if (h < a.ldk) {
+      xs[h] = xh[j];
+      sp1[h] = 0;
+      sp2[h] = 0;
+    }
+    if (h < a.K) fv_row_candidate(xh[j], rm[j], hit4[j], smx[j], S, E, F);
+  }
+  if (tid == 0) sh_hits = 0;
+  {
+    const uint32_t ws = fv_wave_max_u32(S), we = fv_wave_max_u32(E), wf = fv_wave_max_u32(F);
+    if ((tid & 63) == 0) {
+      red3[tid >> 6][0] = ws;
+      red3[tid >> 6][1] = we;
+      red3[tid >> 6][2] = wf;
+    }
+  }
+  __syncthreads();
+  S = E = F = 0;
+#pragma unroll
+  for (uint32_t i = 0; i < T / 64; ++i) {
+    S = max(S, red3[i][0]);
+    E = max(E, red3[i][1]);
+    F = max(F, red3[i][2]);
+  }
+  const bool fast = a.top2_known && F <= max(S, E);
+  const float4 xq = ((const float4 *)xs)[q];
+
+  float s;
+  bool ok = true;
+  if (fast) {
+    const float nc = __uint_as_float(max(S, E));
+    s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
+    ok = !dead;
+    if (blockIdx.x == 0 && tid == 0 && ok) {
+      a.scalars[0] = nc;
+      a.path_count[0] += 1;
+    }
+  } else {
+    float m = __uint_as_float(S);
+    for (uint32_t c = 0; c < rounds; c += D) {
+#pragma unroll
+      for (int u = 0; u < D; ++u) {
+        const uint32_t row = row0 + (c + u) * row_step;
+        if (active && row < a.n_rows) m = fv_absmax_four(m, xq, w[u]);
+        w[u] = a.Wt4[group_of(row + D * row_step)];
+      }
+    }
+    fv_onepass_exchange(a, m, limit, dead, smem16, &sh_s, &sh_ok);
+    fv_sample_ahead(a, samples0, e0, er0, start0, ahead_entries, TS);  // while the first wave waits
+    __syncthreads();
+    ok = sh_ok != 0;
+    s = sh_s;
+#pragma unroll
+    for (int u = 0; u < D; ++u) w[u] = a.Wt4[group_of(row0 + u * row_step)];  // the stream starts again
+  }
+
+  float t1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, t2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#define FV_STREAM_ELEMENT(member, lane4)                                                       \
+  if (v.member == v.member) {                                                                  \
+    if (changed) e[lane4] = v.member;                                                          \
+  } else {                                                                                     \
+    const uint32_t k = atomicAdd(&sh_hits, 1u);                                                \
+    if (k < FV_STREAM_HIT_CAP)                                                                 \
+      hit_list[k] = make_uint2(__float_as_uint(v.member), 4u * p4 + lane4);                    \
+    else                                                                                       \
+      fv_finish_sparse_element<DELTA>(a, __float_as_uint(v.member), 4u * p4 + lane4, s, ok, xs, sp1, sp2); \
+  }
+  for (uint32_t c = 0; c < rounds; c += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const uint32_t row = row0 + (c + u) * row_step;
+      if (active && row < a.n_rows) {
+        const uint32_t p4 = row * a.ldk4 + q;
+        float4 v = w[u];
+        const bool has_nan = __builtin_isunordered(v.x, v.y) || __builtin_isunordered(v.z, v.w);
+        const bool changed = ok && fv_apply_four(v, xq, s, a.update_cut);
+        if (!has_nan) {
+          if (changed) a.Wt4[p4] = v;
+        } else {
+          float *e = (float *)&a.Wt4[p4];
+          FV_STREAM_ELEMENT(x, 0)
+          FV_STREAM_ELEMENT(y, 1)
+          FV_STREAM_ELEMENT(z, 2)
+          FV_STREAM_ELEMENT(w, 3)
+        }
+        fv_top2_insert(t1[0], t2[0], fv_abs_or_zero(v.x));
+        fv_top2_insert(t1[1], t2[1], fv_abs_or_zero(v.y));
+        fv_top2_insert(t1[2], t2[2], fv_abs_or_zero(v.z));
+        fv_top2_insert(t1[3], t2[3], fv_abs_or_zero(v.w));
+      }
+      w[u] = a.Wt4[group_of(row + D * row_step)];  // the round that takes this one's place
+    }
+  }
+#undef FV_STREAM_ELEMENT
+  if (fast) fv_sample_ahead(a, samples0, e0, er0, start0, ahead_entries, TS);
+  if (active) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pairs[(e * rows_per_round + r) * a.ldk4 + q] = make_float2(t1[e], t2[e]);
+  }
+  __syncthreads();
+  const uint32_t n_hits = min(sh_hits, (uint32_t)FV_STREAM_HIT_CAP);
+  for (uint32_t i = tid; i < n_hits; i += T) {
+    const uint2 hit = hit_list[i];
+    fv_finish_sparse_element<DELTA>(a, hit.x, hit.y, s, ok, xs, sp1, sp2);
+  }
+  __syncthreads();
+  for (uint32_t h = tid; h < a.K; h += T) {
+    const uint32_t e = h & 3u, qq = h >> 2;
+    float m1 = __uint_as_float(sp1[h]), m2 = __uint_as_float(sp2[h]);
+    for (uint32_t rr = 0; rr < rows_per_round; ++rr) {
+      const float2 b = pairs[(e * rows_per_round + rr) * a.ldk4 + qq];
+      fv_top2_merge(m1, m2, b.x, b.y);
+    }
+    a.top2_part[(uint64_t)blockIdx.x * a.ldk + h] = make_float2(m1, m2);
+  }
+}
+
+static int fv_stream_fits(size_t smem) {
+  int nb = 0, nb2 = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fv_dense_stream_kernel<false>, FV_ONEPASS_THREADS, smem) !=
+          hipSuccess ||
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb2, fv_dense_stream_kernel<true>, FV_ONEPASS_THREADS, smem) !=
+          hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return nb >= 1 && nb2 >= 1;
 }
 
 template <int U, bool DELTA>
@@ -2064,7 +2269,7 @@ static int fv_trainer_alloc(fv_trainer *t) {
   const size_t idx_entries = (size_t)t->B * t->idx_stride + FV_IDX_PAD;
   FV_HIP(hipMalloc((void **)&t->idx, idx_entries * sizeof(int32_t)));
   FV_HIP(hipMemsetAsync(t->idx, 0xff, idx_entries * sizeof(int32_t), t->stream));
-  if (t->onepass_unroll) {
+  if (t->onepass_blocks) {
     FV_HIP(hipMalloc((void **)&t->idx_ahead, idx_entries * sizeof(int32_t)));
     FV_HIP(hipMemsetAsync(t->idx_ahead, 0xff, idx_entries * sizeof(int32_t), t->stream));
   }
@@ -2125,7 +2330,7 @@ static int fv_trainer_alloc(fv_trainer *t) {
   FV_HIP(hipMemsetAsync(t->Wt, 0, elems * sizeof(float), t->stream));
   FV_HIP(hipMemsetAsync(t->xx, 0, (size_t)t->ldk * sizeof(float), t->stream));
   FV_HIP(hipMemsetAsync(t->scalars, 0, 16 * sizeof(float), t->stream));
-  if (t->onepass_unroll) {
+  if (t->onepass_blocks) {
     FV_HIP(hipMalloc((void **)&t->arrive, ((size_t)t->onepass_blocks + 1) * sizeof(unsigned long long)));
     FV_HIP(hipMemsetAsync(t->arrive, 0, ((size_t)t->onepass_blocks + 1) * sizeof(unsigned long long), t->stream));
     FV_HIP(hipHostMalloc((void **)&t->onepass_status, sizeof(uint32_t), hipHostMallocDefault));
@@ -2143,8 +2348,14 @@ static size_t fv_onepass_smem(const fv_trainer *t) {
          (size_t)FV_ONEPASS_THREADS * 4 * sizeof(float2);
 }
 
+static size_t fv_stream_smem(const fv_trainer *t) {
+  return (size_t)t->ldk * 3 * sizeof(float) + (size_t)FV_STREAM_HIT_CAP * sizeof(uint2) +
+         (size_t)FV_ONEPASS_THREADS * 4 * sizeof(float2);
+}
+
 static void fv_choose_onepass(fv_trainer *t, uint64_t cu) {
   t->onepass_blocks = t->onepass_unroll = t->onepass_active = 0;
+  t->stream_ok = t->onepass_stream = t->onepass = false;
   t->onepass_spin_limit = FV_ONEPASS_SPIN_LIMIT;
   const uint32_t ldk4 = t->ldk / 4;
   if (ldk4 > FV_ONEPASS_THREADS) return;
@@ -2153,15 +2364,29 @@ static void fv_choose_onepass(fv_trainer *t, uint64_t cu) {
   uint64_t blocks = (t->N + rows_per_round - 1) / rows_per_round;
   if (blocks > cu * FV_ONEPASS_BLOCKS_PER_CU) blocks = cu * FV_ONEPASS_BLOCKS_PER_CU;
   const uint64_t need = (t->N + blocks * rows_per_round - 1) / (blocks * rows_per_round);
-  if (need > FV_ONEPASS_MAX_UNROLL) return;
-  const unsigned unroll = need <= 8 ? 8 : 16;
-  const size_t smem = fv_onepass_smem(t);
-  const int fits = unroll == 8 ? fv_onepass_fits<8>(smem) : fv_onepass_fits<16>(smem);
-  if (!fits) return;
+  {
+    // the streaming form: its sentinel list takes more LDS than a launch may have without asking
+    const size_t smem = fv_stream_smem(t);
+    if (hipFuncSetAttribute((const void *)fv_dense_stream_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) == hipSuccess &&
+        hipFuncSetAttribute((const void *)fv_dense_stream_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) == hipSuccess)
+      t->stream_ok = fv_stream_fits(smem) != 0;
+    else
+      (void)hipGetLastError();
+  }
+  unsigned unroll = 0;
+  if (need <= FV_ONEPASS_MAX_UNROLL) {
+    unroll = need <= 8 ? 8 : 16;
+    const size_t smem = fv_onepass_smem(t);
+    if (!(unroll == 8 ? fv_onepass_fits<8>(smem) : fv_onepass_fits<16>(smem))) unroll = 0;
+  }
+  if (!unroll && !t->stream_ok) return;
   t->onepass_blocks = (unsigned)blocks;
   t->onepass_unroll = unroll;
   t->onepass_active = rows_per_round * ldk4;
   t->onepass = true;
+  t->onepass_stream = unroll == 0;
 }
 
 extern "C" int fv_trainer_create(const fv_train_config *cfg, fv_trainer **out_trainer) {
@@ -2731,7 +2956,13 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
 #define FV_CASE(U)                                                                     \
   if (anti) fv_launch_onepass<U, true>(d, t->onepass_blocks, smem1, t->stream);        \
   else fv_launch_onepass<U, false>(d, t->onepass_blocks, smem1, t->stream);
-      if (t->onepass_unroll == 8) { FV_CASE(8) } else { FV_CASE(16) }
+      if (t->onepass_stream) {
+        const dim3 grid(t->onepass_blocks), block(FV_ONEPASS_THREADS);
+        if (anti)
+          hipLaunchKernelGGL(fv_dense_stream_kernel<true>, grid, block, fv_stream_smem(t), t->stream, d);
+        else
+          hipLaunchKernelGGL(fv_dense_stream_kernel<false>, grid, block, fv_stream_smem(t), t->stream, d);
+      } else if (t->onepass_unroll == 8) { FV_CASE(8) } else { FV_CASE(16) }
 #undef FV_CASE
       t->top2_valid = true;  // this launch leaves the shares of the matrix it writes
       t->top2_n_part = t->onepass_blocks;
@@ -2884,11 +3115,13 @@ extern "C" int fv_trainer_set_stale_tail(fv_trainer *t, uint32_t on) {
 
 extern "C" int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches) {
   FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
-  FV_REQUIRE(launches <= 2, FV_ERR_INVALID, "launches must be 0 (choose), 1 or 2");
-  FV_REQUIRE(launches != 1 || t->onepass_unroll, FV_ERR_INVALID,
-             "a %llu x %u matrix does not fit the registers of this device: the dense passes need two launches",
-             (unsigned long long)t->N, t->K);
-  t->onepass = launches == 2 ? false : t->onepass_unroll != 0;
+  FV_REQUIRE(launches <= 3, FV_ERR_INVALID, "launches must be 0 (choose), 1, 2 or 3 (one launch, rows streamed)");
+  FV_REQUIRE(launches != 1 || t->onepass_blocks, FV_ERR_INVALID,
+             "a row of %u neurons does not fit a block of this device: the dense passes need separate launches", t->K);
+  FV_REQUIRE(launches != 3 || t->stream_ok, FV_ERR_INVALID,
+             "the streaming dense launch does not fit this device: the dense passes need separate launches");
+  t->onepass = launches == 2 ? false : t->onepass_blocks != 0;
+  t->onepass_stream = launches == 3 || t->onepass_unroll == 0;
   FV_HIP(hipMemsetAsync(t->scalars + 1, 0, sizeof(float), t->stream));  // "a launch has given up"
   return FV_OK;
 }

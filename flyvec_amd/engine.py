@@ -163,8 +163,9 @@ class Trainer:
         return out.value
 
     def set_dense_launches(self, launches):
-        """1: both passes over the matrix in one launch (it must fit the device's registers),
-        2: two launches, 0: as chosen at creation.  Same results either way."""
+        """1: both passes over the matrix in one launch (kept in registers between them where it fits,
+        its rows streamed otherwise), 3: the streaming form whatever the size, 2: separate launches,
+        0: as chosen at creation.  Same results either way."""
         check(self.lib.fv_trainer_set_dense_launches(self.handle, int(launches)))
 
     def set_grouping_launch(self, separate):

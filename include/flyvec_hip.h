@@ -200,12 +200,14 @@ int fv_trainer_sync(fv_trainer *t);
 int fv_trainer_get_giveups_recovered(fv_trainer *t, uint64_t *out_count);
 
 /* The two passes over the matrix of a step (max|ds|, flyvec/src/cu_special_reduction.cu:241, and
- * the update, flyvec/src/cuda_funcs.cu:1787-1806) run as ONE launch when the matrix fits the registers of
- * the device (64 MiB on 256 compute units) and a step has fewer than 2^23 slot records, else as two.
- * launches = 1 or 2 forces the form (1 fails with FV_ERR_INVALID when the matrix does not fit),
- * 0 returns to the choice made at creation. Results are bit-identical either way. The single
+ * the update, flyvec/src/cuda_funcs.cu:1787-1806) run as ONE launch wherever a block of the device holds a row
+ * of the matrix (every hid this library takes) and a sentinel can number the step's slot records (fewer than 2^23): with
+ * the matrix kept in registers between the passes where it fits them (64 MiB on 256 compute units), with its
+ * rows streamed through the registers otherwise. launches = 1 asks for the single launch (FV_ERR_INVALID where
+ * there is none), 3 for its streaming form whatever the matrix size, 2 for separate launches (maximum, update,
+ * sparse elements), 0 returns to the choice made at creation. Results are bit-identical in all forms. The single
  * launch needs the whole device for itself, so while a process holds more than one trainer every
- * step takes two launches whatever is set here. */
+ * step takes separate launches whatever is set here. */
 int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches);
 /* The single launch carries the two largest |W| of every row from step to step; from them and from what
  * the sparse-element launch reports it usually knows max|ds| (flyvec/src/cu_special_reduction.cu:241) before
