@@ -128,6 +128,7 @@ struct fv_trainer {
   bool onepass;  // in use (fv_trainer_set_dense_launches)
   // the same launch with the rows streamed through the registers (any matrix size): available, in use
   bool stream_ok, onepass_stream;
+  uint32_t hit_cap_limit;  // fv_trainer_set_sentinel_list: 0, or fewer entries than the launches' LDS lists hold
   // The two largest |W| of every row, kept by the single dense launch so that it knows max|ds| without
   // a pass over the matrix: each block's share after a launch (top2_part), merged by the next step's
   // winner kernel (row_top2); what the sparse launch reports on them (row_hits); whether top2_part
@@ -1259,6 +1260,7 @@ struct fv_dense_args {
   uint32_t n_rows, active;
   uint32_t n_slots;  // records the slot regions hold (what a sentinel can name)
   uint32_t slot_region;  // not 0: records per block of the sparse launch, which has a region of its own (fv_sparse_args)
+  uint32_t hit_cap;      // sentinels a block of the single launch notes in its LDS list (no more than the list holds)
   // the two largest |W[h][i]| of every row before this step (v1 >= v2), when known, and for every block of
   // the sparse launch how many of its elements hold them (fv_sparse_args.row_hits)
   const float2 *row_top2;
@@ -1805,7 +1807,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
     if (changed) e[lane4] = v.member;                                                          \
   } else {                                                                                     \
     const uint32_t k = atomicAdd(&sh_hits, 1u);                                                \
-    if (k < FV_ONEPASS_HIT_CAP)                                                                \
+    if (k < a.hit_cap)                                                                         \
       hit_list[k] = make_uint2(__float_as_uint(v.member), 4u * p4 + lane4);                    \
     else                                                                                       \
       fv_finish_sparse_element<DELTA>(a, __float_as_uint(v.member), 4u * p4 + lane4, s, ok, xs, sp1, sp2); \
@@ -1845,7 +1847,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   }
   __syncthreads();
   // the sentinels the block has met, dealt over its threads
-  const uint32_t n_hits = min(sh_hits, (uint32_t)FV_ONEPASS_HIT_CAP);
+  const uint32_t n_hits = min(sh_hits, a.hit_cap);
   for (uint32_t i = tid; i < n_hits; i += T) {
     const uint2 hit = hit_list[i];
     fv_finish_sparse_element<DELTA>(a, hit.x, hit.y, s, ok, xs, sp1, sp2);
@@ -1987,7 +1989,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
     if (changed) e[lane4] = v.member;                                                          \
   } else {                                                                                     \
     const uint32_t k = atomicAdd(&sh_hits, 1u);                                                \
-    if (k < FV_STREAM_HIT_CAP)                                                                 \
+    if (k < a.hit_cap)                                                                         \
       hit_list[k] = make_uint2(__float_as_uint(v.member), 4u * p4 + lane4);                    \
     else                                                                                       \
       fv_finish_sparse_element<DELTA>(a, __float_as_uint(v.member), 4u * p4 + lane4, s, ok, xs, sp1, sp2); \
@@ -2025,7 +2027,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
     for (int e = 0; e < 4; ++e) pairs[(e * rows_per_round + r) * a.ldk4 + q] = make_float2(t1[e], t2[e]);
   }
   __syncthreads();
-  const uint32_t n_hits = min(sh_hits, (uint32_t)FV_STREAM_HIT_CAP);
+  const uint32_t n_hits = min(sh_hits, a.hit_cap);
   for (uint32_t i = tid; i < n_hits; i += T) {
     const uint2 hit = hit_list[i];
     fv_finish_sparse_element<DELTA>(a, hit.x, hit.y, s, ok, xs, sp1, sp2);
@@ -2892,6 +2894,10 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.invf = t->invf;
   d.slots = anti ? t->slots2 : slot_region ? t->slots_blocks : t->slots;
   d.slot_region = slot_region;
+  {
+    const uint32_t holds = t->onepass_stream ? FV_STREAM_HIT_CAP : FV_ONEPASS_HIT_CAP;
+    d.hit_cap = t->hit_cap_limit && t->hit_cap_limit < holds ? t->hit_cap_limit : holds;
+  }
   d.slot_count = t->slot_count;
   d.group_base = t->group_base;
   d.group_base2 = t->group_base2;
@@ -3130,6 +3136,12 @@ extern "C" int fv_trainer_set_grouping_launch(fv_trainer *t, uint32_t separate) 
   FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
   FV_REQUIRE(separate <= 1, FV_ERR_INVALID, "separate must be 0 or 1");
   t->separate_grouping = separate != 0;
+  return FV_OK;
+}
+
+extern "C" int fv_trainer_set_sentinel_list(fv_trainer *t, uint32_t entries) {
+  FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
+  t->hit_cap_limit = entries;
   return FV_OK;
 }
 

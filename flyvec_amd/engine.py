@@ -179,6 +179,11 @@ class Trainer:
         Same results either way."""
         check(self.lib.fv_trainer_set_slot_regions(self.handle, 1 if per_block else 0))
 
+    def set_sentinel_list(self, entries):
+        """Test hook: the single dense launch's LDS list of sparse elements counts as full after `entries`
+        (0: its real size); the elements beyond are finished where they are met.  Same results."""
+        check(self.lib.fv_trainer_set_sentinel_list(self.handle, int(entries)))
+
     @property
     def grouping_launch(self):
         """True when a step without the anti-Hebbian term groups in a launch of its own."""

@@ -229,7 +229,12 @@ int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate);
  * than a gigabyte in all, so no block has to count the windows of the neurons before it; per_block = 0: the
  * blocks share one region per class, each behind the records of the neurons before it, as the other launch
  * forms do. Results are bit-identical either way. No counterpart in the reference. */
-int fv_trainer_set_slot_regions(fv_trainer *t, uint32_t per_block); /* the form a step without the anti-Hebbian term takes */
+int fv_trainer_set_slot_regions(fv_trainer *t, uint32_t per_block);
+/* Test hook. A block of the single dense launch notes the sparse elements it meets (their sentinels) in an LDS
+ * list and finishes them when its dense elements are done; an element that finds the list full is finished on
+ * the spot. entries > 0 makes the list count as full after that many (no more than it holds: 2048, or 8192 in
+ * the streaming form), 0 restores its size. Results are bit-identical. No counterpart in the reference. */
+int fv_trainer_set_sentinel_list(fv_trainer *t, uint32_t entries); /* the form a step without the anti-Hebbian term takes */
 /* Test hook: between its two passes a single-launch dense pass waits for all its blocks, at most
  * `rounds` polling rounds (2^14 by default, tens of milliseconds); 0 makes every block give up at once, which
  * is how the error path of fv_trainer_sync is exercised. No counterpart in the reference. */

@@ -867,6 +867,36 @@ def test_random_configurations_match_the_oracle(gpu, oracle_lib, case):
         assert np.array_equal(Wg.view(np.uint32), Wo.view(np.uint32)), f"W, separate grouping {separate}, {c}"
 
 
+@pytest.mark.parametrize("launches,entries", [(1, 1), (1, 37), (3, 1), (3, 300)])
+def test_sparse_elements_beyond_the_sentinel_list_are_finished_where_they_are_met(gpu, oracle_lib, launches, entries):
+    """The single dense launch with a sentinel list that counts as full after a few entries: nearly every sparse
+    element takes the path of an element that finds the list full."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    V, K, w, B = 700, 130, 9, 2500
+    tokens, offsets = small_corpus(70000, V, seed=8)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    perm = np.random.default_rng(9).permutation(len(starts)).astype(np.uint64)
+    W0 = synthetic.synapses(K, V, seed=2, sigma=0.02)
+    Wo = W0.copy()
+    t = Trainer(V, K, w, B, initial_learning_rate=1e-3)
+    t.set_dense_launches(launches)
+    t.set_sentinel_list(entries)
+    t.set_corpus(tokens, offsets)
+    t.set_permutation(perm)
+    t.set_weights(W0)
+    for s in range(4):
+        ref = to.train_step(Wo, to.inflate(tokens, starts, perm, s * B, B, w, V), invf, 1e-3)
+        t.step(s * B, B, 1e-3)
+        xx, nc = t.step_stats()
+        assert np.array_equal(xx, ref["xx"]) and nc == ref["nc"]
+    Wg = t.get_weights()
+    known, made = t.dense_path_counts
+    t.close()
+    assert known >= 1 and made >= 1   # both ways through the launch
+    assert np.array_equal(Wg.view(np.uint32), Wo.view(np.uint32))
+
+
 @pytest.mark.parametrize("launches", [1, 2, 3])
 @pytest.mark.parametrize("per_block", [True, False])
 def test_slot_records_per_block_or_per_class(gpu, oracle_lib, launches, per_block):
