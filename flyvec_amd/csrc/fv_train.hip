@@ -435,6 +435,7 @@ __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, ui
 #endif
 #define FV_NB_CLASSES (1 << FV_NB_CLASS_SHIFT)  // column classes per neuron (kernel 3)
 #define FV_NB_CNT_WORDS 5120    // LDS counter words per class block (20 KB)
+#define FV_NB_CNT_WORDS_WIDE 6272  // or 24.5 KB, where that saves a pass
 #define FV_SP_LIST_CAP 1024     // positions of non-zero counters collected in LDS at a time
 #define FV_SP_CHUNK 16          // window positions read by 4 neighbouring lanes, 16 bytes each
 #define FV_IDX_PAD 80            // entries of -1 behind the index matrix: a padding row (up to 64 entries) and spare
@@ -826,11 +827,11 @@ __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uin
 // window ids in LDS by rank, and adds the neuron's scaled activations in the grouping kernel's order;
 // the block of class 0 leaves xx[h], the neuron's count and its base for the dense launch and clears
 // the neuron's row of the other bit-row buffer.
-template <bool DELTA, bool GROUPING>
+template <bool DELTA, bool GROUPING, int CW>
 __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   static_assert(!(DELTA && GROUPING), "the anti-Hebbian form has its two lists grouped by launches of their own");
-  __shared__ uint32_t cnt[FV_NB_CNT_WORDS];
-  __shared__ uint32_t cnt2[DELTA ? FV_NB_CNT_WORDS : 4];
+  __shared__ uint32_t cnt[CW];
+  __shared__ uint32_t cnt2[DELTA ? CW : 4];
   __shared__ uint16_t list[FV_SP_LIST_CAP];
   // window ids of a grouping step (at most 64 * FV_SP_THREADS windows, and the padding row behind them)
   // fit 16 bits: the smaller array lets one more block share a compute unit
@@ -915,7 +916,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       }
       base = fv_block_sum_u32((uint32_t)(-((int)below.x + (int)below.y)), red2);
     }
-    for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+    for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
     if (q == 0 && tid == 0) {
       a.group_base_out[h] = base;  // used where it was counted
       a.group_count_out[h] = c_h;
@@ -955,9 +956,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
 
   const bool staged_once = !DELTA && c_h <= FV_SP_STAGE;  // the usual case: the neuron's window ids are staged here
   if (!GROUPING) {
-    for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+    for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
     if (DELTA)
-      for (uint32_t i = tid; i < FV_NB_CNT_WORDS / 4; i += T) ((uint4 *)cnt2)[i] = make_uint4(0, 0, 0, 0);
+      for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt2)[i] = make_uint4(0, 0, 0, 0);
   }
   // xx[h] is added up in the grouping kernel's order: lane l of the first wave adds the values number
   // l, l + 64, ... onto 0, then the partial sums are added onto 0 in lane order (those of the lanes
@@ -979,7 +980,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     if (!xx_pending) {
       // A neuron with many windows: the activations are fetched by rank into the counter array
       // (cleared behind the block scan, and again by the first wave once it has added them).
-      static_assert(FV_SP_STAGE <= FV_NB_CNT_WORDS && FV_SP_STAGE % 64 == 0 && FV_SP_STAGE <= 8 * T,
+      static_assert(FV_SP_STAGE <= CW && FV_SP_STAGE % 64 == 0 && FV_SP_STAGE <= 8 * T,
                     "a stage of activations fits the counters and one trip to memory");
       float *scbuf = (float *)cnt;
       float part = 0.0f;
@@ -1036,7 +1037,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   // No counter can exceed the neuron's number of window positions: below 2^16 of them, two 16-bit
   // counters share a word and one pass covers twice as many columns.
   const bool narrow = m_ent < 65536u;
-  const uint32_t span = narrow ? 2 * FV_NB_CNT_WORDS : FV_NB_CNT_WORDS;          // class columns per pass
+  const uint32_t span = narrow ? 2 * CW : CW;          // class columns per pass
   const uint32_t class_cols = (n_cols + FV_NB_CLASSES - 1) >> FV_NB_CLASS_SHIFT;  // columns of a class
   uint32_t emitted = 0;
 
@@ -1090,12 +1091,12 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       }
       {
         // bit 8 * i + u of `mine`: counter u of the thread's i-th group of four words is non-zero
-        constexpr int n_groups = (FV_NB_CNT_WORDS / 4 + T - 1) / T;
+        constexpr int n_groups = (CW / 4 + T - 1) / T;
         static_assert(n_groups <= 8, "a 64-bit mask holds eight groups");
         uint64_t mine = 0;
 #pragma unroll
         for (int i = 0; i < n_groups; ++i) {
-          const uint32_t g4 = min(tid + i * T, (uint32_t)FV_NB_CNT_WORDS / 4 - 1);
+          const uint32_t g4 = min(tid + i * T, (uint32_t)CW / 4 - 1);
           uint4 c4 = ((const uint4 *)cnt)[g4];
           if (DELTA) {
             const uint4 d4 = ((const uint4 *)cnt2)[g4];
@@ -1106,7 +1107,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
               c4.x |= d4.x; c4.y |= d4.y; c4.z |= d4.z; c4.w |= d4.w;
             }
           }
-          if (tid + i * T >= FV_NB_CNT_WORDS / 4) c4 = make_uint4(0, 0, 0, 0);
+          if (tid + i * T >= CW / 4) c4 = make_uint4(0, 0, 0, 0);
           const uint32_t cw[4] = {c4.x, c4.y, c4.z, c4.w};
           uint32_t bits = 0;
 #pragma unroll
@@ -1211,16 +1212,24 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   }
 }
 
-template <bool DELTA>
+// CW: words of the block's LDS counter array (two 16-bit counters each while a neuron has fewer than 2^16
+// window positions). FV_NB_CNT_WORDS, six blocks per compute unit, covers the 10000 columns per class of the
+// headline shape in one pass; FV_NB_CNT_WORDS_WIDE, five blocks per compute unit, is taken where it saves a pass
+// (25000 columns per class at V = 50000: two passes instead of three).
+template <bool DELTA, int CW>
 __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
-  fv_sparse_block<DELTA, false>(a);
+  fv_sparse_block<DELTA, false, CW>(a);
 }
 
 // The form that groups for itself: with its 16-bit window ids six blocks fit a compute unit's LDS, and
 // the register count is held to what six waves per SIMD allow.
 __global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6))) void fv_sparse_grouping_kernel(
     fv_sparse_args a) {
-  fv_sparse_block<false, true>(a);
+  fv_sparse_block<false, true, FV_NB_CNT_WORDS>(a);
+}
+
+__global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_grouping_wide_kernel(fv_sparse_args a) {
+  fv_sparse_block<false, true, FV_NB_CNT_WORDS_WIDE>(a);
 }
 
 // ---- kernel 4: dense passes over the matrix (one launch, or 4a + 5 + 6) ---------------------------
@@ -2880,12 +2889,24 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.xx_out = t->xx;
   if (which & 4u) {
     const dim3 sp_grid(t->K * FV_NB_CLASSES), sp_block(FV_SP_THREADS);
-    if (anti)
-      hipLaunchKernelGGL(fv_sparse_kernel<true>, sp_grid, sp_block, 0, t->stream, sp);
-    else if (grouping_in_sparse)
-      hipLaunchKernelGGL(fv_sparse_grouping_kernel, sp_grid, sp_block, 0, t->stream, sp);
-    else
-      hipLaunchKernelGGL(fv_sparse_kernel<false>, sp_grid, sp_block, 0, t->stream, sp);
+    // the wider counter array where it saves a pass over the neuron's windows
+    const uint32_t class_cols = (uint32_t)((t->N + FV_NB_CLASSES - 1) / FV_NB_CLASSES);
+    // (counted for 16-bit counters, two to a word: what all but the heaviest neurons of a large minibatch use)
+    const auto passes = [&](uint32_t words) { return (class_cols + 2 * words - 1) / (2 * words); };
+    const bool wide = passes(FV_NB_CNT_WORDS_WIDE) < passes(FV_NB_CNT_WORDS);
+#define FV_LAUNCH_SPARSE(CW, GROUPING_KERNEL)                                                       \
+  if (anti)                                                                                         \
+    hipLaunchKernelGGL((fv_sparse_kernel<true, CW>), sp_grid, sp_block, 0, t->stream, sp);          \
+  else if (grouping_in_sparse)                                                                      \
+    hipLaunchKernelGGL(GROUPING_KERNEL, sp_grid, sp_block, 0, t->stream, sp);                       \
+  else                                                                                              \
+    hipLaunchKernelGGL((fv_sparse_kernel<false, CW>), sp_grid, sp_block, 0, t->stream, sp);
+    if (wide) {
+      FV_LAUNCH_SPARSE(FV_NB_CNT_WORDS_WIDE, fv_sparse_grouping_wide_kernel)
+    } else {
+      FV_LAUNCH_SPARSE(FV_NB_CNT_WORDS, fv_sparse_grouping_kernel)
+    }
+#undef FV_LAUNCH_SPARSE
   }
   if (ev) FV_HIP(hipEventRecord(ev[3], t->stream));
   fv_dense_args d;

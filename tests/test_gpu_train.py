@@ -557,7 +557,7 @@ def test_delta_small_config_bit_exact(gpu, oracle_lib, tie):
 
 
 @pytest.mark.parametrize("K,w,V,B", [(1, 1, 5, 1), (2, 3, 9, 7), (65, 15, 200, 256), (130, 64, 300, 64),
-                                     (30, 11, 30000, 700)])
+                                     (30, 11, 30000, 700), (20, 7, 22000, 500)])  # the last: the wider counter arrays
 def test_delta_shapes_bit_exact(gpu, oracle_lib, K, w, V, B):
     n_tokens = 40000 if V < 20000 else 120000
     Wg, Wo = run_both_delta(oracle_lib, V=V, K=K, w=w, B=B, steps=4, delta=0.25, n_tokens=n_tokens)
