@@ -1,0 +1,537 @@
+// Kernel 3 of the training step (device code of fv_train.hip).
+#pragma once
+
+#include "fv_train_group.h"
+
+// ---- kernel 3: sparse elements -----------------------------------------------------------------------
+//
+// FV_NB_CLASSES blocks per neuron h; block q owns the elements (h, column i) with
+// i mod FV_NB_CLASSES == q, so a neuron that won a large share of the minibatch is spread over
+// several blocks and no two blocks share an element.  A block counts the occurrences of each of
+// its columns over the neuron's windows in LDS, and for every distinct one saves
+// (element, count, weight) in a slot record and plants the sentinel in W.
+
+struct fv_sparse_args {
+  const uint32_t *order;
+  const uint32_t *group_base;
+  const uint32_t *group_count;
+  const int32_t *idx;  // followed by FV_IDX_PAD entries of -1
+  float *Wt;
+  fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records
+  uint64_t slot_stride;
+  // Not 0 (grouping form only): every block has a region of slot_region records of its own in slots[], at
+  // blockIdx * slot_region, and a sentinel names a record by its place in the block's region. A block has no
+  // more records than its class has columns, so no block needs to know what the others write.
+  uint32_t slot_region;
+  const float *xx;
+  const float *invf;
+  float *bmax_sparse;    // one maximum of |ds| per block
+  uint32_t *slot_count;  // records written per block
+  uint32_t ldk, w, V, pad_row;  // pad_row: the row index just behind the index matrix
+  uint32_t stride;              // entries per row of idx (a multiple of 4)
+  // anti-Hebbian form only: the windows in which the neuron came second, grouped like the others;
+  // the count of those occurrences of an element goes to slot_n2 beside its record
+  const uint32_t *order2;
+  const uint32_t *group_base2;
+  const uint32_t *group_count2;
+  uint32_t *slot_n2;
+  float delta;
+  float lmid, lbase;  // weight of a window's centre position (columns >= V) and of the others
+  // grouping form only: the block finds the neuron's windows in the winner array itself
+  const uint32_t *won;        // row h: bit r set where neuron h won window r (won_words words, an even number)
+  const uint16_t *win;        // 16-bit winners; behind the last one, up to a multiple of 64 entries, 0x7fff
+  uint32_t won_words;
+  uint32_t *won_clear;  // the other buffer: the class-0 block of neuron h clears row h
+  const float *sc;      // scaled activations of the windows
+  uint32_t n;           // windows of the step
+  uint32_t *order_out;  // a neuron's window ids beyond what LDS stages go through here
+  uint32_t *group_base_out, *group_count_out;
+  float *xx_out;
+  // The two largest |W[h][i]| of every row as the step finds the matrix (row_top2[h] = (v1, v2), v1 >= v2),
+  // when known: the block reports in row_hits how many of its elements hold v1 and, where v2 < v1, how
+  // many hold v2 (bits 0-1 and 2-3, each saturated at 3). The dense launch then knows whether the
+  // largest weight of a row is one of the step's sparse elements.
+  const float2 *row_top2;
+  uint32_t *row_hits;
+  uint32_t top2_known;
+};
+
+// Counting pass of one class block over the windows whose ids are staged in LDS: ord[0 .. n_staged),
+// followed up to the next multiple of FV_SP_WPS * LOADS by the id of the padding row behind the
+// index matrix (all -1). A row of idx is `stride` entries, a multiple of 4, those past w holding -1;
+// four consecutive lanes read the sixteen positions of a chunk of one window 16 bytes each, so a
+// wave's load covers sixteen windows. A lane issues LOADS loads back to back with no branch between
+// them (the compiler waits for every load in flight at a branch target), then counts. With the
+// class in the top bits and the column of the class below, one subtraction and one comparison tell
+// whether an entry is this block's: of class q, inside [lo, lo + span), not masked, not padding.
+#define FV_SP_WPS (FV_SP_THREADS / 4)  // windows the block takes per step
+#define FV_SLOT_REGIONS_MAX_BYTES (1ull << 30)  // most memory spent on slot regions per block
+template <bool NARROW>
+__device__ __forceinline__ void fv_sparse_count_entry(uint32_t *cnt, int32_t iv, uint32_t drop, uint32_t origin,
+                                                      uint32_t span) {
+  const uint32_t t = __builtin_rotateright32((uint32_t)iv | drop, FV_NB_CLASS_SHIFT) - origin;
+  if (t < span) {
+    if (NARROW)
+      atomicAdd(&cnt[t >> 1], 1u << (16 * (t & 1)));
+    else
+      atomicAdd(&cnt[t], 1u);
+  }
+}
+
+template <bool NARROW, int LOADS, typename Ord>
+__device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const Ord *ord, uint32_t n_staged,
+                                                const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
+                                                uint32_t lo, uint32_t span, uint32_t tid) {
+  const uint32_t c4 = 4u * (tid & 3u), slot = tid >> 2;
+  const uint32_t steps = (n_staged + FV_SP_WPS - 1) / FV_SP_WPS;
+  const uint32_t origin = (q << (32 - FV_NB_CLASS_SHIFT)) | lo;
+  for (uint32_t c0 = 0; c0 < stride; c0 += FV_SP_CHUNK) {
+    const bool live = c0 + c4 < stride;  // a row shorter than the chunk: the lanes past its end read its start again
+    const uint32_t cc = live ? c0 + c4 : 0u;
+    const uint32_t drop = live ? 0u : 0xffffffffu;
+    for (uint32_t s0 = 0; s0 < steps; s0 += LOADS) {
+      int4 iv[LOADS];
+#pragma unroll
+      for (int b = 0; b < LOADS; ++b)
+        iv[b] = *(const int4 *)(idx + (uint64_t)ord[(s0 + b) * FV_SP_WPS + slot] * stride + cc);
+#pragma unroll
+      for (int b = 0; b < LOADS; ++b) {
+        fv_sparse_count_entry<NARROW>(cnt, iv[b].x, drop, origin, span);
+        fv_sparse_count_entry<NARROW>(cnt, iv[b].y, drop, origin, span);
+        fv_sparse_count_entry<NARROW>(cnt, iv[b].z, drop, origin, span);
+        fv_sparse_count_entry<NARROW>(cnt, iv[b].w, drop, origin, span);
+      }
+    }
+  }
+}
+
+// The same with the number of loads in flight fitted to the number of windows; pads ord[].
+template <bool NARROW, typename Ord>
+__device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uint32_t n_staged, uint32_t pad_row,
+                                                    const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
+                                                    uint32_t lo, uint32_t span, uint32_t tid) {
+  static_assert(FV_SP_STAGE % (FV_SP_WPS * FV_SP_LOADS) == 0 && FV_SP_LOADS % 4 == 0, "padding of ord[] stays inside it");
+  const uint32_t per = FV_SP_WPS * (n_staged <= FV_SP_WPS ? 1 : n_staged <= FV_SP_WPS * 4 ? 4 : FV_SP_LOADS);
+  const uint32_t padded = (n_staged + per - 1) / per * per;
+  for (uint32_t i = n_staged + tid; i < padded; i += FV_SP_THREADS) ord[i] = (Ord)pad_row;
+  fv_lds_barrier();
+  if (per == FV_SP_WPS)
+    fv_sparse_count<NARROW, 1, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+  else if (per == FV_SP_WPS * 4)
+    fv_sparse_count<NARROW, 4, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+  else
+    fv_sparse_count<NARROW, FV_SP_LOADS, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+}
+
+// DELTA: the neuron's elements are counted over two lists of windows, those it won and those in
+// which it came second, into two counter arrays; a record carries both counts.
+// GROUPING: no grouping launch has run. Every class block takes its neuron's windows from the bit row
+// the winner kernel has filled (a thread's two words are 64 windows: the step has no more than
+// 64 * FV_SP_THREADS), counts the windows of lower neurons in the 16-bit winner array, stages the
+// window ids in LDS by rank, and adds the neuron's scaled activations in the grouping kernel's order;
+// the block of class 0 leaves xx[h], the neuron's count and its base for the dense launch and clears
+// the neuron's row of the other bit-row buffer.
+template <bool DELTA, bool GROUPING, int CW>
+__device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
+  static_assert(!(DELTA && GROUPING), "the anti-Hebbian form has its two lists grouped by launches of their own");
+  __shared__ uint32_t cnt[CW];
+  __shared__ uint32_t cnt2[DELTA ? CW : 4];
+  __shared__ uint16_t list[FV_SP_LIST_CAP];
+  // window ids of a grouping step (at most 64 * FV_SP_THREADS windows, and the padding row behind them)
+  // fit 16 bits: the smaller array lets one more block share a compute unit
+  static_assert(64 * FV_SP_THREADS < 65536, "ids of a grouping step fit 16 bits");
+  typedef typename std::conditional<GROUPING, uint16_t, uint32_t>::type ord_t;
+  __shared__ ord_t ord[FV_SP_STAGE];
+  __shared__ uint32_t sh_pos;
+  __shared__ float sh_xx;
+  __shared__ uint32_t sh_hits[2];
+  __shared__ float sc64[GROUPING ? 64 : 1];  // activations of a neuron with up to 64 windows, by rank
+  __shared__ float wave_max[16];
+  __shared__ uint32_t red[17];
+  constexpr uint32_t T = FV_SP_THREADS;
+  const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT;
+  const uint32_t q = blockIdx.x & (FV_NB_CLASSES - 1);
+  const uint32_t tid = threadIdx.x;
+  __shared__ uint32_t red2[GROUPING ? 17 : 1];
+  uint32_t c_h, base, my_off = 0, r0 = 0;
+  bool sc_complete = true;  // every thread's matches have their activations in pf[]
+  uint64_t mask = 0;
+  constexpr int PF = 4;
+  float pf[PF];
+  if (GROUPING) {
+    const uint32_t n = a.n;
+    // thread t takes windows 64 t .. 64 t + 63: two words of the neuron's row
+    r0 = 64 * tid;
+    uint2 mw = make_uint2(0u, 0u);
+    if (2 * tid < a.won_words) mw = *(const uint2 *)(a.won + (uint64_t)h * a.won_words + 2 * tid);
+    mask = (uint64_t)mw.x | ((uint64_t)mw.y << 32);
+    const uint32_t eq = (uint32_t)__popcll(mask);
+    if (q == 0) {
+      if (2 * tid < a.won_words) *(uint2 *)(a.won_clear + (uint64_t)h * a.won_words + 2 * tid) = make_uint2(0u, 0u);
+    }
+    // the scaled activations of a thread's first matches travel while the scan runs
+    uint64_t mm = mask;
+#pragma unroll
+    for (int e = 0; e < PF; ++e) {
+      const uint32_t r = mm ? r0 + (uint32_t)__ffsll((long long)mm) - 1 : r0;
+      pf[e] = a.sc[min(r, n - 1)];
+      mm &= mm - 1;
+    }
+    // one block scan gives the ranks and the neuron's count, and tells whether any thread has more matches
+    // than it has fetched activations for
+    const bool wave_more = __ballot(eq > (uint32_t)PF) != 0ull;
+    const uint32_t incl = fv_wave_inclusive_scan_u32(eq);
+    if ((tid & 63u) == 63u) red[tid >> 6] = incl, red[8 + (tid >> 6)] = wave_more;
+    fv_lds_barrier();
+    uint32_t before = 0, total = 0;
+    bool more = false;
+#pragma unroll
+    for (uint32_t i = 0; i < T / 64; ++i) {
+      const uint32_t t = red[i];
+      before += i < (tid >> 6) ? t : 0u;
+      total += t;
+      more = more || red[8 + i] != 0;
+    }
+    c_h = total;
+    my_off = before + incl - eq;
+    sc_complete = !more;
+    base = 0;
+    if (c_h != 0 && (a.slot_region == 0 || c_h > FV_SP_STAGE)) {
+      // The number of windows won by lower neurons is the neuron's place in order[] (more windows than LDS
+      // stages go through there) and in a class's slot region (where the blocks have no regions of their
+      // own). It is counted in the 16-bit winner array: 16-byte pieces dealt over the threads, two winners
+      // compared per operation (winner - h is negative in a 16-bit half exactly where the winner is lower;
+      // both are below 2^15). The entries behind the step's last window, up to the end of its piece, hold
+      // 0x7fff.
+      const uint32_t n8 = (n + 7) / 8;
+      const fv_short2 hh = {(short)h, (short)h};
+      fv_short2 below = {0, 0};
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {  // n <= 8 * 8 * T
+        if (g * T < n8) {            // the same answer in the whole block
+          const uint32_t i4 = tid + g * T;
+          int4 v = ((const int4 *)a.win)[min(i4, n8 - 1)];
+          if (i4 >= n8) v = make_int4(0x7fff7fff, 0x7fff7fff, 0x7fff7fff, 0x7fff7fff);
+          below += (__builtin_bit_cast(fv_short2, v.x) - hh) >> 15;
+          below += (__builtin_bit_cast(fv_short2, v.y) - hh) >> 15;
+          below += (__builtin_bit_cast(fv_short2, v.z) - hh) >> 15;
+          below += (__builtin_bit_cast(fv_short2, v.w) - hh) >> 15;
+        }
+      }
+      base = fv_block_sum_u32((uint32_t)(-((int)below.x + (int)below.y)), red2);
+    }
+    for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+    if (q == 0 && tid == 0) {
+      a.group_base_out[h] = base;  // used where it was counted
+      a.group_count_out[h] = c_h;
+      if (c_h == 0) a.xx_out[h] = 0.0f;
+    }
+  } else {
+    c_h = a.group_count[h];
+  }
+  const uint32_t c2_h = DELTA ? a.group_count2[h] : 0u;
+  if (c_h == 0 && c2_h == 0) {
+    if (tid == 0) {
+      a.bmax_sparse[blockIdx.x] = 0.0f;
+      a.slot_count[blockIdx.x] = 0;
+      a.row_hits[blockIdx.x] = 0;
+    }
+    return;
+  }
+  // counts of the block's elements that hold the row's largest / second largest weight (every path to the
+  // elements passes a barrier)
+  if (tid == 0) sh_hits[0] = sh_hits[1] = 0;
+  uint32_t hits1 = 0, hits2 = 0;  // the same in all lanes of a wave
+  // The launch lasts as long as its few heaviest blocks: their waves go first wherever they share a
+  // SIMD with the waves of light blocks.
+  if (c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
+  if (!GROUPING) base = a.group_base[h];
+  const uint32_t base2 = DELTA ? a.group_base2[h] : 0u;
+  float x_h = GROUPING ? 0.0f : a.xx[h];
+  float ds_max = 0.0f;
+  const uint32_t *order = (GROUPING ? a.order_out : a.order) + base;  // GROUPING: also written here, through order_out
+  const uint32_t n_cols = 2 * a.V;
+  const uint32_t m_ent = max(c_h, c2_h) * a.w;
+  // the block's records: no more than (c_h + c2_h) * w of them, behind those of the lower neurons
+  const bool regions = GROUPING && a.slot_region != 0;
+  const uint64_t slot_first = regions ? (uint64_t)blockIdx.x * a.slot_region
+                                      : (uint64_t)q * a.slot_stride + (uint64_t)(base + base2) * a.w;
+  fv_slot *slots = a.slots + slot_first;
+
+  const bool staged_once = !DELTA && c_h <= FV_SP_STAGE;  // the usual case: the neuron's window ids are staged here
+  if (!GROUPING) {
+    for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+    if (DELTA)
+      for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt2)[i] = make_uint4(0, 0, 0, 0);
+  }
+  // xx[h] is added up in the grouping kernel's order: lane l of the first wave adds the values number
+  // l, l + 64, ... onto 0, then the partial sums are added onto 0 in lane order (those of the lanes
+  // from c_h on are +0 and change nothing). A neuron with up to 64 windows, each thread holding the
+  // activations of all its matches, does that behind the counting pass, where the value is first
+  // needed and the loads have long returned.
+  bool xx_pending = GROUPING && staged_once && sc_complete && c_h <= 64;
+  if (GROUPING) {
+    // Window ids by rank: into LDS, or (more than LDS stages) to the neuron's part of order[], where
+    // the neuron's four blocks write the same values.
+    uint32_t rank = my_off;
+    for (uint64_t mm = mask; mm; mm &= mm - 1) {
+      const uint32_t r = r0 + (uint32_t)__ffsll((long long)mm) - 1;
+      if (staged_once)
+        ord[rank++] = (ord_t)r;
+      else
+        a.order_out[base + rank++] = r;
+    }
+    if (!xx_pending) {
+      // A neuron with many windows: the activations are fetched by rank into the counter array
+      // (cleared behind the block scan, and again by the first wave once it has added them).
+      static_assert(FV_SP_STAGE <= CW && FV_SP_STAGE % 64 == 0 && FV_SP_STAGE <= 8 * T,
+                    "a stage of activations fits the counters and one trip to memory");
+      float *scbuf = (float *)cnt;
+      float part = 0.0f;
+      if (staged_once)
+        fv_lds_barrier();  // the ids are in LDS
+      else
+        __syncthreads();  // the ids are in memory
+      for (uint32_t j0 = 0; j0 < c_h; j0 += FV_SP_STAGE) {
+        const uint32_t mr = min(c_h - j0, (uint32_t)FV_SP_STAGE);
+        float v8[8];  // eight loads in flight per thread
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const uint32_t j = j0 + min(tid + u * T, mr - 1);
+          v8[u] = a.sc[staged_once ? (uint32_t)ord[j] : order[j]];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (tid + u * T < mr) scbuf[tid + u * T] = v8[u];
+        fv_lds_barrier();
+        if (tid < 64) {
+          uint32_t j = tid;
+          for (; j + 192 < mr; j += 256) {  // four values fetched together, added one after the other
+            const float v0 = scbuf[j], v1 = scbuf[j + 64], v2 = scbuf[j + 128], v3 = scbuf[j + 192];
+            part = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(part, v0), v1), v2), v3);
+          }
+          for (; j < mr; j += 64) part = __fadd_rn(part, scbuf[j]);
+        }
+        if (j0 + FV_SP_STAGE < c_h) fv_lds_barrier();  // before the next stage overwrites this one
+      }
+      if (tid < 64) {
+        float xx = 0.0f;
+        if (c_h >= 64) {
+#pragma unroll
+          for (int l = 0; l < 64; ++l) xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), l)));
+        } else {
+          for (uint32_t l = 0; l < c_h; ++l)
+            xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), (int)l)));
+        }
+        if (tid == 0) {
+          sh_xx = xx;
+          if (q == 0) a.xx_out[h] = xx;
+        }
+        const uint32_t used = (min(c_h, (uint32_t)FV_SP_STAGE) + 3) / 4;
+        for (uint32_t i = tid; i < used; i += 64) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+      }
+    }
+    // the counting pass starts behind a barrier; sh_xx is read behind that pass
+  } else {
+    if (staged_once)
+      for (uint32_t i = tid; i < c_h; i += T) ord[i] = (ord_t)order[i];
+    fv_lds_barrier();
+  }
+
+  // No counter can exceed the neuron's number of window positions: below 2^16 of them, two 16-bit
+  // counters share a word and one pass covers twice as many columns.
+  const bool narrow = m_ent < 65536u;
+  const uint32_t span = narrow ? 2 * CW : CW;          // class columns per pass
+  const uint32_t class_cols = (n_cols + FV_NB_CLASSES - 1) >> FV_NB_CLASS_SHIFT;  // columns of a class
+  uint32_t emitted = 0;
+
+  for (uint32_t lo = 0; lo < class_cols; lo += span) {
+    for (int l = 0; l < (DELTA ? 2 : 1); ++l) {
+      const uint32_t *ids = l == 0 ? order : a.order2 + base2;
+      const uint32_t n_ids = l == 0 ? c_h : c2_h;
+      uint32_t *counters = l == 0 ? cnt : cnt2;
+      for (uint32_t j0 = 0; j0 < n_ids; j0 += FV_SP_STAGE) {
+        const uint32_t n_staged = min(n_ids - j0, (uint32_t)FV_SP_STAGE);
+        if (!staged_once) {
+          fv_lds_barrier();  // the previous part has been counted
+          for (uint32_t i = tid; i < n_staged; i += T) ord[i] = (ord_t)ids[j0 + i];
+          fv_lds_barrier();
+        }
+        if (narrow)
+          fv_sparse_count_any<true, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
+        else
+          fv_sparse_count_any<false, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
+      }
+    }
+    // Every non-zero counter is one distinct element. Their positions are collected in LDS, up to
+    // FV_SP_LIST_CAP at a time; a counter is cleared when its element is taken, so what did not fit
+    // is found again by the next round.
+    uint32_t found;
+    do {
+      if (tid == 0) sh_pos = 0;
+      if (GROUPING && xx_pending) {
+        uint32_t rk = my_off;
+        uint64_t mm = mask;
+#pragma unroll
+        for (int e = 0; e < PF; ++e)
+          if (mm) {
+            sc64[rk++] = pf[e];
+            mm &= mm - 1;
+          }
+      }
+      fv_lds_barrier();
+      if (GROUPING && xx_pending) {
+        if (tid < 64) {
+          const float part = tid < c_h ? __fadd_rn(0.0f, sc64[tid]) : 0.0f;
+          float xx = 0.0f;
+          for (uint32_t l = 0; l < c_h; ++l)
+            xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), (int)l)));
+          if (tid == 0) {
+            sh_xx = xx;
+            if (q == 0) a.xx_out[h] = xx;
+          }
+        }
+        xx_pending = false;
+      }
+      {
+        // bit 8 * i + u of `mine`: counter u of the thread's i-th group of four words is non-zero
+        constexpr int n_groups = (CW / 4 + T - 1) / T;
+        static_assert(n_groups <= 8, "a 64-bit mask holds eight groups");
+        uint64_t mine = 0;
+#pragma unroll
+        for (int i = 0; i < n_groups; ++i) {
+          const uint32_t g4 = min(tid + i * T, (uint32_t)CW / 4 - 1);
+          uint4 c4 = ((const uint4 *)cnt)[g4];
+          if (DELTA) {
+            const uint4 d4 = ((const uint4 *)cnt2)[g4];
+            if (narrow) {
+              // a 16-bit half is non-zero in the union if it is in either word: OR keeps that
+              c4.x |= d4.x; c4.y |= d4.y; c4.z |= d4.z; c4.w |= d4.w;
+            } else {
+              c4.x |= d4.x; c4.y |= d4.y; c4.z |= d4.z; c4.w |= d4.w;
+            }
+          }
+          if (tid + i * T >= CW / 4) c4 = make_uint4(0, 0, 0, 0);
+          const uint32_t cw[4] = {c4.x, c4.y, c4.z, c4.w};
+          uint32_t bits = 0;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            if (narrow) {
+              bits |= ((cw[u] & 0xffffu) ? 1u : 0u) << (2 * u);
+              bits |= ((cw[u] >> 16) ? 1u : 0u) << (2 * u + 1);
+            } else {
+              bits |= (cw[u] ? 1u : 0u) << u;
+            }
+          }
+          mine |= (uint64_t)bits << (8 * i);
+        }
+        // list positions: prefix sum inside the wave, one LDS atomic per wave
+        const uint32_t my = (uint32_t)__popcll(mine);
+        const int lane = tid & 63;
+        const uint32_t incl = fv_wave_inclusive_scan_u32(my);
+        uint32_t wave_base = 0;
+        if (lane == 63 && incl) wave_base = atomicAdd(&sh_pos, incl);
+        wave_base = fv_readlane(wave_base, 63);
+        uint32_t e = wave_base + incl - my;
+        while (mine) {
+          const uint32_t b = (uint32_t)__ffsll((long long)mine) - 1;
+          mine &= mine - 1;
+          if (e < FV_SP_LIST_CAP) list[e] = (uint16_t)((tid + (b >> 3) * T) * (narrow ? 8u : 4u) + (b & 7u));
+          ++e;
+        }
+      }
+      fv_lds_barrier();
+      found = sh_pos;
+      if (GROUPING) x_h = sh_xx;
+      const uint32_t take = min(found, (uint32_t)FV_SP_LIST_CAP);
+      // one element per thread (four in flight): save its weight and its count in a slot record,
+      // plant the sentinel, take |ds| (the dense term plus count additions of 1/f; a row with
+      // xx == 0 has ds == 0)
+      // number of the round's first record, for the sentinels (saturated: a step with more records than a
+      // sentinel can name is not finished by the launch that reads the numbers)
+      const uint32_t record0 = (uint32_t)min((regions ? 0ull : slot_first) + emitted, (uint64_t)FV_SENTINEL_MAX);
+      // the row's two largest weights: the same address in the whole block, fetched where they are used
+      const float2 top2 = a.top2_known ? a.row_top2[h] : make_float2(0.0f, 0.0f);
+      for (uint32_t eb = tid; eb < take; eb += 4 * T) {
+        uint32_t pe[4], ne[4], n2e[4];
+        float wv[4], fe[4], le[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const uint32_t k = list[min(eb + u * T, take - 1)];
+          const uint32_t word = narrow ? cnt[k >> 1] : cnt[k];
+          ne[u] = narrow ? (word >> (16 * (k & 1))) & 0xffffu : word;
+          n2e[u] = 0;
+          if (DELTA) {
+            const uint32_t word2 = narrow ? cnt2[k >> 1] : cnt2[k];
+            n2e[u] = narrow ? (word2 >> (16 * (k & 1))) & 0xffffu : word2;
+          }
+          const uint32_t col = ((lo + k) << FV_NB_CLASS_SHIFT) | q;
+          pe[u] = col * a.ldk + h;
+          wv[u] = a.Wt[pe[u]];
+          fe[u] = a.invf[col >= a.V ? col - a.V : col];
+          le[u] = col >= a.V ? a.lmid : a.lbase;
+          if (eb + u * T < take) {
+            if (narrow) {
+              atomicAnd(&cnt[k >> 1], 0xffff0000u >> (16 * (k & 1)));
+              if (DELTA) atomicAnd(&cnt2[k >> 1], 0xffff0000u >> (16 * (k & 1)));
+            } else {
+              cnt[k] = 0;
+              if (DELTA) cnt2[k] = 0;
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (eb + u * T < take) {
+            fv_slot rec;
+            rec.p = pe[u];
+            rec.n = ne[u];
+            rec.wv = wv[u];
+            rec.f = fe[u];
+            slots[emitted + eb + u * T] = rec;
+            if (DELTA) a.slot_n2[slot_first + emitted + eb + u * T] = n2e[u];
+            a.Wt[pe[u]] = fv_sentinel(record0 + eb + u * T);
+            // counted per wave from lane masks: the counts stay in scalar registers
+            const float aw = fabsf(wv[u]);
+            hits1 += (uint32_t)__popcll(__ballot(aw == top2.x));
+            hits2 += (uint32_t)__popcll(__ballot(aw == top2.y && top2.y < top2.x));
+            if (x_h != 0.0f)
+              ds_max = fv_absmax_keep(ds_max, DELTA ? fv_sparse_ds2(x_h, wv[u], fe[u], ne[u], a.delta, n2e[u], le[u])
+                                                    : fv_sparse_ds(x_h, wv[u], fe[u], ne[u], le[u]));
+          }
+      }
+      emitted += take;
+      fv_lds_barrier();
+    } while (found > FV_SP_LIST_CAP);
+  }
+  if ((tid & 63u) == 0 && (hits1 | hits2)) {
+    atomicAdd(&sh_hits[0], hits1);
+    atomicAdd(&sh_hits[1], hits2);
+  }
+  const float bm = fv_block_max_nonneg(ds_max, wave_max);  // behind its barriers every wave's hits are counted
+  if (tid == 0) {
+    a.bmax_sparse[blockIdx.x] = bm;
+    a.slot_count[blockIdx.x] = emitted;
+    a.row_hits[blockIdx.x] = min(sh_hits[0], 3u) | (min(sh_hits[1], 3u) << 2);
+  }
+}
+
+// CW: words of the block's LDS counter array (two 16-bit counters each while a neuron has fewer than 2^16
+// window positions). FV_NB_CNT_WORDS, six blocks per compute unit, covers the 10000 columns per class of the
+// headline shape in one pass; FV_NB_CNT_WORDS_WIDE, five blocks per compute unit, is taken where it saves a pass
+// (25000 columns per class at V = 50000: two passes instead of three).
+template <bool DELTA, int CW>
+__global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
+  fv_sparse_block<DELTA, false, CW>(a);
+}
+
+// The form that groups for itself: with its 16-bit window ids six blocks fit a compute unit's LDS, and
+// the register count is held to what six waves per SIMD allow.
+__global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6))) void fv_sparse_grouping_kernel(
+    fv_sparse_args a) {
+  fv_sparse_block<false, true, FV_NB_CNT_WORDS>(a);
+}
+
+__global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_grouping_wide_kernel(fv_sparse_args a) {
+  fv_sparse_block<false, true, FV_NB_CNT_WORDS_WIDE>(a);
+}
