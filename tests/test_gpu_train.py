@@ -136,7 +136,8 @@ def test_dense_launch_forms(gpu):
         Trainer(V, K, w, B).set_dense_launches(4)
 
 
-def test_single_dense_launch_gives_up_cleanly(gpu, oracle_lib):
+@pytest.mark.parametrize("form", [1, 3])  # the matrix kept in registers between the passes / its rows streamed
+def test_single_dense_launch_gives_up_cleanly(gpu, oracle_lib, form):
     """The wait between the two passes of the single launch is bounded. With a limit of zero rounds every block
     gives up at once (all kernels still run to their end): the step leaves W alone, the next synchronisation
     reports it, and the trainer carries on with two launches."""
@@ -145,7 +146,7 @@ def test_single_dense_launch_gives_up_cleanly(gpu, oracle_lib):
     V, K, w, B = 300, 64, 7, 128
     tokens, offsets = small_corpus(20000, V)
     W0 = synthetic.synapses(K, V)
-    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, launches=1)
+    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, launches=form)
     t._set_wait_limit(0)
     t.step(0, B, 1e-3)
     with pytest.raises(_lib.FlyvecError) as e:
@@ -155,7 +156,7 @@ def test_single_dense_launch_gives_up_cleanly(gpu, oracle_lib):
     t.sync()                                   # reported once
     assert np.array_equal(t.get_weights(), W0)
     starts, invf = oracle_inputs(to, tokens, offsets, V, w)
-    for launches in (2, 1):                    # usable afterwards, in either form
+    for launches in (2, form):                 # usable afterwards, in either form
         t._set_wait_limit(1 << 14)
         t.set_dense_launches(launches)
         t.set_weights(W0)
