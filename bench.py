@@ -39,6 +39,10 @@ HBM_PEAK = 8.0e12  # B/s, MI355X
 # vector-ALU issue rate: 256 compute units x 4 SIMDs, one wave64 instruction per SIMD every 4 cycles
 # (16 lanes per SIMD), at the 2.4 GHz peak engine clock
 VALU_ISSUE_PEAK = 256 * 4 * 2.4e9 / 4
+# L2 request throughput: 8 XCDs x 16 channels, one 128-byte request per channel and clock (the per-channel rate
+# of the CDNA 3 L2; no figure is published for this part), at the same clock
+L2_REQUEST_BYTES = 128
+L2_PEAK = 8 * 16 * L2_REQUEST_BYTES * 2.4e9
 
 TRAIN = dict(K=400, V=20000, w=11, B=10000, n_tokens=10_000_000, lr0=2e-4, n_epochs=15, prec=1e-30,
              zipf_s=1.07, mean_chunk=25)
@@ -125,6 +129,13 @@ def gather_entry(kernel, nbytes, ms, counters, source):
         out["valu_issue"] = {"bound": "valu_issue", "achieved": insts / (ms * 1e-3) / 1e9, "peak": VALU_ISSUE_PEAK / 1e9,
                              "unit": "G wave-instructions/s", "frac": insts / (ms * 1e-3) / VALU_ISSUE_PEAK,
                              "insts_per_launch": insts, "insts_source": source}
+    reqs = counters.get(kernel, {}).get("tcc_req")
+    if reqs:
+        out["l2_requests"] = {"bound": "l2", "achieved": reqs * L2_REQUEST_BYTES / (ms * 1e-3) / 1e9, "peak": L2_PEAK / 1e9,
+                              "unit": "GB/s", "frac": reqs * L2_REQUEST_BYTES / (ms * 1e-3) / L2_PEAK,
+                              "requests_per_launch": reqs, "requests_source": source,
+                              "basis": "TCC_REQ_sum x 128 B / duration against 8 XCDs x 16 channels x 128 B per clock "
+                                       "at 2.4 GHz"}
     return out
 
 
