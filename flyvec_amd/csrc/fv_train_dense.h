@@ -582,6 +582,11 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   // The update. A group without a sentinel is stored whole where something changed; in a group with
   // one the other elements are stored one by one and the sentinel is noted for later. The two largest
   // |W| of what the thread leaves behind are kept per neuron.
+  // the token of the thread's first entry of the minibatch sampled ahead: fetched before the stream over the
+  // rows, so that a corpus too large for the Infinity Cache does not lengthen the launch's tail
+  const uint32_t c0 = e0 - er0 * a.idx_stride;
+  int32_t tok0 = -1;
+  if (fast && samples0 && c0 < a.w) tok0 = a.corpus[start0 + c0];
   float t1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, t2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #define FV_ONEPASS_ELEMENT(member, lane4)                                                      \
   if (v.member == v.member) {                                                                  \
@@ -621,7 +626,10 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
     }
   }
 #undef FV_ONEPASS_ELEMENT
-  if (fast) fv_sample_ahead(a, samples0, e0, er0, start0, ahead_entries, TS);
+  if (fast) {
+    if (samples0) a.idx_ahead[e0] = c0 < a.w ? fv_column_index(tok0, c0, a.w, a.V) : -1;
+    fv_sample_ahead(a, false, e0, er0, start0, ahead_entries, TS);  // the entries beyond the first, if any
+  }
   if (active) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) pairs[(e * rows_per_round + r) * a.ldk4 + q] = make_float2(t1[e], t2[e]);
@@ -764,6 +772,10 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
     for (int u = 0; u < D; ++u) w[u] = a.Wt4[group_of(row0 + u * row_step)];  // the stream starts again
   }
 
+  // (as in fv_dense_onepass_kernel: the first token of the minibatch sampled ahead travels during the stream)
+  const uint32_t c0 = e0 - er0 * a.idx_stride;
+  int32_t tok0 = -1;
+  if (fast && samples0 && c0 < a.w) tok0 = a.corpus[start0 + c0];
   float t1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, t2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #define FV_STREAM_ELEMENT(member, lane4)                                                       \
   if (v.member == v.member) {                                                                  \
@@ -802,7 +814,10 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
     }
   }
 #undef FV_STREAM_ELEMENT
-  if (fast) fv_sample_ahead(a, samples0, e0, er0, start0, ahead_entries, TS);
+  if (fast) {
+    if (samples0) a.idx_ahead[e0] = c0 < a.w ? fv_column_index(tok0, c0, a.w, a.V) : -1;
+    fv_sample_ahead(a, false, e0, er0, start0, ahead_entries, TS);
+  }
   if (active) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) pairs[(e * rows_per_round + r) * a.ldk4 + q] = make_float2(t1[e], t2[e]);
