@@ -369,11 +369,28 @@ __device__ __forceinline__ void fv_sample_ahead(const fv_dense_args &a, bool sam
     const uint32_t c = e0 - er0 * a.idx_stride;
     a.idx_ahead[e0] = c < a.w ? fv_column_index(a.corpus[start0 + c], c, a.w, a.V) : -1;
   }
-  if (threadIdx.x >= 64)
-    for (uint32_t e = e0 + gridDim.x * TS; e < ahead_entries; e += gridDim.x * TS) {
-      const uint32_t r = e / a.idx_stride, c = e - r * a.idx_stride;
-      a.idx_ahead[e] = c < a.w ? fv_column_index(a.corpus[a.pstart[a.ahead_first + r] + c], c, a.w, a.V) : -1;
+  if (threadIdx.x >= 64) {
+    // four entries at a time: their window starts travel together, then their tokens
+    const uint32_t step = gridDim.x * TS;
+    for (uint32_t e = e0 + step; e < ahead_entries; e += 4 * step) {
+      uint32_t c[4];
+      uint64_t at[4];
+      int32_t tok[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t ek = e + k * step < ahead_entries ? e + k * step : e;
+        const uint32_t r = ek / a.idx_stride;
+        c[k] = ek - r * a.idx_stride;
+        at[k] = a.pstart[a.ahead_first + r];
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) tok[k] = a.corpus[at[k] + (c[k] < a.w ? c[k] : 0u)];
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (e + k * step < ahead_entries)
+          a.idx_ahead[e + k * step] = c[k] < a.w ? fv_column_index(tok[k], c[k], a.w, a.V) : -1;
     }
+  }
 }
 
 // The one decision of a launch that makes the pass for max|ds|: whether all its blocks go on to the update,
