@@ -55,6 +55,7 @@ class Trainer:
         if getattr(self, "handle", None) is not None and self.handle.value:
             self.lib.fv_trainer_destroy(self.handle)
         self.handle = None
+        self._checkpoint = None  # the page-locked buffer of save_weights
 
     def __del__(self):
         try:
@@ -102,10 +103,22 @@ class Trainer:
             raise ValueError(f"weights must be ({self.hid}, {2 * self.vocab}), got {W.shape}")
         check(self.lib.fv_trainer_set_weights(self.handle, ptr(W)))
 
-    def get_weights(self):
-        out = np.empty((self.hid, 2 * self.vocab), dtype=np.float32)
+    def get_weights(self, out=None):
+        """The K x 2V matrix in the checkpoint's layout. `out`: a C-contiguous float32 array of that shape to
+        fill (page-locked memory from _lib.pinned_empty is copied by DMA, five times as fast)."""
+        if out is None:
+            out = np.empty((self.hid, 2 * self.vocab), dtype=np.float32)
+        if out.shape != (self.hid, 2 * self.vocab) or out.dtype != np.float32 or not out.flags.c_contiguous:
+            raise ValueError(f"out must be a C-contiguous float32 array of shape {(self.hid, 2 * self.vocab)}")
         check(self.lib.fv_trainer_get_weights(self.handle, ptr(out)))
         return out
+
+    def save_weights(self, path):
+        """Writes the matrix as a .npy checkpoint (flyvec/train_flyvec.py:262: np.save of the K x 2V fp32
+        matrix) through a page-locked buffer the trainer keeps for this."""
+        if getattr(self, "_checkpoint", None) is None:
+            self._checkpoint = _lib.pinned_empty((self.hid, 2 * self.vocab), np.float32)
+        np.save(path, self.get_weights(self._checkpoint))
 
     def shuffle(self, seed=0):
         check(self.lib.fv_trainer_shuffle(self.handle, int(seed)))

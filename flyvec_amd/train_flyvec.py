@@ -111,7 +111,7 @@ def train(args, log=print):
         t2 = time.time()
         log(f"time per epoch =  {t2 - t1} [s]   py_model_arrays_reshuffle_indices time =  {t11 - t1} [s]")
         if ((i + 1) % args.save_every) == 0 or i == (args.Nep - 1):
-            np.save(output + str(ep), trainer.get_weights())
+            trainer.save_weights(output + str(ep))
             saved.append(output + str(ep) + ".npy")
     trainer.close()
     return saved
