@@ -868,6 +868,41 @@ def test_random_configurations_match_the_oracle(gpu, oracle_lib, case):
         assert np.array_equal(Wg.view(np.uint32), Wo.view(np.uint32)), f"W, separate grouping {separate}, {c}"
 
 
+@pytest.mark.parametrize("K,w,V,B", [(50, 5, 2000, 20000), (300, 11, 800, 40000), (7, 3, 50, 65535)])
+def test_minibatches_beyond_16384_windows(gpu, oracle_lib, K, w, V, B):
+    """More than 16384 windows per minibatch (the grouping launch is a launch of its own there, up to 64 windows
+    per thread of its blocks; the last case is the largest batch whose window ids fit 16 bits): three steps against
+    the checker, the last one partial, in both forms of the single dense launch and as separate launches."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    tokens, offsets = small_corpus(3 * B * 2 + 40000, V, seed=12)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    assert len(starts) >= 3 * B
+    perm = np.random.default_rng(13).permutation(len(starts)).astype(np.uint64)
+    W0 = synthetic.synapses(K, V, seed=4, sigma=0.02)
+    sizes = [B, B, B // 3 + 1]
+    Wo, ref, first = W0.copy(), [], 0
+    for n in sizes:
+        ref.append(to.train_step(Wo, to.inflate(tokens, starts, perm, first, n, w, V), invf, 1e-3))
+        first += n
+    for launches in (1, 2, 3):
+        t = Trainer(V, K, w, B, initial_learning_rate=1e-3)
+        t.set_dense_launches(launches)
+        t.set_corpus(tokens, offsets)
+        t.set_permutation(perm)
+        t.set_weights(W0)
+        first = 0
+        for s, n in enumerate(sizes):
+            t.step(first, n, 1e-3)
+            first += n
+            assert np.array_equal(t.winners(n), ref[s]["winners"]), f"winners, step {s}, launches {launches}"
+            xx, nc = t.step_stats()
+            assert np.array_equal(xx, ref[s]["xx"]) and nc == ref[s]["nc"], f"xx / max|ds|, step {s}, launches {launches}"
+        Wg = t.get_weights()
+        t.close()
+        assert np.array_equal(Wg.view(np.uint32), Wo.view(np.uint32)), f"W, launches {launches}"
+
+
 @pytest.mark.parametrize("launches,entries", [(1, 1), (1, 37), (3, 1), (3, 300)])
 def test_sparse_elements_beyond_the_sentinel_list_are_finished_where_they_are_met(gpu, oracle_lib, launches, entries):
     """The single dense launch with a sentinel list that counts as full after a few entries: nearly every sparse
