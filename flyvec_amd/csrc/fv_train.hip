@@ -803,6 +803,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
     hipLaunchKernelGGL((fv_sparse_kernel<true, CW>), sp_grid, sp_block, 0, t->stream, sp);          \
   else if (grouping_in_sparse)                                                                      \
     hipLaunchKernelGGL(GROUPING_KERNEL, sp_grid, sp_block, 0, t->stream, sp);                       \
+  else if (t->B < 65535u)                                                                           \
+    hipLaunchKernelGGL((fv_sparse_kernel<false, CW, true>), sp_grid, sp_block, 0, t->stream, sp);   \
   else                                                                                              \
     hipLaunchKernelGGL((fv_sparse_kernel<false, CW>), sp_grid, sp_block, 0, t->stream, sp);
     if (wide) {

@@ -131,7 +131,9 @@ __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uin
 // window ids in LDS by rank, and adds the neuron's scaled activations in the grouping kernel's order;
 // the block of class 0 leaves xx[h], the neuron's count and its base for the dense launch and clears
 // the neuron's row of the other bit-row buffer.
-template <bool DELTA, bool GROUPING, int CW>
+// IDS16: the window ids staged in LDS are 16 bits wide (a batch below 65535 windows, so that the id of the padding
+// row behind the index matrix fits too): the smaller array lets one more block share a compute unit.
+template <bool DELTA, bool GROUPING, int CW, bool IDS16 = GROUPING>
 __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   static_assert(!(DELTA && GROUPING), "the anti-Hebbian form has its two lists grouped by launches of their own");
   __shared__ uint32_t cnt[CW];
@@ -140,7 +142,8 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   // window ids of a grouping step (at most 64 * FV_SP_THREADS windows, and the padding row behind them)
   // fit 16 bits: the smaller array lets one more block share a compute unit
   static_assert(64 * FV_SP_THREADS < 65536, "ids of a grouping step fit 16 bits");
-  typedef typename std::conditional<GROUPING, uint16_t, uint32_t>::type ord_t;
+  static_assert(IDS16 || !GROUPING, "a grouping step's ids are 16 bits wide");
+  typedef typename std::conditional<IDS16, uint16_t, uint32_t>::type ord_t;
   __shared__ ord_t ord[FV_SP_STAGE];
   __shared__ uint32_t sh_pos;
   __shared__ float sh_xx;
@@ -520,9 +523,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
 // window positions). FV_NB_CNT_WORDS, six blocks per compute unit, covers the 10000 columns per class of the
 // headline shape in one pass; FV_NB_CNT_WORDS_WIDE, five blocks per compute unit, is taken where it saves a pass
 // (25000 columns per class at V = 50000: two passes instead of three).
-template <bool DELTA, int CW>
+template <bool DELTA, int CW, bool IDS16 = false>
 __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_kernel(fv_sparse_args a) {
-  fv_sparse_block<DELTA, false, CW>(a);
+  fv_sparse_block<DELTA, false, CW, IDS16>(a);
 }
 
 // The form that groups for itself: with its 16-bit window ids six blocks fit a compute unit's LDS, and
