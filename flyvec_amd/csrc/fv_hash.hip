@@ -90,9 +90,31 @@ __global__ __launch_bounds__(256) void fv_hash_kernel(fv_hash_args a) {
       key[j] = valid ? fv_ord_key(acc[j]) : 0u;  // pads sort below every real value
     }
 
-    // largest cand with count(key >= cand) >= k, built from the top bit down
+    // largest cand with count(key >= cand) >= k, built from the top bit down. The sign and exponent bits are
+    // usually settled in two steps instead of nine: the largest key M bounds cand from above, so if at least
+    // k keys reach the start t of M's binade, cand lies in [t, t + 2^23) -- nothing reaches t + 2^23 -- and only
+    // its mantissa bits are open; else the binade below is tried, where the count at t + 2^23 is known to be
+    // short of k. Past three binades of positive values the search runs over all 32 bits.
     uint32_t cand = 0, c_at = 0;
-    for (int bit = 31; bit >= 0; --bit) {
+    int bit = 31;
+    {
+      uint32_t m = key[0];
+#pragma unroll
+      for (int j = 1; j < NV; ++j) m = max(m, key[j]);
+      uint32_t t = fv_wave_max_u32(m) & 0xff800000u;
+      for (int tries = 0; tries < 3 && t > 0x80000000u; ++tries, t -= 0x00800000u) {  // keys of positive floats
+        uint32_t c = 0;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) c += (uint32_t)__popcll(__ballot(key[j] >= t));
+        if (c >= a.k) {
+          cand = t;
+          c_at = c;
+          bit = c == a.k ? -1 : 22;
+          break;
+        }
+      }
+    }
+    for (; bit >= 0; --bit) {
       const uint32_t t = cand | (1u << bit);
       uint32_t c = 0;
 #pragma unroll
