@@ -101,7 +101,8 @@ __global__ __launch_bounds__(256) void fv_hash_kernel(fv_hash_args a) {
       uint32_t m = key[0];
 #pragma unroll
       for (int j = 1; j < NV; ++j) m = max(m, key[j]);
-      uint32_t t = fv_wave_max_u32(m) & 0xff800000u;
+      // (the maximum is the same in every lane: said to the compiler, so that the search runs on scalar registers)
+      uint32_t t = (uint32_t)__builtin_amdgcn_readfirstlane((int)fv_wave_max_u32(m)) & 0xff800000u;
       for (int tries = 0; tries < 3 && t > 0x80000000u; ++tries, t -= 0x00800000u) {  // keys of positive floats
         uint32_t c = 0;
 #pragma unroll
@@ -114,25 +115,29 @@ __global__ __launch_bounds__(256) void fv_hash_kernel(fv_hash_args a) {
         }
       }
     }
-    for (; bit >= 0; --bit) {
-      const uint32_t t = cand | (1u << bit);
+    while (bit >= 0) {
+      // the threshold, the count and the decision are the same in every lane: kept in scalar registers
+      const uint32_t t = (uint32_t)__builtin_amdgcn_readfirstlane((int)(cand | (1u << bit)));
       uint32_t c = 0;
 #pragma unroll
       for (int j = 0; j < NV; ++j) c += (uint32_t)__popcll(__ballot(key[j] >= t));
-      if (c >= a.k) {
-        cand = t;
-        c_at = c;
-        if (c == a.k) break;
-      }
+      const bool take = c >= a.k;
+      cand = take ? t : cand;
+      c_at = take ? c : c_at;
+      bit = c == a.k ? -1 : bit - 1;
     }
-    uint32_t lo = 0xffffffffu, hi = 0u;
+    // The k-th largest is the smallest key >= cand, the (k+1)-th the largest key below it (or the k-th again
+    // where more than k keys reach cand). As unsigned differences both are minima without a comparison: key -
+    // cand is smallest for the smallest key >= cand (a key below cand wraps around to more than any such
+    // difference), and cand - 1 - key likewise for the largest key below cand (a pad, key 0, if nothing else).
+    uint32_t up = 0xffffffffu, down = 0xffffffffu;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-      if (key[j] >= cand) lo = key[j] < lo ? key[j] : lo;
-      else hi = key[j] > hi ? key[j] : hi;
+      up = min(up, key[j] - cand);
+      down = min(down, cand - 1u - key[j]);
     }
-    const float a_k = fv_ord_unkey(fv_wave_min_u32(lo));  // k-th largest
-    const float a_k1 = c_at > a.k ? a_k : fv_ord_unkey(fv_wave_max_u32(hi));  // (k+1)-th largest
+    const float a_k = fv_ord_unkey(cand + fv_wave_min_u32(up));  // k-th largest
+    const float a_k1 = c_at > a.k ? a_k : fv_ord_unkey(cand - 1u - fv_wave_min_u32(down));  // (k+1)-th largest
     const float thr = __fmul_rn(__fadd_rn(a_k, a_k1), 0.5f);
 
     uint64_t mine = 0;

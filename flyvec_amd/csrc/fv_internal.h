@@ -113,10 +113,12 @@ __device__ __forceinline__ uint64_t fv_wave_max_u64(uint64_t v) {
 }
 
 __device__ __forceinline__ uint32_t fv_wave_max_u32(uint32_t v) {
-#define FV_STEP32(CTRL)              \
-  {                                  \
-    uint32_t o = fv_dpp<CTRL>(v);    \
-    v = o > v ? o : v;               \
+  // old = 0 with bound_ctrl: every lane of these patterns has a source, and 0 is the identity of an unsigned
+  // maximum, which lets the compiler fold the lane move into the maximum (one instruction per step)
+#define FV_STEP32(CTRL)                                                                    \
+  {                                                                                        \
+    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true); \
+    v = o > v ? o : v;                                                                     \
   }
   FV_STEP32(FV_DPP_QUAD_XOR1)
   FV_STEP32(FV_DPP_QUAD_XOR2)
