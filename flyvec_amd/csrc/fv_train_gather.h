@@ -169,15 +169,15 @@ __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, ui
   for (int j = 0; j < NV; ++j)
     key[j] = (j < NV - 1 || (uint32_t)lane + 64u * j < a.K) ? fv_ord_key((float)acc[j]) : 0u;
   const uint32_t hstar = fv_wave_argmax<NV>(key, a.K, a.tie_rule, lane);
-  // the window's bit in the winner's row: issued first, it travels while the scaled activation is formed
-  if (lane == 0 && a.won && hstar < a.K)
-    atomicOr(&a.won[(uint64_t)hstar * a.won_words + (r >> 5)], 1u << (r & 31u));
   // the scaled activation is only ever read at the chosen neurons (flyvec/src/cuda_funcs.cu:731)
   const float s = fv_scaled_activation<WEIGHTED>(a, idx, hstar);
   if (lane == 0) {
     a.win[r] = (int32_t)hstar;
     a.win16[r] = (uint16_t)hstar;
     a.sc[r] = s;
+    // The window's bit in the winner's row, last: behind a branch the compiler waits for everything in flight,
+    // and issued before the scaled activation the atomic's trip to memory stood in front of that one's loads.
+    if (a.won && hstar < a.K) atomicOr(&a.won[(uint64_t)hstar * a.won_words + (r >> 5)], 1u << (r & 31u));
   }
   // the wave of the step's last window fills the 16-bit winners up to the next multiple of 64 with a
   // value no neuron has
