@@ -81,7 +81,8 @@ __global__ __launch_bounds__(256) void fv_hash_kernel(fv_hash_args a) {
     float acc[NV];
 #pragma unroll
     for (int j = 0; j < NV; ++j) acc[j] = 0.0f;
-    fv_gather_accumulate<NV, fv_rows_per_batch<NV>::value, float>(a.Wt, a.ldk, a.K, a.n_cols, lane, (int)a.w, idx, acc);
+    fv_gather_accumulate<NV, fv_rows_per_batch<NV>::value, float, false, true>(a.Wt, a.ldk, a.K, a.n_cols, lane, (int)a.w,
+                                                                               idx, acc);
 
     uint32_t key[NV];
 #pragma unroll

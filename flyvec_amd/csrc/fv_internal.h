@@ -171,19 +171,32 @@ __device__ __forceinline__ uint32_t fv_wave_sum_u32(uint32_t v) {
 // WEIGHTED: every weight is first multiplied, in fp32, by the weight of its window position --
 // l_mid for the centre, whose column lies in the second half of the columns, l_base for the others
 // (flyvec/src/cuda_funcs.cu:266-286).
-template <int NV, int RB, typename Acc, bool WEIGHTED = false>
+template <int NV, int RB, typename Acc, bool WEIGHTED = false, bool MASK_TAIL = false>
 __device__ __forceinline__ void fv_gather_batch(const float *__restrict__ Wt, uint32_t ldk, uint32_t n_cols, int lane,
                                                 int c0, int32_t idx_lane, Acc (&acc)[NV], float l_mid = 1.0f,
-                                                float l_base = 1.0f) {
+                                                float l_base = 1.0f, int tail = 64) {
   float v[RB][NV];
   float l[RB];
+  const float *rows[RB];
 #pragma unroll
   for (int b = 0; b < RB; ++b) {
     const uint32_t i = fv_readlane((uint32_t)idx_lane, c0 + b);
     l[b] = i >= n_cols / 2 ? l_mid : l_base;
-    const float *row = Wt + (uint64_t)(i < n_cols ? i : n_cols) * ldk;  // the same in every lane
+    rows[b] = Wt + (uint64_t)(i < n_cols ? i : n_cols) * ldk;  // the same in every lane
 #pragma unroll
-    for (int j = 0; j < NV; ++j) v[b][j] = row[lane + 64 * j];
+    for (int j = 0; j < NV - 1; ++j) v[b][j] = rows[b][lane + 64 * j];
+    if (MASK_TAIL)
+      v[b][NV - 1] = 0.0f;
+    else
+      v[b][NV - 1] = rows[b][lane + 64 * (NV - 1)];
+  }
+  // MASK_TAIL: the last register holds neurons in its first `tail` lanes only, and the other lanes stay out of its
+  // loads, which then fetch the end of the row and not the start of the next one (3 % on the hashing kernel,
+  // nothing on the training kernel, which does without). These loads come last in the batch, so the wait the
+  // compiler puts behind the branch is the wait for the batch.
+  if (MASK_TAIL && lane < tail) {
+#pragma unroll
+    for (int b = 0; b < RB; ++b) v[b][NV - 1] = rows[b][lane + 64 * (NV - 1)];
   }
 #pragma unroll
   for (int b = 0; b < RB; ++b) {
@@ -192,18 +205,19 @@ __device__ __forceinline__ void fv_gather_batch(const float *__restrict__ Wt, ui
   }
 }
 
-template <int NV, int RB, typename Acc, bool WEIGHTED = false>
+template <int NV, int RB, typename Acc, bool WEIGHTED = false, bool MASK_TAIL = false>
 __device__ __forceinline__ void fv_gather_accumulate(const float *__restrict__ Wt, uint32_t ldk, uint32_t K,
                                                      uint32_t n_cols, int lane, int w, int32_t idx_lane,
                                                      Acc (&acc)[NV], float l_mid = 1.0f, float l_base = 1.0f) {
-  (void)K;
+  const int tail = (int)K - 64 * (NV - 1);  // lanes of the last register that hold neurons
   int c0 = 0;
   for (; c0 + RB <= w; c0 += RB)
-    fv_gather_batch<NV, RB, Acc, WEIGHTED>(Wt, ldk, n_cols, lane, c0, idx_lane, acc, l_mid, l_base);
+    fv_gather_batch<NV, RB, Acc, WEIGHTED, MASK_TAIL>(Wt, ldk, n_cols, lane, c0, idx_lane, acc, l_mid, l_base, tail);
   // the rows left over, in batches of 8, 4, 2, 1 rather than one at a time: fewer dependent trips
 #define FV_TAIL(R)                                                                                    \
   if (RB > R && (w - c0) >= R) {                                                                      \
-    fv_gather_batch<NV, (R < RB ? R : 1), Acc, WEIGHTED>(Wt, ldk, n_cols, lane, c0, idx_lane, acc, l_mid, l_base); \
+    fv_gather_batch<NV, (R < RB ? R : 1), Acc, WEIGHTED, MASK_TAIL>(Wt, ldk, n_cols, lane, c0, idx_lane, acc, l_mid,     \
+                                                                    l_base, tail);                                   \
     c0 += R;                                                                                          \
   }
   FV_TAIL(8) FV_TAIL(4) FV_TAIL(2) FV_TAIL(1)
