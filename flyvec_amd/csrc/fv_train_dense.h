@@ -110,6 +110,22 @@ __device__ __forceinline__ void fv_dense_load(const fv_dense_args &a, uint32_t p
 // |w| for the bookkeeping of a row's largest weights; a NaN (a sentinel) counts as 0
 __device__ __forceinline__ float fv_abs_or_zero(float w) { return w == w ? fabsf(w) : 0.0f; }
 
+// A 16-byte group's four weights into the four neurons' pairs of largest weights; has_nan says whether any of
+// the four is a sentinel (the usual group has none and takes the short form).
+__device__ __forceinline__ void fv_top2_insert_four(float (&t1)[4], float (&t2)[4], const float4 &v, bool has_nan) {
+  if (!has_nan) {
+    fv_top2_insert_abs(t1[0], t2[0], v.x);
+    fv_top2_insert_abs(t1[1], t2[1], v.y);
+    fv_top2_insert_abs(t1[2], t2[2], v.z);
+    fv_top2_insert_abs(t1[3], t2[3], v.w);
+  } else {
+    fv_top2_insert(t1[0], t2[0], fv_abs_or_zero(v.x));
+    fv_top2_insert(t1[1], t2[1], fv_abs_or_zero(v.y));
+    fv_top2_insert(t1[2], t2[2], fv_abs_or_zero(v.z));
+    fv_top2_insert(t1[3], t2[3], fv_abs_or_zero(v.w));
+  }
+}
+
 // What one row adds to what is known of max|ds| before the matrix is seen (all three as bit patterns of
 // non-negative floats): S, the largest |ds| of a sparse element; E, the largest, over the rows whose largest
 // dense weight is known, of fl(|xx| * that weight); F, the same over the other rows with an upper bound of
@@ -251,12 +267,10 @@ __global__ __launch_bounds__(TB) void fv_update_kernel(fv_dense_args a) {
       const uint32_t rr = row + u * row_step;
       if (rr < a.n_rows) {
         float4 v = w[u];
+        const bool has_nan = __builtin_isunordered(v.x, v.y) || __builtin_isunordered(v.z, v.w);
         // a sentinel goes back as it came; the slot launch replaces it
         if (fv_apply_four(v, xq, s, a.update_cut)) a.Wt4[rr * a.ldk4 + q] = v;
-        fv_top2_insert(t1[0], t2[0], fv_abs_or_zero(v.x));
-        fv_top2_insert(t1[1], t2[1], fv_abs_or_zero(v.y));
-        fv_top2_insert(t1[2], t2[2], fv_abs_or_zero(v.z));
-        fv_top2_insert(t1[3], t2[3], fv_abs_or_zero(v.w));
+        fv_top2_insert_four(t1, t2, v, has_nan);
       }
     }
     row += FV_UPDATE_UNROLL * row_step;
@@ -632,10 +646,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
         FV_ONEPASS_ELEMENT(z, 2)
         FV_ONEPASS_ELEMENT(w, 3)
       }
-      fv_top2_insert(t1[0], t2[0], fv_abs_or_zero(v.x));
-      fv_top2_insert(t1[1], t2[1], fv_abs_or_zero(v.y));
-      fv_top2_insert(t1[2], t2[2], fv_abs_or_zero(v.z));
-      fv_top2_insert(t1[3], t2[3], fv_abs_or_zero(v.w));
+      fv_top2_insert_four(t1, t2, v, has_nan);
     }
     if (fast && u + DEPTH < U) {  // the next load takes the place of the one just used
       const uint32_t rown = row0 + (u + DEPTH) * row_step;
@@ -822,10 +833,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
           FV_STREAM_ELEMENT(z, 2)
           FV_STREAM_ELEMENT(w, 3)
         }
-        fv_top2_insert(t1[0], t2[0], fv_abs_or_zero(v.x));
-        fv_top2_insert(t1[1], t2[1], fv_abs_or_zero(v.y));
-        fv_top2_insert(t1[2], t2[2], fv_abs_or_zero(v.z));
-        fv_top2_insert(t1[3], t2[3], fv_abs_or_zero(v.w));
+        fv_top2_insert_four(t1, t2, v, has_nan);
       }
       w[u] = a.Wt4[group_of(row + D * row_step)];  // the round that takes this one's place
     }

@@ -11,6 +11,14 @@ __device__ __forceinline__ void fv_top2_insert(float &m1, float &m2, float a) {
   m2 = fmaxf(m2, fminf(m1, a));
   m1 = fmaxf(m1, a);
 }
+// The same with |w| of a weight known not to be a NaN, in two instructions with |w| as an operand modifier:
+// the median of (m1, m2, |w|) is the new second value, max(m1, |w|) the new first. The maximum is written as
+// the instruction itself: from fmaxf the compiler makes three, two of them to quieten signalling NaNs that
+// cannot be there.
+__device__ __forceinline__ void fv_top2_insert_abs(float &m1, float &m2, float w) {
+  m2 = __builtin_amdgcn_fmed3f(m1, m2, __builtin_fabsf(w));
+  asm("v_max_f32_e64 %0, %1, |%2|" : "=v"(m1) : "v"(m1), "v"(w));
+}
 __device__ __forceinline__ void fv_top2_merge(float &m1, float &m2, float b1, float b2) {
   const float lo = fminf(m1, b1);
   m1 = fmaxf(m1, b1);
