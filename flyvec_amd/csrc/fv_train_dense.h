@@ -142,7 +142,10 @@ __device__ __forceinline__ void fv_row_candidate(float x, float2 top2, uint4 hit
   const bool first = v1 == v2 ? n1 <= 1 : n1 == 0;
   const bool exact = first || (v1 != v2 && n2 == 0);
   const uint32_t cand = __float_as_uint(__fmul_rn(fabsf(x), first ? v1 : v2));
-  if (exact) E = max(E, cand); else F = max(F, cand);
+  // both maxima updated, one of them with 0: a store to whichever of the two the row chooses would keep them
+  // in memory, behind the loads of the matrix already in flight
+  E = max(E, exact ? cand : 0u);
+  F = max(F, exact ? 0u : cand);
   S = max(S, __float_as_uint(fmaxf(fmaxf(smx.x, smx.y), fmaxf(smx.z, smx.w))));
 }
 

@@ -78,10 +78,12 @@ __device__ __forceinline__ void fv_sparse_count_entry(uint32_t *cnt, int32_t iv,
   }
 }
 
-template <bool NARROW, int LOADS, typename Ord>
+// behind_first_loads() runs once, between the issue of the first loads and the counting of what they bring: the
+// place for work on values whose own loads were issued earlier and so have returned by then.
+template <bool NARROW, int LOADS, typename Ord, typename Hook>
 __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const Ord *ord, uint32_t n_staged,
                                                 const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
-                                                uint32_t lo, uint32_t span, uint32_t tid) {
+                                                uint32_t lo, uint32_t span, uint32_t tid, Hook &behind_first_loads) {
   const uint32_t c4 = 4u * (tid & 3u), slot = tid >> 2;
   const uint32_t steps = (n_staged + FV_SP_WPS - 1) / FV_SP_WPS;
   const uint32_t origin = (q << (32 - FV_NB_CLASS_SHIFT)) | lo;
@@ -94,6 +96,7 @@ __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const Ord *ord, u
 #pragma unroll
       for (int b = 0; b < LOADS; ++b)
         iv[b] = *(const int4 *)(idx + (uint64_t)ord[(s0 + b) * FV_SP_WPS + slot] * stride + cc);
+      if (c0 == 0 && s0 == 0) behind_first_loads();
 #pragma unroll
       for (int b = 0; b < LOADS; ++b) {
         fv_sparse_count_entry<NARROW>(cnt, iv[b].x, drop, origin, span);
@@ -106,21 +109,21 @@ __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const Ord *ord, u
 }
 
 // The same with the number of loads in flight fitted to the number of windows; pads ord[].
-template <bool NARROW, typename Ord>
+template <bool NARROW, typename Ord, typename Hook>
 __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uint32_t n_staged, uint32_t pad_row,
                                                     const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
-                                                    uint32_t lo, uint32_t span, uint32_t tid) {
+                                                    uint32_t lo, uint32_t span, uint32_t tid, Hook &behind_first_loads) {
   static_assert(FV_SP_STAGE % (FV_SP_WPS * FV_SP_LOADS) == 0 && FV_SP_LOADS % 4 == 0, "padding of ord[] stays inside it");
   const uint32_t per = FV_SP_WPS * (n_staged <= FV_SP_WPS ? 1 : n_staged <= FV_SP_WPS * 4 ? 4 : FV_SP_LOADS);
   const uint32_t padded = (n_staged + per - 1) / per * per;
   for (uint32_t i = n_staged + tid; i < padded; i += FV_SP_THREADS) ord[i] = (Ord)pad_row;
   fv_lds_barrier();
   if (per == FV_SP_WPS)
-    fv_sparse_count<NARROW, 1, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+    fv_sparse_count<NARROW, 1, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid, behind_first_loads);
   else if (per == FV_SP_WPS * 4)
-    fv_sparse_count<NARROW, 4, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+    fv_sparse_count<NARROW, 4, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid, behind_first_loads);
   else
-    fv_sparse_count<NARROW, FV_SP_LOADS, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid);
+    fv_sparse_count<NARROW, FV_SP_LOADS, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid, behind_first_loads);
 }
 
 // DELTA: the neuron's elements are counted over two lists of windows, those it won and those in
@@ -348,6 +351,24 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   const uint32_t class_cols = (n_cols + FV_NB_CLASSES - 1) >> FV_NB_CLASS_SHIFT;  // columns of a class
   uint32_t emitted = 0;
 
+  // The activations a thread fetched at the start go to LDS by rank as soon as they can be had without a wait
+  // of their own, behind the issue of the counting pass's first loads: held any longer they would sit in
+  // registers through the whole pass. (xx_pending implies a neuron with windows, so the pass has a first load.)
+  bool pf_staged = false;
+  auto stage_activations = [&]() {
+    if (GROUPING && xx_pending && !pf_staged) {
+      uint32_t rk = my_off;
+      uint64_t mm = mask;
+#pragma unroll
+      for (int e = 0; e < PF; ++e)
+        if (mm) {
+          sc64[rk++] = pf[e];
+          mm &= mm - 1;
+        }
+      pf_staged = true;
+    }
+  };
+
   for (uint32_t lo = 0; lo < class_cols; lo += span) {
     for (int l = 0; l < (DELTA ? 2 : 1); ++l) {
       const uint32_t *ids = l == 0 ? order : a.order2 + base2;
@@ -361,9 +382,11 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
           fv_lds_barrier();
         }
         if (narrow)
-          fv_sparse_count_any<true, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
+          fv_sparse_count_any<true, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid,
+                                           stage_activations);
         else
-          fv_sparse_count_any<false, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid);
+          fv_sparse_count_any<false, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid,
+                                            stage_activations);
       }
     }
     // Every non-zero counter is one distinct element. Their positions are collected in LDS, up to
@@ -372,16 +395,6 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     uint32_t found;
     do {
       if (tid == 0) sh_pos = 0;
-      if (GROUPING && xx_pending) {
-        uint32_t rk = my_off;
-        uint64_t mm = mask;
-#pragma unroll
-        for (int e = 0; e < PF; ++e)
-          if (mm) {
-            sc64[rk++] = pf[e];
-            mm &= mm - 1;
-          }
-      }
       fv_lds_barrier();
       if (GROUPING && xx_pending) {
         if (tid < 64) {
