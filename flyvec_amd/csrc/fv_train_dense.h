@@ -622,6 +622,10 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   int32_t tok0 = -1;
   if (fast && samples0 && c0 < a.w) tok0 = a.corpus[start0 + c0];
   float t1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, t2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  // A sentinel that finds the block's list full is finished by its own thread behind the stream (bit 4 u + e:
+  // element e of the thread's group u), from memory, where it still stands.
+  static_assert(4 * U <= 64, "one bit per element of a thread");
+  uint64_t beyond_list = 0;
 #define FV_ONEPASS_ELEMENT(member, lane4)                                                      \
   if (v.member == v.member) {                                                                  \
     if (changed) e[lane4] = v.member;                                                          \
@@ -630,7 +634,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
     if (k < a.hit_cap)                                                                         \
       hit_list[k] = make_uint2(__float_as_uint(v.member), 4u * p4 + lane4);                    \
     else                                                                                       \
-      fv_finish_sparse_element<DELTA>(a, __float_as_uint(v.member), 4u * p4 + lane4, s, ok, xs, sp1, sp2); \
+      beyond_list |= 1ull << (4 * u + lane4);                                                  \
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -660,6 +664,12 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   if (fast) {
     if (samples0) a.idx_ahead[e0] = c0 < a.w ? fv_column_index(tok0, c0, a.w, a.V) : -1;
     fv_sample_ahead(a, false, e0, er0, start0, ahead_entries, TS);  // the entries beyond the first, if any
+  }
+  while (beyond_list) {
+    const uint32_t b = (uint32_t)__ffsll((long long)beyond_list) - 1u;
+    beyond_list &= beyond_list - 1;
+    const uint32_t at = 4u * ((row0 + (b >> 2) * row_step) * a.ldk4 + q) + (b & 3u);
+    fv_finish_sparse_element<DELTA>(a, __float_as_uint(((const float *)a.Wt4)[at]), at, s, ok, xs, sp1, sp2);
   }
   if (active) {
 #pragma unroll
