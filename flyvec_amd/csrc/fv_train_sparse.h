@@ -212,16 +212,23 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       const uint32_t n8 = (n + 7) / 8;
       const fv_short2 hh = {(short)h, (short)h};
       fv_short2 below = {0, 0};
+      // n <= 8 * 8 * T: up to eight pieces per thread, in two batches of four loads with no branch between them (a
+      // piece past the end reads the last one again and counts as 0x7fff)
 #pragma unroll
-      for (int g = 0; g < 8; ++g) {  // n <= 8 * 8 * T
-        if (g * T < n8) {            // the same answer in the whole block
-          const uint32_t i4 = tid + g * T;
-          int4 v = ((const int4 *)a.win)[min(i4, n8 - 1)];
-          if (i4 >= n8) v = make_int4(0x7fff7fff, 0x7fff7fff, 0x7fff7fff, 0x7fff7fff);
-          below += (__builtin_bit_cast(fv_short2, v.x) - hh) >> 15;
-          below += (__builtin_bit_cast(fv_short2, v.y) - hh) >> 15;
-          below += (__builtin_bit_cast(fv_short2, v.z) - hh) >> 15;
-          below += (__builtin_bit_cast(fv_short2, v.w) - hh) >> 15;
+      for (int g0 = 0; g0 < 8; g0 += 4) {
+        if (g0 * T < n8) {  // the same answer in the whole block
+          int4 v4[4];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) v4[g] = ((const int4 *)a.win)[min(tid + (g0 + g) * T, n8 - 1)];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            int4 v = v4[g];
+            if (tid + (g0 + g) * T >= n8) v = make_int4(0x7fff7fff, 0x7fff7fff, 0x7fff7fff, 0x7fff7fff);
+            below += (__builtin_bit_cast(fv_short2, v.x) - hh) >> 15;
+            below += (__builtin_bit_cast(fv_short2, v.y) - hh) >> 15;
+            below += (__builtin_bit_cast(fv_short2, v.z) - hh) >> 15;
+            below += (__builtin_bit_cast(fv_short2, v.w) - hh) >> 15;
+          }
         }
       }
       base = fv_block_sum_u32((uint32_t)(-((int)below.x + (int)below.y)), red2);
@@ -300,12 +307,19 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
         __syncthreads();  // the ids are in memory
       for (uint32_t j0 = 0; j0 < c_h; j0 += FV_SP_STAGE) {
         const uint32_t mr = min(c_h - j0, (uint32_t)FV_SP_STAGE);
-        float v8[8];  // eight loads in flight per thread
+        // eight loads in flight per thread: the ids first, all of them, from LDS or from memory (a choice
+        // made inside the loop would put a wait for the previous activation in front of every load)
+        uint32_t id8[8];
+        float v8[8];
+        if (staged_once) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const uint32_t j = j0 + min(tid + u * T, mr - 1);
-          v8[u] = a.sc[staged_once ? (uint32_t)ord[j] : order[j]];
+          for (int u = 0; u < 8; ++u) id8[u] = (uint32_t)ord[j0 + min(tid + u * T, mr - 1)];
+        } else {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) id8[u] = order[j0 + min(tid + u * T, mr - 1)];
         }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v8[u] = a.sc[id8[u]];
 #pragma unroll
         for (int u = 0; u < 8; ++u)
           if (tid + u * T < mr) scbuf[tid + u * T] = v8[u];
