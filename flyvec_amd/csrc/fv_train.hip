@@ -630,6 +630,10 @@ static int fv_trainer_alloc_delta(fv_trainer *t) {
   return FV_OK;
 }
 
+// Whether the sparse launch of a step without the anti-Hebbian term groups for itself: the trainer has the bit rows
+// (a minibatch of up to 64 windows per thread of a class block).
+static bool fv_groups_in_sparse(const fv_trainer *t) { return t->won[0] && !t->separate_grouping; }
+
 // n_fresh < n: only the first n_fresh windows are sampled (from `first` on), the rows behind them are what
 // the index buffer of the previous step holds.
 static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps, float delta, hipEvent_t *ev,
@@ -681,8 +685,9 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   // the sparse launch's blocks group for themselves from those rows. A whole step takes the pair of
   // buffers the last such step's sparse launch has cleared; a launch on its own (measurement) stays
   // on the last step's pair, cleared here first unless it repeats the launch before it.
-  const bool grouping_in_sparse =
-      which == 0x3f ? !anti && t->won[0] && !t->separate_grouping : t->last_grouped_in_sparse;
+  // (beyond 64 windows per thread of a class block only with a slot region per block: without one every block
+  // would count the lower neurons' windows in the whole winner array)
+  const bool grouping_in_sparse = which == 0x3f ? !anti && fv_groups_in_sparse(t) : t->last_grouped_in_sparse;
   if (which == 0x3f) t->last_grouped_in_sparse = grouping_in_sparse;
   // the blocks of a sparse launch that groups for itself write their records to regions of their own, where
   // the trainer has them, and a sentinel names a record inside its block's region
@@ -1080,14 +1085,14 @@ extern "C" int fv_trainer_set_slot_regions(fv_trainer *t, uint32_t per_block) {
 
 extern "C" int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate) {
   FV_REQUIRE(t && out_separate, FV_ERR_INVALID, "null argument");
-  *out_separate = (t->won[0] && !t->separate_grouping) ? 0u : 1u;
+  *out_separate = fv_groups_in_sparse(t) ? 0u : 1u;
   return FV_OK;
 }
 
 extern "C" int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches) {
   FV_REQUIRE(t && out_launches, FV_ERR_INVALID, "null argument");
   // what a sentinel has to number in a step without the anti-Hebbian term
-  const bool regions = t->won[0] && !t->separate_grouping && t->slot_region && !t->no_block_regions;
+  const bool regions = fv_groups_in_sparse(t) && t->slot_region && !t->no_block_regions;
   const uint64_t n_slots = regions ? t->slot_region : (uint64_t)FV_NB_CLASSES * t->B * t->w;
   *out_launches = t->onepass && fv_trainers_alive.load() == 1 && n_slots + 1 < FV_SENTINEL_MAX ? 1u : 2u;
   return FV_OK;

@@ -136,7 +136,11 @@ __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uin
 // the neuron's row of the other bit-row buffer.
 // IDS16: the window ids staged in LDS are 16 bits wide (a batch below 65535 windows, so that the id of the padding
 // row behind the index matrix fits too): the smaller array lets one more block share a compute unit.
-template <bool DELTA, bool GROUPING, int CW, bool IDS16 = GROUPING>
+// NW (GROUPING): 64-bit words of the neuron's bit row per thread; a step has up to 64 * NW * FV_SP_THREADS windows.
+// (Four words per thread, for steps of up to 65534 windows, were built and measured at K = 1000, B = 50000: the
+// four class blocks of a neuron then each fetch and add its activations, and the launch takes as much longer
+// as the grouping launch it replaces lasts; only the one-word form is instantiated.)
+template <bool DELTA, bool GROUPING, int CW, bool IDS16 = GROUPING, int NW = 1>
 __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   static_assert(!(DELTA && GROUPING), "the anti-Hebbian form has its two lists grouped by launches of their own");
   __shared__ uint32_t cnt[CW];
@@ -144,7 +148,8 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   __shared__ uint16_t list[FV_SP_LIST_CAP];
   // window ids of a grouping step (at most 64 * FV_SP_THREADS windows, and the padding row behind them)
   // fit 16 bits: the smaller array lets one more block share a compute unit
-  static_assert(64 * FV_SP_THREADS < 65536, "ids of a grouping step fit 16 bits");
+  static_assert(NW == 1 || NW == 4, "one or four words of the bit row per thread");
+  static_assert(64 * FV_SP_THREADS < 65536, "ids of a grouping step fit 16 bits (the host keeps a step below 65535 windows)");
   static_assert(IDS16 || !GROUPING, "a grouping step's ids are 16 bits wide");
   typedef typename std::conditional<IDS16, uint16_t, uint32_t>::type ord_t;
   __shared__ ord_t ord[FV_SP_STAGE];
@@ -161,27 +166,51 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   __shared__ uint32_t red2[GROUPING ? 17 : 1];
   uint32_t c_h, base, my_off = 0, r0 = 0;
   bool sc_complete = true;  // every thread's matches have their activations in pf[]
-  uint64_t mask = 0;
+  uint64_t mask[NW];
+#pragma unroll
+  for (int i = 0; i < NW; ++i) mask[i] = 0;
+  uint32_t eq = 0;  // the thread's matches
   constexpr int PF = 4;
   float pf[PF];
   if (GROUPING) {
     const uint32_t n = a.n;
-    // thread t takes windows 64 t .. 64 t + 63: two words of the neuron's row
-    r0 = 64 * tid;
-    uint2 mw = make_uint2(0u, 0u);
-    if (2 * tid < a.won_words) mw = *(const uint2 *)(a.won + (uint64_t)h * a.won_words + 2 * tid);
-    mask = (uint64_t)mw.x | ((uint64_t)mw.y << 32);
-    const uint32_t eq = (uint32_t)__popcll(mask);
+    // thread t takes windows 64 NW t .. 64 NW (t + 1) - 1: 2 NW words of the neuron's row
+    r0 = 64 * NW * tid;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const uint32_t word = 2 * (NW * tid + i);
+      uint2 mw = make_uint2(0u, 0u);
+      if (word < a.won_words) mw = *(const uint2 *)(a.won + (uint64_t)h * a.won_words + word);
+      mask[i] = (uint64_t)mw.x | ((uint64_t)mw.y << 32);
+    }
+#pragma unroll
+    for (int i = 0; i < NW; ++i) eq += (uint32_t)__popcll(mask[i]);
     if (q == 0) {
-      if (2 * tid < a.won_words) *(uint2 *)(a.won_clear + (uint64_t)h * a.won_words + 2 * tid) = make_uint2(0u, 0u);
+#pragma unroll
+      for (int i = 0; i < NW; ++i) {
+        const uint32_t word = 2 * (NW * tid + i);
+        if (word < a.won_words) *(uint2 *)(a.won_clear + (uint64_t)h * a.won_words + word) = make_uint2(0u, 0u);
+      }
     }
     // the scaled activations of a thread's first matches travel while the scan runs
-    uint64_t mm = mask;
+    {
+      uint64_t left[NW];
 #pragma unroll
-    for (int e = 0; e < PF; ++e) {
-      const uint32_t r = mm ? r0 + (uint32_t)__ffsll((long long)mm) - 1 : r0;
-      pf[e] = a.sc[min(r, n - 1)];
-      mm &= mm - 1;
+      for (int i = 0; i < NW; ++i) left[i] = mask[i];
+#pragma unroll
+      for (int e = 0; e < PF; ++e) {
+        // the first word with a bit left, its lowest bit taken (no word left: the thread's first window)
+        uint32_t r = r0;
+        bool taken = false;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+          const bool here = !taken && left[i] != 0;
+          if (here) r = r0 + 64 * i + (uint32_t)__ffsll((long long)left[i]) - 1;
+          left[i] = here ? left[i] & (left[i] - 1) : left[i];
+          taken = taken || here;
+        }
+        pf[e] = a.sc[min(r, n - 1)];
+      }
     }
     // one block scan gives the ranks and the neuron's count, and tells whether any thread has more matches
     // than it has fetched activations for
@@ -202,20 +231,19 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     my_off = before + incl - eq;
     sc_complete = !more;
     base = 0;
-    if (c_h != 0 && (a.slot_region == 0 || c_h > FV_SP_STAGE)) {
-      // The number of windows won by lower neurons is the neuron's place in order[] (more windows than LDS
-      // stages go through there) and in a class's slot region (where the blocks have no regions of their
-      // own). It is counted in the 16-bit winner array: 16-byte pieces dealt over the threads, two winners
+    if (c_h != 0 && a.slot_region == 0) {
+      // The number of windows won by lower neurons is the neuron's place in a class's slot region where the
+      // blocks have no regions of their own. It is counted in the 16-bit winner array: 16-byte pieces dealt over the threads, two winners
       // compared per operation (winner - h is negative in a 16-bit half exactly where the winner is lower;
       // both are below 2^15). The entries behind the step's last window, up to the end of its piece, hold
       // 0x7fff.
       const uint32_t n8 = (n + 7) / 8;
       const fv_short2 hh = {(short)h, (short)h};
       fv_short2 below = {0, 0};
-      // n <= 8 * 8 * T: up to eight pieces per thread, in two batches of four loads with no branch between them (a
+      // n <= 8 * 8 * NW * T: up to 8 NW pieces per thread, in batches of four loads with no branch between them (a
       // piece past the end reads the last one again and counts as 0x7fff)
 #pragma unroll
-      for (int g0 = 0; g0 < 8; g0 += 4) {
+      for (int g0 = 0; g0 < 8 * NW; g0 += 4) {
         if (g0 * T < n8) {  // the same answer in the whole block
           int4 v4[4];
 #pragma unroll
@@ -283,17 +311,20 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   // activations of all its matches, does that behind the counting pass, where the value is first
   // needed and the loads have long returned.
   bool xx_pending = GROUPING && staged_once && sc_complete && c_h <= 64;
+  // GROUPING: the window ids of ranks [j0, j0 + FV_SP_STAGE) into LDS, every thread those of its own matches (its
+  // ranks start at my_off; a neuron with more windows than LDS stages is staged part by part, each time
+  // from the bit row's words in registers)
+  auto stage_ids = [&](uint32_t j0) {
+    uint32_t at = my_off - j0;  // wraps below 0 for the ranks in front of the part
+#pragma unroll
+    for (int i = 0; i < NW; ++i)
+      for (uint64_t mm = mask[i]; mm; mm &= mm - 1) {
+        if (at < (uint32_t)FV_SP_STAGE) ord[at] = (ord_t)(r0 + 64 * i + (uint32_t)__ffsll((long long)mm) - 1);
+        ++at;
+      }
+  };
   if (GROUPING) {
-    // Window ids by rank: into LDS, or (more than LDS stages) to the neuron's part of order[], where
-    // the neuron's four blocks write the same values.
-    uint32_t rank = my_off;
-    for (uint64_t mm = mask; mm; mm &= mm - 1) {
-      const uint32_t r = r0 + (uint32_t)__ffsll((long long)mm) - 1;
-      if (staged_once)
-        ord[rank++] = (ord_t)r;
-      else
-        a.order_out[base + rank++] = r;
-    }
+    if (staged_once) stage_ids(0);
     if (!xx_pending) {
       // A neuron with many windows: the activations are fetched by rank into the counter array
       // (cleared behind the block scan, and again by the first wave once it has added them).
@@ -301,23 +332,15 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
                     "a stage of activations fits the counters and one trip to memory");
       float *scbuf = (float *)cnt;
       float part = 0.0f;
-      if (staged_once)
-        fv_lds_barrier();  // the ids are in LDS
-      else
-        __syncthreads();  // the ids are in memory
       for (uint32_t j0 = 0; j0 < c_h; j0 += FV_SP_STAGE) {
         const uint32_t mr = min(c_h - j0, (uint32_t)FV_SP_STAGE);
-        // eight loads in flight per thread: the ids first, all of them, from LDS or from memory (a choice
-        // made inside the loop would put a wait for the previous activation in front of every load)
+        if (!staged_once) stage_ids(j0);  // (the barrier that ends a part stands in front of this)
+        fv_lds_barrier();                 // the ids are in LDS
+        // eight loads in flight per thread: the ids first, all of them
         uint32_t id8[8];
         float v8[8];
-        if (staged_once) {
 #pragma unroll
-          for (int u = 0; u < 8; ++u) id8[u] = (uint32_t)ord[j0 + min(tid + u * T, mr - 1)];
-        } else {
-#pragma unroll
-          for (int u = 0; u < 8; ++u) id8[u] = order[j0 + min(tid + u * T, mr - 1)];
-        }
+        for (int u = 0; u < 8; ++u) id8[u] = (uint32_t)ord[min(tid + u * T, mr - 1)];
 #pragma unroll
         for (int u = 0; u < 8; ++u) v8[u] = a.sc[id8[u]];
 #pragma unroll
@@ -371,14 +394,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   bool pf_staged = false;
   auto stage_activations = [&]() {
     if (GROUPING && xx_pending && !pf_staged) {
-      uint32_t rk = my_off;
-      uint64_t mm = mask;
 #pragma unroll
       for (int e = 0; e < PF; ++e)
-        if (mm) {
-          sc64[rk++] = pf[e];
-          mm &= mm - 1;
-        }
+        if ((uint32_t)e < eq) sc64[my_off + e] = pf[e];  // a thread's matches have consecutive ranks
       pf_staged = true;
     }
   };
@@ -392,7 +410,11 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
         const uint32_t n_staged = min(n_ids - j0, (uint32_t)FV_SP_STAGE);
         if (!staged_once) {
           fv_lds_barrier();  // the previous part has been counted
-          for (uint32_t i = tid; i < n_staged; i += T) ord[i] = (ord_t)ids[j0 + i];
+          if (GROUPING) {
+            stage_ids(j0);
+          } else {
+            for (uint32_t i = tid; i < n_staged; i += T) ord[i] = (ord_t)ids[j0 + i];
+          }
           fv_lds_barrier();
         }
         if (narrow)
