@@ -65,10 +65,16 @@ template <int NV>
 __global__ __launch_bounds__(256) void fv_hash_kernel(fv_hash_args a) {
   const int lane = threadIdx.x & 63;
   const uint64_t n_waves = (uint64_t)gridDim.x * 4;
-  for (uint64_t r = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6); r < a.n; r += n_waves) {
+  const uint64_t r_first = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  // a window's ids are fetched one window ahead: the load is on its way while the rows of the window before are
+  // gathered, and the wave's chain of dependent trips is one shorter per window
+  int32_t raw_ahead = -1;
+  if (r_first < a.n && lane < (int)a.w) raw_ahead = a.idx[r_first * a.w + lane];
+  for (uint64_t r = r_first; r < a.n; r += n_waves) {
     int32_t idx = -1;
+    const int32_t raw = raw_ahead;
+    if (r + n_waves < a.n && lane < (int)a.w) raw_ahead = a.idx[(r + n_waves) * a.w + lane];
     if (lane < (int)a.w) {
-      const int32_t raw = a.idx[r * a.w + lane];
       if (raw != -1 || a.shift != 0) {
         const int64_t col = (int64_t)raw + a.shift;
         if (raw >= 0 && col < (int64_t)a.n_cols)
