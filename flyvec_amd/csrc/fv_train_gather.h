@@ -67,6 +67,12 @@ __device__ __forceinline__ int32_t fv_column_index(int32_t tok, uint32_t c, uint
 // receives the anti-Hebbian terms. WEIGHTED: position weights other than 1 (:266-286, :307-327).
 template <int NV, bool DELTA, bool WEIGHTED>
 __global__ __launch_bounds__(256) void fv_gather_winner_kernel(fv_gather_args a) {
+  // The arguments of the usual path are asked for here, together: the compiler fetches an argument where it is first
+  // used, and three or four of those scalar loads, each behind a branch, stood one after the other in front of the
+  // first load of a window's ids.
+  asm volatile("" ::"s"(a.Wt), "s"(a.idx), "s"(a.invf), "s"(a.win), "s"(a.win16), "s"(a.won), "s"(a.sc), "s"(a.n),
+               "s"(a.K), "s"(a.ldk), "s"(a.w), "s"(a.V), "s"(a.tie_rule), "s"(a.stride), "s"(a.sampled),
+               "s"(a.n_fresh), "s"(a.won_words), "s"(a.merge_rows));
   if (blockIdx.x < a.merge_rows) {
     fv_merge_row_top2(a.merge, blockIdx.x);
     return;
