@@ -16,10 +16,14 @@ HBM before the timed region.  One JSON line is printed:
   kernels            the same for every kernel of the step; the window gathers, whose bytes are largely
                      served by the L2 caches, are held against measured HBM-side traffic and against the
                      vector-ALU issue rate instead of against their algorithmic bytes
-  step_roofline_frac (byte model of the whole step / 8 TB/s) / measured time per step
+  step_roofline_frac (byte model of the whole step, 4BwK + 12KN + 16Bw, / 8 TB/s) / measured time per step
+  step_moved_frac    the same with the bytes the step's scheme has to move, 4BwK + 8KN + 16Bw: max|ds| comes from
+                     the carried row maxima, so the matrix is read once and written once (null, and the figure
+                     under step_moved_byte_model_comparison, where it exceeds 1 because caches serve the gathers)
   cpu_baseline       the CPU restatement of the same step (oracle/, C + OpenMP) timed on this host
   hash               the batched top-k hash (1,048,576 windows, k = 32, bit-packed), device-resident,
-                     with the reference's numpy per-word path as its CPU baseline
+                     with the reference's numpy per-word path as its CPU baseline; targets_4096 and per_word_us:
+                     the reference-shaped calls (4096 target ids in one call; one word per call)
   hash_host          the same batch through the host-buffer entry point (copies included)
   large_step         K = 1000, V = 50000, w = 15, B = 50000 on a 200 M-token corpus (400 MB matrix)
   epoch              one full epoch over a 100 M-token corpus with device shuffle and one checkpoint
@@ -80,16 +84,18 @@ def traffic_bytes(counters, kernel):
     return (c["fetch_kib"] * FETCH_SCALE + c["write_kib"] * WRITE_SCALE) * 1024
 
 
-def kernel_bytes(K, N, w, B):
+def kernel_bytes(K, N, w, B, single_dense_launch=False):
     """Bytes every kernel of a step has to move. The window gather reads w rows of K floats per window
     (largely from L2: the rows repeat); the dense passes read the matrix for max|ds| and read + write it
     for the update -- the single launch keeps it in registers or knows max|ds| beforehand and so moves it
-    once each way; token ids, 1/f look-ups, slot records and sparse elements are 8 bytes per window
-    position and kernel."""
+    once each way. The sparse term is 16 bytes per window position in the byte model (token id, 1/f look-up,
+    read and write of the element): as six launches half of it falls to the sparse launch and half to the slot
+    update; with the single dense launch the sparse launch is held to all 16 (it reads the ids and 1/f, reads the
+    elements and writes the sentinels) and the dense launch's share is the records it reads back."""
     return {
         "gather_winner": 4 * B * w * K,
         "group_xx": 8 * B,
-        "sparse_owners": 8 * B * w,
+        "sparse_owners": (16 if single_dense_launch else 8) * B * w,
         "absmax_ds": 4 * K * N,
         "update": 8 * K * N,
         "slot_update": 8 * B * w,
@@ -102,6 +108,21 @@ def step_byte_model(K, N, w, B):
     written for the update (12 K N), 16 bytes per window position. A scheme that skips one of those
     passes scores above its share of this model; that is said where it applies."""
     return 4 * B * w * K + 12 * K * N + 16 * B * w
+
+
+def step_moved_model(K, N, w, B):
+    """The bytes the step's own scheme has to move: as step_byte_model, but max|ds| is taken from the carried two
+    largest weights of every row, so the matrix is read once and written once (8 K N)."""
+    return 4 * B * w * K + 8 * K * N + 16 * B * w
+
+
+def frac_fields(prefix, model, seconds):
+    """{prefix_frac: model time at 8 TB/s / measured time}; a figure above 1 is no fraction of a roof (caches
+    served bytes the model counts): it goes under a key that says so and the fraction reads null."""
+    value = (model / HBM_PEAK) / seconds
+    if value <= 1.0:
+        return {prefix + "_frac": value}
+    return {prefix + "_frac": None, prefix + "_byte_model_comparison": value}
 
 
 def hash_bytes_per_window(K, w):
@@ -191,7 +212,7 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, which="step", dense_launche
     t.close()
 
     N = 2 * c["V"]
-    per_kernel = kernel_bytes(c["K"], N, c["w"], c["B"])
+    per_kernel = kernel_bytes(c["K"], N, c["w"], c["B"], single_dense_launch=launches == 1)
     if launches == 1:
         # max|ds|, the update and the slot update ran as one launch (timed under the first name; the others are empty)
         kern_ms["dense_update"] = sum(kern_ms.pop(k) for k in ("absmax_ds", "update", "slot_update"))
@@ -232,8 +253,10 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, which="step", dense_launche
         "grouping_launch": "own" if grouping_separate else "in sparse_owners",
         "step_roofline_frac": (model / HBM_PEAK) / (ms_per_step * 1e-3),
         "step_byte_model": model,
+        "step_moved_model": step_moved_model(c["K"], N, c["w"], c["B"]),
         "n_windows": nwin,
     }
+    out.update(frac_fields("step_moved", out["step_moved_model"], ms_per_step * 1e-3))
     if graph:
         out["hip_graph"] = graph
     if launches == 1:
@@ -295,7 +318,8 @@ def bench_epoch(c=EPOCH):
     t.close()
     n_steps = (nwin + c["B"] - 1) // c["B"]
     model = step_byte_model(c["K"], 2 * c["V"], c["w"], c["B"])
-    return {"metric": "train windows/s over one full epoch", "value": nwin / total, "unit": "windows/s",
+    moved = frac_fields("step_moved", step_moved_model(c["K"], 2 * c["V"], c["w"], c["B"]) * (nwin / c["B"]), t_steps)
+    return {**moved, "metric": "train windows/s over one full epoch", "value": nwin / total, "unit": "windows/s",
             "config": {"workload": f"full training epoch: {c['n_tokens']} Zipf({c['zipf_s']}) tokens, K={c['K']} "
                                    f"Nvoc={c['V']} w={c['w']} B={c['B']}, {nwin} windows, device shuffle before "
                                    f"and one .npy checkpoint after (second epoch of a run)"},
@@ -305,6 +329,48 @@ def bench_epoch(c=EPOCH):
                             "setup_once": t_setup, "synthetic_corpus_generation": t_gen},
             "step_roofline_frac": (model * (nwin / c["B"]) / HBM_PEAK) / t_steps,
             "dense_launch_paths": {"knew_max_ds": known1 - known0, "made_the_pass": made1 - made0}}
+
+
+def bench_reference_shaped_calls(h, W, c):
+    """The calls in the shape the reference's API has (flyvec/core.py:139-163, 187-211): the 4096 Zipf target ids
+    of the CPU-runnable configuration (k = 50, int8 codes) in one fv_hash_targets call from host memory, and one
+    word per Python call -- through FlyVec.get_sparse_embedding, which reads a whole-vocabulary table that one
+    device launch fills on first use, and, for comparison, as one launch per word."""
+    from flyvec_amd import FlyVec, synthetic
+    ids = synthetic.zipf_ids(4096, c["V"], seed=2)
+    h.hash_targets(ids, 50)
+    best = float("inf")
+    for _ in range(20):
+        t0 = time.perf_counter()
+        h.hash_targets(ids, 50)
+        best = min(best, time.perf_counter() - t0)
+    vocab = ["<UNK>"] + [f"t{i}" for i in range(1, c["V"])]
+    words = [vocab[i] for i in ids]
+    model = FlyVec(W, tokenizer=vocab, normalize_synapses=False)
+    t0 = time.perf_counter()
+    model.code_table(50)
+    table_ms = (time.perf_counter() - t0) * 1e3
+    for word in words[:64]:
+        model.get_sparse_embedding(word)
+    t0 = time.perf_counter()
+    for word in words:
+        model.get_sparse_embedding(word)
+    per_word = (time.perf_counter() - t0) / len(words)
+    t0 = time.perf_counter()
+    for i in ids[:512]:
+        model.hasher.hash_targets([int(i)], 50)
+    per_launch = (time.perf_counter() - t0) / 512
+    model.hasher.close()
+    return {"targets_4096": {"value": len(ids) / best, "unit": "codes/s", "ms_per_call": best * 1e3,
+                             "workload": "fv_hash_targets: 4096 Zipf(1.07) target ids in host memory -> int8 codes of "
+                                         "length 400 in host memory, k = 50, one call (copies and launch included)"},
+            "per_word_us": per_word * 1e6,
+            "per_word": {"us_per_word": per_word * 1e6, "codes_per_s": 1.0 / per_word,
+                         "workload": "FlyVec.get_sparse_embedding(word) in a Python loop over the same 4096 words "
+                                     "(tokenizer look-up included), served from the whole-vocabulary table",
+                         "table_fill_ms": table_ms,
+                         "table": f"{c['V']} x {c['K']} int8 per hash length, one fv_hash_targets call on first use",
+                         "one_launch_per_word_us": per_launch * 1e6}}
 
 
 def bench_hash(reps, cpu_seconds, host_reps=5, host=True):
@@ -329,6 +395,7 @@ def bench_hash(reps, cpu_seconds, host_reps=5, host=True):
            "byte_model_frac": (bpw * c["n"] / HBM_PEAK) / (ms * 1e-3),
            "byte_model_note": "time the algorithmic bytes would take at 8 TB/s / measured time; above 1 because the "
                               "64 MB matrix is served by the L2 and Infinity caches"}
+    out.update(bench_reference_shaped_calls(h, W, c))
     if not host:
         h.close()
         d_idx.free()
@@ -387,7 +454,8 @@ def train_line(c, tr, steps, warmup):
                                f"{c['n_tokens']} Zipf({c['zipf_s']}) tokens, geometric chunks (mean {c['mean_chunk']}), "
                                f"{tr['n_windows']} windows, lr 2e-4, fp32"},
     }
-    for k in ("roofline", "step_roofline_frac", "step_byte_model", "event_ms_per_step", "kernels", "dense_launches",
+    for k in ("roofline", "step_roofline_frac", "step_byte_model", "step_moved_frac", "step_moved_byte_model_comparison",
+              "step_moved_model", "event_ms_per_step", "kernels", "dense_launches",
               "grouping_launch", "dense_launch_paths", "hip_graph", "cpu_baseline"):
         if k in tr:
             line[k] = tr[k]

@@ -49,6 +49,7 @@ SIGNATURES = {
     "fv_device_count": [C.POINTER(C.c_int)],
     "fv_set_device": [_i32],
     "fv_device_info": [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(_u64)],
+    "fv_device_memory": [C.POINTER(_u64), C.POINTER(_u64)],
     "fv_host_alloc_pinned": [C.c_size_t, _pp],
     "fv_host_free_pinned": [_vp],
     "fv_dev_alloc": [C.c_size_t, _pp],
@@ -101,6 +102,7 @@ SIGNATURES = {
     "fv_hasher_destroy": [_vp],
     "fv_hasher_normalize": [_vp, _f32],
     "fv_hasher_row_sumsq": [_vp, _vp],
+    "fv_hasher_row_sum_pow": [_vp, _u32, _vp],
     "fv_hasher_scale_rows": [_vp, _vp],
     "fv_hasher_get_weights": [_vp, _vp],
     "fv_hash_targets": [_vp, _vp, _u64, _u32, _vp],
@@ -154,6 +156,13 @@ def device_info():
     mem = C.c_uint64(0)
     check(load().fv_device_info(name, 256, C.byref(cus), C.byref(mem)))
     return {"name": name.value.decode(), "compute_units": cus.value, "hbm_bytes": mem.value}
+
+
+def device_memory():
+    """(free, total) bytes of the current device."""
+    free, total = C.c_uint64(0), C.c_uint64(0)
+    check(load().fv_device_memory(C.byref(free), C.byref(total)))
+    return free.value, total.value
 
 
 def calibration_copy(nbytes, reps=5):

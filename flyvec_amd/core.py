@@ -55,6 +55,8 @@ class FlyVec:
             self.hasher.normalize()  # flyvec/core.py:87
         self._synapses = None
         self._stop_ids = None
+        # hash_length -> (version of the resident matrix, codes of every token id): what the per-word calls read
+        self._code_tables = {}
 
     @classmethod
     def load(cls, force_redownload=False):
@@ -88,9 +90,9 @@ class FlyVec:
     @property
     def synapses(self):
         """The (normalised) matrix as the device holds it, K x 2V."""
-        if self._synapses is None:
-            self._synapses = self.hasher.weights()
-        return self._synapses
+        if self._synapses is None or self._synapses[0] != self.hasher.version:
+            self._synapses = (self.hasher.version, self.hasher.weights())
+        return self._synapses[1]
 
     @property
     def token_vocab(self):
@@ -137,12 +139,31 @@ class FlyVec:
         return self._first_token_id(token)[1] == 0
 
     # -- embeddings --------------------------------------------------------------------------------
+    CODE_TABLES_KEPT = 4  # hash lengths whose whole-vocabulary tables are kept (8 MB each at K = 400, V = 20000)
+
+    def code_table(self, hash_length: int = 50) -> np.ndarray:
+        """(n_vocab, K) int8: the code of every token id for this hash length, computed on the device by one
+        batched launch the first time the length is asked for and kept until the resident matrix changes.
+        The reference's API hashes one word per call (flyvec/core.py:139-163, looped at :187-211); a launch, two
+        copies and a synchronisation per word cost more than the arithmetic, so the per-word calls read here."""
+        entry = self._code_tables.get(hash_length)
+        if entry is None or entry[0] != self.hasher.version:
+            codes = self.hasher.hash_targets(np.arange(self.n_vocab, dtype=np.int32), hash_length)
+            codes.setflags(write=False)
+            self._code_tables.pop(hash_length, None)
+            while len(self._code_tables) >= self.CODE_TABLES_KEPT:
+                self._code_tables.pop(next(iter(self._code_tables)))
+            entry = self._code_tables[hash_length] = (self.hasher.version, codes)
+        return entry[1]
+
     def get_sparse_embedding(self, word, hash_length: int = 50):
         """flyvec/core.py:139-163; ``word`` may also be a token id."""
         tok, tok_id = self._first_token_id(word)
         if tok_id == 0:
             return self.unknown_embedding_info
-        code = self.hasher.hash_targets([tok_id], hash_length)[0]
+        if not 0 <= tok_id < self.n_vocab:
+            raise IndexError(f"token id {tok_id} is outside the vocabulary of {self.n_vocab}")
+        code = self.code_table(hash_length)[tok_id].copy()  # the caller's own array, as the reference returns
         return {"token": tok if tok is not None else self._id2token(tok_id), "id": tok_id, "embedding": code}
 
     def get_dense_embedding(self, word):

@@ -7,8 +7,11 @@
 //   * the output slot of a chunk's first window is an exclusive prefix sum of per-chunk window
 //     counts (three-pass scan: block totals, scan of totals, rescan + expansion);
 //   * the reference counts occurrences in an fp32 accumulator, which stops at 2^24; an integer
-//     histogram clamped to 2^24 gives the same value.
+//     histogram clamped to 2^24 gives the same value. The counters saturate (at 2^31) instead of wrapping,
+//     so a corpus of any length is counted right: the reference indexes its corpus with uint64_t
+//     (flyvec/src/model_arrays.cu:396-424) and was run on 5.8 G tokens (flyvec/src/test_inv.cpp:10-11).
 #include "fv_internal.h"
+#include "fv_histogram.h"
 
 #define FV_MAXLEN 214ull  // flyvec/src/prune_input.cpp:7
 #define FV_SCAN_THREADS 256
@@ -161,6 +164,18 @@ int fv_dev_build_window_starts(const uint64_t *offsets_dev, uint64_t n_chunks, u
 // ---- inverse unigram frequency ---------------------------------------------------------
 #define FV_HIST_LDS 12288  // ids below this are counted in LDS first (Zipf head), the rest in HBM
 
+// counts[i] = min(counts[i] + add, FV_HIST_SATURATED), whatever the other blocks add meanwhile
+__device__ __forceinline__ void fv_saturating_add(uint32_t *counter, uint32_t add) {
+  uint32_t seen = *counter;
+  for (;;) {
+    const uint32_t want = fv_hist_saturated_sum(seen, add);
+    if (want == seen) return;
+    const uint32_t old = atomicCAS(counter, seen, want);
+    if (old == seen) return;
+    seen = old;
+  }
+}
+
 __global__ __launch_bounds__(256) void fv_histogram_kernel(const int32_t *__restrict__ corpus,
                                                            uint64_t n_tokens, uint32_t vocab,
                                                            uint32_t *__restrict__ counts,
@@ -175,16 +190,19 @@ __global__ __launch_bounds__(256) void fv_histogram_kernel(const int32_t *__rest
     lo = t < lo ? t : lo;
     hi = t > hi ? t : hi;
     if (t >= 0 && (uint32_t)t < vocab) {
-      if (t < FV_HIST_LDS)
+      if (t < FV_HIST_LDS) {
         atomicAdd(&hist[t], 1u);
-      else
-        atomicAdd(&counts[t], 1u);
+      } else if (atomicAdd(&counts[t], 1u) >= FV_HIST_SATURATED + (1u << 30)) {
+        // far beyond the stop: back to it. Every thread that sees this writes the same value, and between the
+        // stop and the wrap lie 2^30 more additions than there are threads in flight.
+        atomicExch(&counts[t], FV_HIST_SATURATED);
+      }
     }
   }
   __syncthreads();
   const uint32_t lim = vocab < FV_HIST_LDS ? vocab : FV_HIST_LDS;
   for (uint32_t i = threadIdx.x; i < lim; i += 256)
-    if (hist[i]) atomicAdd(&counts[i], hist[i]);
+    if (hist[i]) fv_saturating_add(&counts[i], hist[i]);
   for (int d = 32; d >= 1; d >>= 1) {
     int32_t ol = __shfl_down(lo, d, 64), oh = __shfl_down(hi, d, 64);
     lo = ol < lo ? ol : lo;
@@ -200,9 +218,7 @@ __global__ void fv_invert_counts_kernel(const uint32_t *__restrict__ counts, uin
                                         float *__restrict__ invf) {
   uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= vocab) return;
-  uint32_t c = counts[i];
-  if (c > (1u << 24)) c = 1u << 24;  // where the reference's fp32 counter stops
-  invf[i] = c ? (float)(1.0 / (double)(float)c) : 0.0f;
+  invf[i] = fv_hist_invert(counts[i]);
 }
 
 int fv_dev_inverse_frequency(const int32_t *corpus_dev, uint64_t n_tokens, uint64_t vocab,
@@ -210,7 +226,7 @@ int fv_dev_inverse_frequency(const int32_t *corpus_dev, uint64_t n_tokens, uint6
                              hipStream_t stream) {
   FV_REQUIRE(vocab > 0 && vocab < (1ull << 30), FV_ERR_INVALID, "vocabulary size %llu out of range",
              (unsigned long long)vocab);
-  FV_REQUIRE(n_tokens < (1ull << 32), FV_ERR_INVALID, "corpus of %llu tokens exceeds 2^32",
+  FV_REQUIRE(n_tokens < FV_HIST_MAX_TOKENS, FV_ERR_INVALID, "corpus of %llu tokens exceeds 2^42",
              (unsigned long long)n_tokens);
   uint32_t *counts = nullptr;
   FV_HIP(hipMalloc((void **)&counts, vocab * sizeof(uint32_t) + 2 * sizeof(int32_t)));
@@ -220,8 +236,7 @@ int fv_dev_inverse_frequency(const int32_t *corpus_dev, uint64_t n_tokens, uint6
   if (e == hipSuccess)
     e = hipMemcpyAsync(minmax, init, sizeof init, hipMemcpyHostToDevice, stream);
   if (e == hipSuccess && n_tokens) {
-    uint64_t want = (n_tokens + 256 * 16 - 1) / (256 * 16);
-    unsigned blocks = (unsigned)(want < 1 ? 1 : (want > 2048 ? 2048 : want));
+    const unsigned blocks = fv_hist_blocks(n_tokens);
     hipLaunchKernelGGL(fv_histogram_kernel, dim3(blocks), dim3(256), 0, stream, corpus_dev, n_tokens,
                        (uint32_t)vocab, counts, minmax);
     e = hipGetLastError();
@@ -324,9 +339,10 @@ extern "C" int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, ui
 }
 
 // ---- inverse unigram frequency without any allocation -------------------------------------------------
-// For callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
-// harnesses that forbid hipMalloc): the occurrence counters and the id range live in a file-scope
-// device array instead of a buffer from hipMalloc. Every device the library runs on holds its own
+// For callers that cannot allocate device memory (tight serving loops, harnesses that forbid hipMalloc,
+// a process whose memory is all spoken for): the occurrence counters and the id range live in a file-scope
+// device array instead of a buffer from hipMalloc. The call itself runs on the null stream and ends with a
+// blocking copy of the id range to the host, so it cannot be captured into a graph as it is. Every device the library runs on holds its own
 // copy of the array, at its own address, until the process ends; host code reaches it only through
 // the address hipGetSymbolAddress returns for the device that is current.
 #define FV_STATIC_MAX_VOCAB (1u << 20)  // counters of the array: 4 MiB
@@ -351,8 +367,7 @@ static int fv_static_scratch_on_device(uint32_t **out) {
   return FV_OK;
 }
 
-// counters[0 .. vocab) = 0 and the id range to (INT_MAX, INT_MIN): a kernel, not a memset, so that a
-// caller may capture the call sequence in a graph.
+// counters[0 .. vocab) = 0 and the id range to (INT_MAX, INT_MIN), by a kernel.
 __global__ __launch_bounds__(256) void fv_static_clear_kernel(uint32_t *__restrict__ counts, uint32_t vocab,
                                                               int32_t *__restrict__ minmax) {
   for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < vocab; i += gridDim.x * 256) counts[i] = 0;
@@ -370,7 +385,7 @@ extern "C" int fv_inverse_frequency_static(const int32_t *corpus_dev, uint64_t n
              "fv_inverse_frequency_static: vocabulary of %llu ids; the built-in scratch array holds counters for at "
              "most %u (use fv_inverse_frequency, which allocates)",
              (unsigned long long)vocab, FV_STATIC_MAX_VOCAB);
-  FV_REQUIRE(n_tokens < (1ull << 32), FV_ERR_INVALID, "fv_inverse_frequency_static: corpus of %llu tokens exceeds 2^32",
+  FV_REQUIRE(n_tokens < FV_HIST_MAX_TOKENS, FV_ERR_INVALID, "fv_inverse_frequency_static: corpus of %llu tokens exceeds 2^42",
              (unsigned long long)n_tokens);
   uint32_t *counts = nullptr;
   FV_TRY(fv_static_scratch_on_device(&counts));
@@ -380,8 +395,7 @@ extern "C" int fv_inverse_frequency_static(const int32_t *corpus_dev, uint64_t n
   const unsigned clear_blocks = (unsigned)((vocab + 255) / 256 < 1024 ? (vocab + 255) / 256 : 1024);
   hipLaunchKernelGGL(fv_static_clear_kernel, dim3(clear_blocks), dim3(256), 0, stream, counts, (uint32_t)vocab, minmax);
   if (n_tokens) {
-    const uint64_t want = (n_tokens + 256 * 16 - 1) / (256 * 16);
-    const unsigned blocks = (unsigned)(want < 1 ? 1 : (want > 2048 ? 2048 : want));
+    const unsigned blocks = fv_hist_blocks(n_tokens);
     hipLaunchKernelGGL(fv_histogram_kernel, dim3(blocks), dim3(256), 0, stream, corpus_dev, n_tokens, (uint32_t)vocab,
                        counts, minmax);
   }

@@ -504,8 +504,8 @@ extern "C" int fv_hasher_time_windows(fv_hasher *h, const int32_t *idx_dev, uint
   return rc;
 }
 
-// ---- normalisation (flyvec/core.py:23-36, p = 2) -----------------------------------------------
-// numpy sums each row of syn**2 in runs of 8192 elements (its buffer size), added in order onto 0;
+// ---- normalisation (flyvec/core.py:23-36) ------------------------------------------------------
+// numpy sums each row of syn**p in runs of 8192 elements (its buffer size), added in order onto 0;
 // each run is summed with its pairwise scheme: blocks of at most 128 elements with 8 interleaved
 // accumulators combined as ((r0+r1)+(r2+r3))+((r4+r5)+(r6+r7)) plus a sequential tail; longer
 // ranges split at n/2 rounded down to a multiple of 8. The leaves of that recursion are
@@ -531,14 +531,28 @@ static void fv_pairwise_plan(uint32_t start, uint32_t n, std::vector<fv_leaf> &l
   prog.push_back(-1);  // pop two, push their sum
 }
 
+// x**p as numpy forms it for a float32 array and a Python integer p: p = 1 is the value itself, p = 2 the fp32
+// product x * x (numpy's fast paths, exact restatements). For p >= 3 numpy calls the platform's powf, whose last
+// bit is the C library's choice; here that case is the product x * x * ... * x taken in double and rounded to
+// fp32 once, which agrees with a correctly rounded powf except for double-rounding cases.
+template <int P>
+__device__ __forceinline__ float fv_elem_pow(float x, uint32_t p) {
+  if (P == 1) return x;
+  if (P == 2) return __fmul_rn(x, x);
+  double r = (double)x;
+  for (uint32_t i = 1; i < p; ++i) r *= (double)x;
+  return (float)r;
+}
+
+template <int P>
 __global__ __launch_bounds__(256) void fv_leaf_sumsq_kernel(const float *__restrict__ Wt, uint32_t K,
                                                             uint32_t ldk, const fv_leaf *__restrict__ leaves,
-                                                            float *__restrict__ leaf_sums) {
+                                                            float *__restrict__ leaf_sums, uint32_t p) {
   const uint32_t h = blockIdx.y * 256 + threadIdx.x;
   if (h >= K) return;
   const fv_leaf lf = leaves[blockIdx.x];
   const float *col = Wt + (uint64_t)lf.start * ldk + h;
-#define FV_SQ(i) __fmul_rn(col[(uint64_t)(i) * ldk], col[(uint64_t)(i) * ldk])
+#define FV_SQ(i) fv_elem_pow<P>(col[(uint64_t)(i) * ldk], p)
   float res;
   if (lf.len < 8) {
     res = -0.0f;
@@ -591,9 +605,12 @@ __global__ __launch_bounds__(256) void fv_scale_rows_kernel(float *__restrict__ 
   }
 }
 
-// out_sums[h] = numpy.sum(W[h]**2) in numpy's fp32 pairwise order
-extern "C" int fv_hasher_row_sumsq(fv_hasher *h, float *out_sums) {
+extern "C" int fv_hasher_row_sumsq(fv_hasher *h, float *out_sums) { return fv_hasher_row_sum_pow(h, 2, out_sums); }
+
+// out_sums[h] = numpy.sum(W[h]**p) in numpy's fp32 pairwise order
+extern "C" int fv_hasher_row_sum_pow(fv_hasher *h, uint32_t p, float *out_sums) {
   FV_REQUIRE(h && out_sums, FV_ERR_INVALID, "null argument");
+  FV_REQUIRE(p >= 1 && p <= 64, FV_ERR_INVALID, "p = %u: the norm's exponent must be an integer from 1 to 64", p);
   std::vector<fv_leaf> leaves;
   std::vector<int32_t> prog;
   prog.push_back(-2);  // push 0: the reduction starts from add's identity
@@ -614,8 +631,13 @@ extern "C" int fv_hasher_row_sumsq(fv_hasher *h, float *out_sums) {
   if (e == hipSuccess)
     e = hipMemcpyAsync(d_prog, prog.data(), prog.size() * sizeof(int32_t), hipMemcpyHostToDevice, h->stream);
   if (e == hipSuccess) {
-    hipLaunchKernelGGL(fv_leaf_sumsq_kernel, dim3((unsigned)leaves.size(), (h->K + 255) / 256), dim3(256), 0,
-                       h->stream, h->Wt, h->K, h->ldk, d_leaves, d_leaf);
+    const dim3 grid((unsigned)leaves.size(), (h->K + 255) / 256);
+    if (p == 1)
+      hipLaunchKernelGGL(fv_leaf_sumsq_kernel<1>, grid, dim3(256), 0, h->stream, h->Wt, h->K, h->ldk, d_leaves, d_leaf, p);
+    else if (p == 2)
+      hipLaunchKernelGGL(fv_leaf_sumsq_kernel<2>, grid, dim3(256), 0, h->stream, h->Wt, h->K, h->ldk, d_leaves, d_leaf, p);
+    else
+      hipLaunchKernelGGL(fv_leaf_sumsq_kernel<0>, grid, dim3(256), 0, h->stream, h->Wt, h->K, h->ldk, d_leaves, d_leaf, p);
     hipLaunchKernelGGL(fv_combine_leaves_kernel, dim3((h->K + 63) / 64), dim3(64), 0, h->stream, d_leaf, h->K,
                        d_prog, (uint32_t)prog.size(), d_out);
     e = hipGetLastError();

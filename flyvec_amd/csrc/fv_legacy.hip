@@ -22,9 +22,11 @@ struct legacy_arrays {
   bool synapses_owned = false;
   const int32_t *corpus = nullptr;
   const uint64_t *starts = nullptr;
+  uint64_t *starts_owned = nullptr;  // the table set_data_pointer("INPUT") builds for a window matrix
   uint64_t n_tokens = 0;
   bool corpus_on_device = false;
-  uint64_t shuffles = 0;
+  uint64_t shuffles = 0;          // shuffles applied so far: the seed of the next one
+  bool shuffle_pending = false;   // the shuffle of the allocation, applied once the window order exists
 };
 
 [[noreturn]] void die(const char *where) {
@@ -53,6 +55,9 @@ void upload_corpus(legacy_arrays *A, const legacy_descriptor *D, const char *whe
       if (A->starts[i] + D->W > n_tokens) n_tokens = A->starts[i] + D->W;
   if (fv_trainer_set_corpus_starts(A->trainer, A->corpus, n_tokens, A->starts, D->Ns_1) != FV_OK) die(where);
   A->corpus_on_device = true;
+  // flyvec/src/model_arrays.cu:180-198: the order is shuffled once when the arrays are allocated; here the order
+  // exists from this moment on (a corpus handed over again starts from the identity and is shuffled again)
+  if (A->shuffle_pending && fv_trainer_shuffle(A->trainer, A->shuffles++) != FV_OK) die(where);
 }
 
 }  // namespace
@@ -168,6 +173,10 @@ extern "C" void model_arrays_allocate_memory(void *descriptor, void *arrays, int
     die_msg("model_arrays_allocate_memory",
             "only the text model of flyvec_train is built: sparse_input = 1 and frequency_scaling = 1");
   if (A->trainer) die_msg("model_arrays_allocate_memory", "called twice");
+  // flyvec/src/model_descriptor.cu:30 sets p = m = 2 and the reference's driver never changes them; the update
+  // rule built here is the p = 2 one (ds = -xx W + input) with the anti-Hebbian term on the 2nd neuron
+  if (D->p != 2) die_msg("model_arrays_allocate_memory", "only p = 2 (the reference's default) is built");
+  if (D->m != 2) die_msg("model_arrays_allocate_memory", "only m = 2 (the reference's default) is built");
   fv_train_config cfg;
   memset(&cfg, 0, sizeof cfg);
   cfg.vocab = D->vocabulary_size;
@@ -192,6 +201,7 @@ extern "C" void model_arrays_allocate_memory(void *descriptor, void *arrays, int
     A->synapses = (float *)p;
     A->synapses_owned = true;
   }
+  A->shuffle_pending = true;  // flyvec/src/model_arrays.cu:180-198, see upload_corpus
 }
 
 extern "C" void push_INPUT_memory_to_GPU(void *arrays, void *descriptor, int device, const char *type) {
@@ -208,10 +218,40 @@ extern "C" void *get_data_pointer(const char *name, void *arrays, int device) {
   return A->synapses;
 }
 
-extern "C" void set_data_pointer(const char *name, void *arrays, void *ptr, int device) {
+// flyvec/src/model_arrays.cu:320: "INPUT" is a matrix of Ns_1 rows of IM_HEIGHT * IM_WIDTH * Nchannels values, row i
+// being input i. For the text model (type "i4") that is a matrix of windows already cut out: window i starts at
+// token i * row of it. The image types belong to the models that are not built here.
+extern "C" void set_data_pointer(const char *name, void *arrays, void *descriptor, void *ptr, const char *type,
+                                 int device) {
   legacy_arrays *A = (legacy_arrays *)arrays;
+  const legacy_descriptor *D = (const legacy_descriptor *)descriptor;
   one_gpu("set_data_pointer", device);
-  if (!A || !name || !ptr || 0 != strcmp(name, "synapses")) die_msg("set_data_pointer", "only \"synapses\" is served");
+  if (!A || !D || !name || !ptr || !type) die_msg("set_data_pointer", "null argument");
+  if (0 != strcmp(name, "INPUT")) {
+    fprintf(stderr, "set_data_pointer: unknown array %s\n", name);  // what the reference does with another name
+    return;
+  }
+  if (0 != strcmp(type, "i4") && 0 != strcmp(type, "I4"))
+    die_msg("set_data_pointer", "only int32 token ids (type \"i4\") are served: the image models are outside this library");
+  const uint64_t row = D->IM_HEIGHT * D->IM_WIDTH * D->Nchannels;
+  if (row == 0 || D->Ns_1 == 0) die_msg("set_data_pointer", "IM_HEIGHT * IM_WIDTH * Nchannels and Ns_1 must be set first");
+  if (row < D->W) die_msg("set_data_pointer", "a row of the INPUT matrix is shorter than the window W");
+  free(A->starts_owned);
+  A->starts_owned = (uint64_t *)malloc(D->Ns_1 * sizeof(uint64_t));
+  if (!A->starts_owned) die_msg("set_data_pointer", "out of memory");
+  for (uint64_t i = 0; i < D->Ns_1; ++i) A->starts_owned[i] = i * row;
+  A->corpus = (const int32_t *)ptr;
+  A->starts = A->starts_owned;
+  A->n_tokens = D->Ns_1 * row;
+  A->corpus_on_device = false;
+}
+
+// No counterpart in the reference, whose matrix lives in managed memory of its own: makes `ptr` (K x 2V fp32,
+// row-major, host memory of the caller that outlives the model) the matrix get_data_pointer("synapses") serves
+// and the epochs read and write.
+extern "C" void flyvec_legacy_set_synapses(void *arrays, void *ptr) {
+  legacy_arrays *A = (legacy_arrays *)arrays;
+  if (!A || !ptr) die_msg("flyvec_legacy_set_synapses", "null argument");
   if (A->synapses_owned) (void)fv_host_free_pinned(A->synapses);
   A->synapses = (float *)ptr;
   A->synapses_owned = false;
@@ -258,6 +298,7 @@ extern "C" void flyvec_legacy_release(void *descriptor, void *arrays) {
   if (A) {
     if (A->trainer) (void)fv_trainer_destroy(A->trainer);
     if (A->synapses_owned && A->synapses) (void)fv_host_free_pinned(A->synapses);
+    free(A->starts_owned);
     delete A;
   }
   delete (legacy_descriptor *)descriptor;

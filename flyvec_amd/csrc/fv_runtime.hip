@@ -54,6 +54,14 @@ extern "C" int fv_device_info(char *name, size_t name_cap, int *out_compute_unit
   return FV_OK;
 }
 
+extern "C" int fv_device_memory(uint64_t *out_free_bytes, uint64_t *out_total_bytes) {
+  size_t free_b = 0, total_b = 0;
+  FV_HIP(hipMemGetInfo(&free_b, &total_b));
+  if (out_free_bytes) *out_free_bytes = (uint64_t)free_b;
+  if (out_total_bytes) *out_total_bytes = (uint64_t)total_b;
+  return FV_OK;
+}
+
 extern "C" int fv_host_alloc_pinned(size_t bytes, void **out_ptr) {
   FV_REQUIRE(out_ptr, FV_ERR_INVALID, "fv_host_alloc_pinned: null output");
   *out_ptr = nullptr;

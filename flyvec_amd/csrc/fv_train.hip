@@ -108,9 +108,12 @@ static void fv_trainer_free_corpus(fv_trainer *t) {
   t->ahead_valid = false;
 }
 
-// Trainers alive in this process. The single dense launch needs every compute unit for itself: two
-// of them in flight at once, from two trainers' streams, could each hold half the machine and wait
-// for the other half, so the form is only used while one trainer exists.
+// Trainers alive in this process. The single dense launch, where it has to make the pass for max|ds|, exchanges
+// the blocks' maxima inside the launch and so needs every compute unit for itself: two of them in flight at
+// once, from two trainers' streams, could each hold half the machine and wait for the other half. While more
+// than one trainer exists a step therefore enqueues the launch twice, in the form that waits for nobody
+// (fv_dense_args.phase): the first does the whole step whenever max|ds| is known beforehand, the second then
+// ends at once.
 static std::atomic<int> fv_trainers_alive{0};
 
 // After a single dense launch has given up: the trainer goes on with two launches per step, and the marks
@@ -278,14 +281,20 @@ static void fv_choose_onepass(fv_trainer *t, uint64_t cu) {
   const uint32_t rows_per_round = FV_ONEPASS_THREADS / ldk4;
   uint64_t blocks = (t->N + rows_per_round - 1) / rows_per_round;
   if (blocks > cu * FV_ONEPASS_BLOCKS_PER_CU) blocks = cu * FV_ONEPASS_BLOCKS_PER_CU;
+  // every block leaves a share of the rows' largest weights, and the next winner kernel merges one chunk of them
+  if (blocks > FV_MERGE_CHUNK) blocks = FV_MERGE_CHUNK;
   const uint64_t need = (t->N + blocks * rows_per_round - 1) / (blocks * rows_per_round);
   {
     // the streaming form: its sentinel list takes more LDS than a launch may have without asking
     const size_t smem = fv_stream_smem(t);
-    if (hipFuncSetAttribute((const void *)fv_dense_stream_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem) == hipSuccess &&
-        hipFuncSetAttribute((const void *)fv_dense_stream_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem) == hipSuccess)
+    bool set = true;
+#define FV_SET(KERNEL)                                                                                              \
+  set = set && hipFuncSetAttribute((const void *)KERNEL, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess;
+    FV_SET((fv_dense_stream_kernel<false, 0>)) FV_SET((fv_dense_stream_kernel<true, 0>))
+    FV_SET((fv_dense_stream_kernel<false, 1>)) FV_SET((fv_dense_stream_kernel<true, 1>))
+    FV_SET((fv_dense_stream_kernel<false, 2>)) FV_SET((fv_dense_stream_kernel<true, 2>))
+#undef FV_SET
+    if (set)
       t->stream_ok = fv_stream_fits(smem) != 0;
     else
       (void)hipGetLastError();
@@ -693,7 +702,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   // the trainer has them, and a sentinel names a record inside its block's region
   const uint32_t slot_region = grouping_in_sparse && !t->no_block_regions ? t->slot_region : 0u;
   if (slot_region) n_slots = slot_region;
-  const bool onepass = t->onepass && fv_trainers_alive.load() == 1 && n_slots + 1 < FV_SENTINEL_MAX;
+  const bool onepass = t->onepass && n_slots + 1 < FV_SENTINEL_MAX;
+  const bool alone = fv_trainers_alive.load() == 1;
   g.won = nullptr;
   g.won_words = t->won_words;
   if (grouping_in_sparse) {
@@ -838,6 +848,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.w = t->w;
   d.arrive = nullptr;
   d.status = nullptr;
+  d.phase = 0;
   d.epoch = d.spin_limit = d.step_tag = 0;
   d.lmid = t->cfg.lmid;
   d.lbase = t->cfg.lbase;
@@ -894,18 +905,21 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
 #define FV_CASE(U)                                                                     \
   if (anti) fv_launch_onepass<U, true>(d, t->onepass_blocks, smem1, t->stream);        \
   else fv_launch_onepass<U, false>(d, t->onepass_blocks, smem1, t->stream);
-      if (t->onepass_stream) {
-        const dim3 grid(t->onepass_blocks), block(FV_ONEPASS_THREADS);
-        if (anti)
-          hipLaunchKernelGGL(fv_dense_stream_kernel<true>, grid, block, fv_stream_smem(t), t->stream, d);
-        else
-          hipLaunchKernelGGL(fv_dense_stream_kernel<false>, grid, block, fv_stream_smem(t), t->stream, d);
-      } else if (t->onepass_unroll == 8) { FV_CASE(8) } else { FV_CASE(16) }
+      // alone on the device: one launch that exchanges the blocks' maxima itself where it needs them; else the
+      // launch twice, in the form that waits for nobody (both with this step's launch number)
+      for (uint32_t phase = alone ? 0u : 1u; phase <= (alone ? 0u : 2u); ++phase) {
+        d.phase = phase;
+        if (t->onepass_stream) {
+          if (anti) fv_launch_stream<true>(d, t->onepass_blocks, fv_stream_smem(t), t->stream);
+          else fv_launch_stream<false>(d, t->onepass_blocks, fv_stream_smem(t), t->stream);
+        } else if (t->onepass_unroll == 8) { FV_CASE(8) } else { FV_CASE(16) }
+      }
 #undef FV_CASE
       t->top2_valid = true;  // this launch leaves the shares of the matrix it writes
       t->top2_n_part = t->onepass_blocks;
       t->top2_merged = false;  // the next winner kernel's first blocks merge them
-      static_assert(FV_ONEPASS_BLOCKS_PER_CU == 1, "a single dense launch leaves no more shares than one chunk holds");
+      FV_REQUIRE(t->top2_n_part <= FV_MERGE_CHUNK, FV_ERR_STATE, "a single dense launch of %u blocks leaves more shares "
+                 "than the %d one chunk holds", t->top2_n_part, FV_MERGE_CHUNK);
     }
     if (ev) FV_HIP(hipEventRecord(ev[4], t->stream));
   } else {
@@ -1030,7 +1044,10 @@ extern "C" int fv_trainer_run_epoch(fv_trainer *t, uint64_t epoch_id, uint64_t n
     uint32_t tag = 0;
     FV_TRY(fv_trainer_take_giveup(t, &tag));
     if (!tag) return FV_OK;
-    FV_REQUIRE(attempt == 0 && tag != 0xffffffffu, FV_ERR_STATE,
+    FV_REQUIRE(tag != 0xffffffffu, FV_ERR_STATE,
+               "a single dense launch of a step enqueued before this epoch (fv_trainer_step without a fv_trainer_sync "
+               "behind it) had given up: neither that step nor the epoch's steps have changed the matrix");
+    FV_REQUIRE(attempt == 0, FV_ERR_STATE,
                "a dense launch gave up although the epoch was already being redone with two launches per step");
     k_first = (uint64_t)(tag - 1u) * t->B;
     t->giveups_recovered++;
@@ -1094,7 +1111,7 @@ extern "C" int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launch
   // what a sentinel has to number in a step without the anti-Hebbian term
   const bool regions = fv_groups_in_sparse(t) && t->slot_region && !t->no_block_regions;
   const uint64_t n_slots = regions ? t->slot_region : (uint64_t)FV_NB_CLASSES * t->B * t->w;
-  *out_launches = t->onepass && fv_trainers_alive.load() == 1 && n_slots + 1 < FV_SENTINEL_MAX ? 1u : 2u;
+  *out_launches = t->onepass && n_slots + 1 < FV_SENTINEL_MAX ? 1u : 2u;
   return FV_OK;
 }
 
@@ -1176,7 +1193,9 @@ extern "C" int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint3
   FV_HIP(hipEventElapsedTime(out_total_ms, e0, e1));
   (void)hipEventDestroy(e0);
   (void)hipEventDestroy(e1);
-  if (rc != FV_OK || !out_kernel_ms) return rc;
+  if (rc != FV_OK) return rc;
+  FV_TRY(fv_trainer_wait(t));  // a launch that gave up makes the figure one of dead launches: FV_ERR_STATE
+  if (!out_kernel_ms) return FV_OK;
 
   const int per = FV_TRAIN_KERNELS + 1;
   std::vector<hipEvent_t> ev((size_t)n_steps * per);
@@ -1194,7 +1213,8 @@ extern "C" int fv_trainer_time_steps(fv_trainer *t, uint64_t first_window, uint3
       }
   }
   for (auto &e : ev) (void)hipEventDestroy(e);
-  return rc;
+  if (rc != FV_OK) return rc;
+  return fv_trainer_wait(t);
 }
 
 // The same steps as fv_trainer_time_steps, enqueued as HIP graphs: the launches of steps_per_graph consecutive
@@ -1243,7 +1263,7 @@ extern "C" int fv_trainer_time_steps_graph(fv_trainer *t, uint64_t first_window,
   if (e1) (void)hipEventDestroy(e1);
   if (rc != FV_OK) return rc;
   if (e != hipSuccess) return fv_fail(FV_ERR_HIP, "steps as graphs failed: %s", hipGetErrorString(e));
-  return FV_OK;
+  return fv_trainer_wait(t);  // FV_ERR_STATE if a launch gave up: the figure would be one of dead launches
 }
 
 extern "C" int fv_trainer_time_kernel(fv_trainer *t, uint32_t kernel_index, uint32_t reps, float *out_mean_ms) {

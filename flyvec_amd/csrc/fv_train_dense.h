@@ -50,6 +50,13 @@ struct fv_dense_args {
   float2 *top2_part;     // out: the same of the matrix this launch leaves, over each block's share: [block][ldk]
   uint32_t part_base;    // separate launches: the update launch's blocks come first, then the slot launch's four
   uint32_t *path_count;  // [0] launches that knew max|ds| when they started, [1] launches that made the pass for it
+  // Single-launch form without any wait between blocks, for a device the launch may have to share (a process with
+  // more than one trainer): the step enqueues the kernel twice with the same launch number. phase 1 does the
+  // whole step when max|ds| is known beforehand; otherwise it only makes the pass for the maximum and leaves
+  // every block's maximum in its arrival word. phase 2 ends at once in the first case (every block evaluates the
+  // same rule on the same inputs) and in the second reads the words, all written when it starts, and makes the
+  // update. phase 0: one launch, the blocks exchange their maxima inside it (they must be resident together).
+  uint32_t phase;
 };
 
 // ds of a dense element is -xx[h] * W (flyvec/src/cuda_funcs.cu:657-672 without the sparse term). No
@@ -493,10 +500,54 @@ __device__ __forceinline__ void fv_onepass_exchange(const fv_dense_args &a, floa
   }
 }
 
+// Phase 1 of the launch that waits for nobody: the block's maximum m of |ds| into its arrival word, for phase 2.
+__device__ __forceinline__ void fv_onepass_publish(const fv_dense_args &a, float m, float *smem16) {
+  constexpr uint32_t T = FV_ONEPASS_THREADS;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
+  if ((tid & 63) == 0) smem16[tid >> 6] = __uint_as_float(wm);
+  __syncthreads();
+  if (tid < 64) {
+    float bm = tid < T / 64 ? smem16[tid] : 0.0f;
+    bm = __uint_as_float(fv_wave_max_u32(__float_as_uint(bm)));
+    if (tid == 0) {
+      __hip_atomic_store(&a.arrive[blockIdx.x], ((unsigned long long)a.epoch << 32) | __float_as_uint(bm),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (blockIdx.x == 0) a.path_count[1] += 1;
+    }
+  }
+}
+
+// Phase 2: the maxima phase 1 left, one word per block, all of this launch number (the launch that wrote them has
+// ended); the step's scale into *sh_s_out (read behind the caller's next barrier). A word of another number can
+// only mean that phase 1 did not run: the update is then withheld (*sh_ok_out = 0).
+__device__ __forceinline__ void fv_onepass_collect(const fv_dense_args &a, float *sh_s_out, uint32_t *sh_ok_out) {
+  const uint32_t tid = threadIdx.x;
+  if (tid < 64) {
+    uint32_t mx = 0;
+    bool all = true;
+    for (uint32_t i = tid; i < gridDim.x; i += 64) {
+      const unsigned long long v = __hip_atomic_load(&a.arrive[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      all = all && (uint32_t)(v >> 32) == a.epoch;
+      mx = max(mx, (uint32_t)v);
+    }
+    mx = fv_wave_max_u32(mx);
+    const bool go = __all(all);
+    if (tid == 0) {
+      const float nc = __uint_as_float(mx);
+      *sh_s_out = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
+      *sh_ok_out = go;
+      if (blockIdx.x == 0) a.scalars[0] = go ? nc : __uint_as_float(0x7fc00000u);
+    }
+  }
+}
+
 static_assert(FV_MAX_HID <= 2 * FV_ONEPASS_THREADS, "two neurons per thread cover every row");
 static_assert(FV_NB_CLASSES == 4, "a neuron's block maxima and hit counts are read as one 16-byte word each");
 
-template <int U, bool DELTA>
+// PHASE: fv_dense_args.phase, fixed at compile time (the branches of the other phases cost the register form
+// its last registers).
+template <int U, bool DELTA, int PHASE = 0>
 __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv_dense_args a) {
   constexpr uint32_t T = FV_ONEPASS_THREADS;
   constexpr int DEPTH = FV_ONEPASS_DEPTH < U ? FV_ONEPASS_DEPTH : U;
@@ -538,10 +589,14 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   const uint32_t limit = dead ? 0u : a.spin_limit;
   float4 w[U];
   __builtin_amdgcn_sched_barrier(0);  // nothing that uses a small load moves up between the loads of W
-#pragma unroll
-  for (int u = 0; u < DEPTH; ++u) {
-    const uint32_t row = row0 + u * row_step;
-    w[u] = a.Wt4[(row < a.n_rows ? row : row_inside) * a.ldk4 + q];
+  // (phase 2 usually ends behind the decision: it asks for the matrix only once it knows that it goes on)
+#define FV_ONEPASS_FIRST_LOADS                                            \
+  _Pragma("unroll") for (int u = 0; u < DEPTH; ++u) {                     \
+    const uint32_t row = row0 + u * row_step;                             \
+    w[u] = a.Wt4[(row < a.n_rows ? row : row_inside) * a.ldk4 + q];       \
+  }
+  if (PHASE != 2) {
+    FV_ONEPASS_FIRST_LOADS
   }
   __builtin_amdgcn_sched_barrier(0);
   // the next minibatch's column indices, by all waves but the first: the window's start now
@@ -583,6 +638,9 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   }
   const bool fast = a.top2_known && F <= max(S, E);  // the same answer in every thread of every block
   const float4 xq = ((const float4 *)xs)[q];
+  if (PHASE == 2 && fast) return;  // phase 1 has made the whole step
+  // the rows are streamed (loaded as their turn comes, updated, stored) rather than held from a pass for the maximum
+  const bool streams = fast || PHASE == 2;
 
   float s;
   bool ok = true;
@@ -594,6 +652,12 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
       a.scalars[0] = nc;
       a.path_count[0] += 1;
     }
+  } else if (PHASE == 2) {
+    FV_ONEPASS_FIRST_LOADS
+    fv_onepass_collect(a, &sh_s, &sh_ok);
+    __syncthreads();
+    ok = sh_ok != 0 && !dead;
+    s = sh_s;
   } else {
     // the pass for the maximum, on registers; the loads not yet issued take the places of those used
     float m = __uint_as_float(S);
@@ -606,12 +670,17 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
         w[u + DEPTH] = a.Wt4[(rown < a.n_rows ? rown : row_inside) * a.ldk4 + q];
       }
     }
+    if (PHASE == 1) {  // the update is phase 2's
+      fv_onepass_publish(a, m, smem16);
+      return;
+    }
     fv_onepass_exchange(a, m, limit, dead, smem16, &sh_s, &sh_ok);
     fv_sample_ahead(a, samples0, e0, er0, start0, ahead_entries, TS);  // while the first wave waits
     __syncthreads();
     ok = sh_ok != 0;
     s = sh_s;
   }
+#undef FV_ONEPASS_FIRST_LOADS
 
   // The update. A group without a sentinel is stored whole where something changed; in a group with
   // one the other elements are stored one by one and the sentinel is noted for later. The two largest
@@ -620,7 +689,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   // rows, so that a corpus too large for the Infinity Cache does not lengthen the launch's tail
   const uint32_t c0 = e0 - er0 * a.idx_stride;
   int32_t tok0 = -1;
-  if (fast && samples0 && c0 < a.w) tok0 = a.corpus[start0 + c0];
+  if (streams && samples0 && c0 < a.w) tok0 = a.corpus[start0 + c0];
   float t1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, t2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   // A sentinel that finds the block's list full is finished by its own thread behind the stream (bit 4 u + e:
   // element e of the thread's group u), from memory, where it still stands.
@@ -655,13 +724,13 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
       }
       fv_top2_insert_four(t1, t2, v, has_nan);
     }
-    if (fast && u + DEPTH < U) {  // the next load takes the place of the one just used
+    if (streams && u + DEPTH < U) {  // the next load takes the place of the one just used
       const uint32_t rown = row0 + (u + DEPTH) * row_step;
       w[u + DEPTH] = a.Wt4[(rown < a.n_rows ? rown : row_inside) * a.ldk4 + q];
     }
   }
 #undef FV_ONEPASS_ELEMENT
-  if (fast) {
+  if (streams) {
     if (samples0) a.idx_ahead[e0] = c0 < a.w ? fv_column_index(tok0, c0, a.w, a.V) : -1;
     fv_sample_ahead(a, false, e0, er0, start0, ahead_entries, TS);  // the entries beyond the first, if any
   }
@@ -706,7 +775,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
 #endif
 #define FV_STREAM_HIT_CAP 8192  // sentinels a block notes in LDS (64 KB)
 
-template <bool DELTA>
+template <bool DELTA, int PHASE = 0>
 __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_dense_args a) {
   constexpr uint32_t T = FV_ONEPASS_THREADS;
   constexpr int D = FV_STREAM_DEPTH;
@@ -744,8 +813,11 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
   const uint32_t limit = dead ? 0u : a.spin_limit;
   float4 w[D];
   auto group_of = [&](uint32_t row) { return (row < a.n_rows ? row : row_inside) * a.ldk4 + q; };
+  // (phase 2 usually ends behind the decision: it asks for the matrix only once it knows that it goes on)
+  if (PHASE != 2) {
 #pragma unroll
-  for (int u = 0; u < D; ++u) w[u] = a.Wt4[group_of(row0 + u * row_step)];
+    for (int u = 0; u < D; ++u) w[u] = a.Wt4[group_of(row0 + u * row_step)];
+  }
   constexpr uint32_t TS = T - 64;
   const uint32_t ahead_entries = a.ahead_n * a.idx_stride;
   const uint32_t e0 = blockIdx.x * TS + (tid - 64);
@@ -783,6 +855,9 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
   }
   const bool fast = a.top2_known && F <= max(S, E);
   const float4 xq = ((const float4 *)xs)[q];
+  if (PHASE == 2 && fast) return;  // phase 1 has made the whole step
+  // the next minibatch is sampled beside the update's stream rather than during a wait
+  const bool streams = fast || PHASE == 2;
 
   float s;
   bool ok = true;
@@ -794,6 +869,13 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
       a.scalars[0] = nc;
       a.path_count[0] += 1;
     }
+  } else if (PHASE == 2) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) w[u] = a.Wt4[group_of(row0 + u * row_step)];
+    fv_onepass_collect(a, &sh_s, &sh_ok);
+    __syncthreads();
+    ok = sh_ok != 0 && !dead;
+    s = sh_s;
   } else {
     float m = __uint_as_float(S);
     for (uint32_t c = 0; c < rounds; c += D) {
@@ -803,6 +885,10 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
         if (active && row < a.n_rows) m = fv_absmax_four(m, xq, w[u]);
         w[u] = a.Wt4[group_of(row + D * row_step)];
       }
+    }
+    if (PHASE == 1) {  // the update is phase 2's
+      fv_onepass_publish(a, m, smem16);
+      return;
     }
     fv_onepass_exchange(a, m, limit, dead, smem16, &sh_s, &sh_ok);
     fv_sample_ahead(a, samples0, e0, er0, start0, ahead_entries, TS);  // while the first wave waits
@@ -816,7 +902,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
   // (as in fv_dense_onepass_kernel: the first token of the minibatch sampled ahead travels during the stream)
   const uint32_t c0 = e0 - er0 * a.idx_stride;
   int32_t tok0 = -1;
-  if (fast && samples0 && c0 < a.w) tok0 = a.corpus[start0 + c0];
+  if (streams && samples0 && c0 < a.w) tok0 = a.corpus[start0 + c0];
   float t1[4] = {0.0f, 0.0f, 0.0f, 0.0f}, t2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #define FV_STREAM_ELEMENT(member, lane4)                                                       \
   if (v.member == v.member) {                                                                  \
@@ -852,7 +938,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
     }
   }
 #undef FV_STREAM_ELEMENT
-  if (fast) {
+  if (streams) {
     if (samples0) a.idx_ahead[e0] = c0 < a.w ? fv_column_index(tok0, c0, a.w, a.V) : -1;
     fv_sample_ahead(a, false, e0, er0, start0, ahead_entries, TS);
   }
@@ -880,9 +966,9 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_stream_kernel(fv_
 
 static int fv_stream_fits(size_t smem) {
   int nb = 0, nb2 = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fv_dense_stream_kernel<false>, FV_ONEPASS_THREADS, smem) !=
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (fv_dense_stream_kernel<false, 0>), FV_ONEPASS_THREADS, smem) !=
           hipSuccess ||
-      hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb2, fv_dense_stream_kernel<true>, FV_ONEPASS_THREADS, smem) !=
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb2, (fv_dense_stream_kernel<true, 0>), FV_ONEPASS_THREADS, smem) !=
           hipSuccess) {
     (void)hipGetLastError();
     return 0;
@@ -892,15 +978,32 @@ static int fv_stream_fits(size_t smem) {
 
 template <int U, bool DELTA>
 static void fv_launch_onepass(const fv_dense_args &d, unsigned blocks, size_t smem, hipStream_t stream) {
-  hipLaunchKernelGGL((fv_dense_onepass_kernel<U, DELTA>), dim3(blocks), dim3(FV_ONEPASS_THREADS), smem, stream, d);
+  const dim3 grid(blocks), block(FV_ONEPASS_THREADS);
+  if (d.phase == 0)
+    hipLaunchKernelGGL((fv_dense_onepass_kernel<U, DELTA, 0>), grid, block, smem, stream, d);
+  else if (d.phase == 1)
+    hipLaunchKernelGGL((fv_dense_onepass_kernel<U, DELTA, 1>), grid, block, smem, stream, d);
+  else
+    hipLaunchKernelGGL((fv_dense_onepass_kernel<U, DELTA, 2>), grid, block, smem, stream, d);
+}
+
+template <bool DELTA>
+static void fv_launch_stream(const fv_dense_args &d, unsigned blocks, size_t smem, hipStream_t stream) {
+  const dim3 grid(blocks), block(FV_ONEPASS_THREADS);
+  if (d.phase == 0)
+    hipLaunchKernelGGL((fv_dense_stream_kernel<DELTA, 0>), grid, block, smem, stream, d);
+  else if (d.phase == 1)
+    hipLaunchKernelGGL((fv_dense_stream_kernel<DELTA, 1>), grid, block, smem, stream, d);
+  else
+    hipLaunchKernelGGL((fv_dense_stream_kernel<DELTA, 2>), grid, block, smem, stream, d);
 }
 
 template <int U>
 static int fv_onepass_fits(size_t smem) {
   int nb = 0, nb2 = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, fv_dense_onepass_kernel<U, false>, FV_ONEPASS_THREADS,
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (fv_dense_onepass_kernel<U, false, 0>), FV_ONEPASS_THREADS,
                                                    smem) != hipSuccess ||
-      hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb2, fv_dense_onepass_kernel<U, true>, FV_ONEPASS_THREADS,
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb2, (fv_dense_onepass_kernel<U, true, 0>), FV_ONEPASS_THREADS,
                                                    smem) != hipSuccess) {
     (void)hipGetLastError();
     return 0;

@@ -275,6 +275,7 @@ class Hasher:
         h = C.c_void_p()
         check(self.lib.fv_hasher_create(ptr(W), self.hid, self.n_columns, C.byref(h)))
         self.handle = h
+        self.version = 0  # counts the changes of the resident matrix (what is derived from it goes stale)
 
     def close(self):
         if getattr(self, "handle", None) is not None and self.handle.value:
@@ -288,15 +289,19 @@ class Hasher:
             pass
 
     def normalize(self, prec=1.0e-32, p=2):
-        """flyvec/core.py:23-36 on the resident matrix: the two passes over the matrix run on the
-        device; the p-th root of the K row sums is numpy's, as in the reference."""
-        if p != 2:
-            raise NotImplementedError("only p = 2 (the reference's default) is built")
+        """flyvec/core.py:23-36 on the resident matrix, p a positive integer: the two passes over the
+        matrix run on the device; the p-th root of the K row sums is numpy's, as in the reference. Equal to the
+        reference bit for bit for p = 1 and p = 2 (its default, all its own code uses); from p = 3 on numpy's
+        float32 power is the C library's powf and the result agrees to rounding."""
+        if int(p) != p or not 1 <= p <= 64:
+            raise ValueError(f"p = {p}: the norm's exponent must be an integer from 1 to 64")
+        p = int(p)
         sums = np.empty(self.hid, dtype=np.float32)
-        check(self.lib.fv_hasher_row_sumsq(self.handle, ptr(sums)))
+        check(self.lib.fv_hasher_row_sum_pow(self.handle, p, ptr(sums)))
         nc = np.power(sums, 1 / p).reshape(self.hid, 1)
         div = np.ascontiguousarray((nc + prec).reshape(-1), dtype=np.float32)
         check(self.lib.fv_hasher_scale_rows(self.handle, ptr(div)))
+        self.version += 1
 
     def weights(self):
         out = np.empty((self.hid, self.n_columns), dtype=np.float32)

@@ -42,6 +42,8 @@ int fv_device_count(int *out_count);
 int fv_set_device(int device);
 /* Name, compute units and HBM bytes of the current device (for logs and the bench). */
 int fv_device_info(char *name, size_t name_cap, int *out_compute_units, uint64_t *out_hbm_bytes);
+/* Free and total memory of the current device as the runtime reports them (either may be NULL). */
+int fv_device_memory(uint64_t *out_free_bytes, uint64_t *out_total_bytes);
 
 /* flyvec/src/cuda_helpers.cu:22 do_gpu_cudaHostAlloc (pinned host staging memory) */
 int fv_host_alloc_pinned(size_t bytes, void **out_ptr);
@@ -79,13 +81,14 @@ int fv_build_window_starts(const uint64_t *offsets, uint64_t n_chunks, uint64_t 
  * reference's fp32 counter does. */
 int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, uint64_t vocab, float *out_invf);
 
-/* fv_inverse_frequency for callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Corpus
- * and output are DEVICE memory of the caller (fv_dev_alloc or any other device allocation); the
- * occurrence counters live in an array built into the library (4 MiB on every device the library
- * runs on, kept until the process ends), so vocab is at most 2^20 = 1,048,576 ids and a larger one is
- * refused with FV_ERR_INVALID. Calls nothing that allocates or frees; runs on the default stream and
- * returns when the result is in out_invf_dev. FV_ERR_DATA on an id >= vocab (the output then ignores
+/* fv_inverse_frequency for callers that cannot allocate device memory (tight serving loops, harnesses
+ * that forbid hipMalloc, a process whose device memory is all spoken for). It has no counterpart in the
+ * reference. Corpus and output are DEVICE memory of the caller (fv_dev_alloc or any other device
+ * allocation); the occurrence counters live in an array built into the library (4 MiB on every device
+ * the library runs on, kept until the process ends), so vocab is at most 2^20 = 1,048,576 ids and a
+ * larger one is refused with FV_ERR_INVALID. Calls nothing that allocates or frees. It runs on the
+ * default stream and ends with a blocking copy of the id range to the host: it returns when the result
+ * is in out_invf_dev, and is not itself a sequence a HIP graph could capture. FV_ERR_DATA on an id >= vocab (the output then ignores
  * such ids). All calls on one device share that device's array: calls that overlap on one device
  * race, results of calls made one after the other do not depend on earlier ones. */
 int fv_inverse_frequency_static(const int32_t *corpus_dev, uint64_t n_tokens, uint64_t vocab,
@@ -205,9 +208,11 @@ int fv_trainer_get_giveups_recovered(fv_trainer *t, uint64_t *out_count);
  * the matrix kept in registers between the passes where it fits them (64 MiB on 256 compute units), with its
  * rows streamed through the registers otherwise. launches = 1 asks for the single launch (FV_ERR_INVALID where
  * there is none), 3 for its streaming form whatever the matrix size, 2 for separate launches (maximum, update,
- * sparse elements), 0 returns to the choice made at creation. Results are bit-identical in all forms. The single
- * launch needs the whole device for itself, so while a process holds more than one trainer every
- * step takes separate launches whatever is set here. */
+ * sparse elements), 0 returns to the choice made at creation. Results are bit-identical in all forms. Where the
+ * single launch has to make the pass for max|ds| its blocks exchange their maxima inside the launch and need the
+ * whole device for themselves; while a process holds more than one trainer a step therefore enqueues the launch
+ * twice in a form that waits for nobody: the first does the whole step when max|ds| is known beforehand (the
+ * usual case) and the second ends at once, else the first makes the pass and the second the update. */
 int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches);
 /* The single launch carries the two largest |W| of every row from step to step; from them and from what
  * the sparse-element launch reports it usually knows max|ds| (flyvec/src/cu_special_reduction.cu:241) before
@@ -215,13 +220,15 @@ int fv_trainer_set_dense_launches(fv_trainer *t, uint32_t launches);
  * maximum first, on registers. Counts of single launches so far that knew it / that made the pass (the
  * first step on a new matrix always makes it). Same results either way. No counterpart in the reference. */
 int fv_trainer_get_dense_path_counts(fv_trainer *t, uint64_t *out_known, uint64_t *out_pass);
-int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches); /* 1 or 2: the form the next step takes */
+/* The form the next step takes: 1 = the single launch (after fv_trainer_set_dense_launches(1) or (3), its
+ * register or its streaming form, as the matrix size and that call decide), 2 = separate launches. */
+int fv_trainer_get_dense_launches(fv_trainer *t, uint32_t *out_launches);
 /* Grouping the windows of a step by winner (what flyvec/src/cuda_funcs.cu:1719-1721 leaves in
  * max_IDs and xx) runs inside the sparse-element launch when the trainer's batch is at most 16384
  * windows and the step has no anti-Hebbian term, as a launch of its own otherwise. separate = 1 forces the launch of its
  * own, 0 returns to that rule. Results are bit-identical either way. */
 int fv_trainer_set_grouping_launch(fv_trainer *t, uint32_t separate);
-int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate);
+int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate); /* the form a step without the anti-Hebbian term takes */
 /* Where the sparse-element launch that groups for itself keeps a step's records of sparse elements (the
  * weight, count and 1/frequency of each element the minibatch touches: the sparse operand of
  * flyvec/src/cuda_funcs.cu:657-672). per_block = 1, the default: every block of that launch has room of its own
@@ -234,7 +241,7 @@ int fv_trainer_set_slot_regions(fv_trainer *t, uint32_t per_block);
  * list and finishes them when its dense elements are done; an element that finds the list full is finished on
  * the spot. entries > 0 makes the list count as full after that many (no more than it holds: 2048, or 8192 in
  * the streaming form), 0 restores its size. Results are bit-identical. No counterpart in the reference. */
-int fv_trainer_set_sentinel_list(fv_trainer *t, uint32_t entries); /* the form a step without the anti-Hebbian term takes */
+int fv_trainer_set_sentinel_list(fv_trainer *t, uint32_t entries);
 /* Test hook: between its two passes a single-launch dense pass waits for all its blocks, at most
  * `rounds` polling rounds (2^14 by default, tens of milliseconds); 0 makes every block give up at once, which
  * is how the error path of fv_trainer_sync is exercised. No counterpart in the reference. */
@@ -288,6 +295,11 @@ int fv_hasher_normalize(fv_hasher *h, float prec);
  * (numpy's power(x, 1/p) is what the reference calls): out_sums[r] = sum_i W[r][i]^2 in numpy's
  * pairwise fp32 order; then W[r][:] /= divisors[r]. */
 int fv_hasher_row_sumsq(fv_hasher *h, float *out_sums /* hid */);
+/* The same for another integer exponent of the norm (flyvec/core.py:23 takes p): out_sums[r] = sum_i W[r][i]^p in the
+ * same order. p = 1 and p = 2 restate numpy exactly (the value, the fp32 product); from p = 3 on numpy's float32
+ * power is the C library's powf, and the power taken here -- the product in double, rounded to fp32 once -- can
+ * differ from it in the last bit of an element. 1 <= p <= 64. */
+int fv_hasher_row_sum_pow(fv_hasher *h, uint32_t p, float *out_sums /* hid */);
 int fv_hasher_scale_rows(fv_hasher *h, const float *divisors /* hid */);
 /* Current resident matrix, K x N row-major. */
 int fv_hasher_get_weights(fv_hasher *h, float *out_W);

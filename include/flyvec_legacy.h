@@ -44,13 +44,18 @@ void print_model_params(void *descriptor);                                   /* 
 
 /* ---- model_arrays.so (flyvec/src/model_arrays.cu) ------------------------------------------------ */
 void *model_create_arrays(int num_gpus);                                               /* :15 */
-void model_arrays_allocate_memory(void *descriptor, void *arrays, int num_gpus);       /* :22 creates the trainer */
+/* :22 creates the trainer; p and m other than 2 (the reference's defaults, which its driver never sets) are refused;
+ * the shuffle of the window order that the reference makes here (:180-198) is applied as soon as the order exists */
+void model_arrays_allocate_memory(void *descriptor, void *arrays, int num_gpus);
 void push_INPUT_memory_to_GPU(void *arrays, void *descriptor, int device, const char *type); /* :250 the corpus is
                                                                                           always resident here */
 /* :305 "synapses": K x 2V fp32 row-major in page-locked host memory; the driver fills it before the first
  * epoch and saves it after any epoch. launch_epoch_INPUT_AS_INT uploads it first and downloads it last. */
 void *get_data_pointer(const char *name, void *arrays, int device);
-void set_data_pointer(const char *name, void *arrays, void *ptr, int device);          /* :320 "synapses" only */
+/* :320 "INPUT", type "i4": a matrix of Ns_1 windows already cut out, IM_HEIGHT * IM_WIDTH * Nchannels (>= W) token
+ * ids per row; 1/frequency is then counted over that matrix. The image types ("f", "u1") report that they are
+ * outside this library and exit; another name is reported and ignored, as in the reference. */
+void set_data_pointer(const char *name, void *arrays, void *descriptor, void *ptr, const char *type, int device);
 /* :358 type "i4": the corpus (int32) and the window-start table compute_offset_phrases wrote */
 void set_up_INPUT_pointer(const char *name, void *arrays, void *descriptor, void *corpus, void *starts,
                           const char *type, int device);
@@ -61,6 +66,9 @@ void do_reshuffle_indices(void *descriptor, void *arrays, int device);          
 /* No counterpart in the reference (it never frees its handles): destroys the trainer, the matrix and both
  * handles. For hosts that create more than one model in a process. */
 void flyvec_legacy_release(void *descriptor, void *arrays);
+/* No counterpart in the reference (its matrix is managed memory of its own): from now on get_data_pointer("synapses")
+ * serves `ptr`, K x 2V fp32 row-major in host memory of the caller, and the epochs read and write it. */
+void flyvec_legacy_set_synapses(void *arrays, void *ptr);
 
 /* ---- cuda_funcs.so (flyvec/src/cuda_funcs.cu) ---------------------------------------------------- */
 /* :1220 one epoch over the current window order */

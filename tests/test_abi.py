@@ -107,7 +107,8 @@ def test_legacy_surface_is_declared_and_exported(tmp_path):
     assert set(LEGACY_SYMBOLS) <= declared
     lib = C.CDLL(str(_lib.LIB_PATH))
     assert not [s for s in LEGACY_SYMBOLS if not hasattr(lib, s)]
-    assert hasattr(lib, "flyvec_legacy_release") and "flyvec_legacy_release" in declared   # the one addition
+    for extra in ("flyvec_legacy_release", "flyvec_legacy_set_synapses"):                # the two additions
+        assert hasattr(lib, extra) and extra in declared
     links = build.install_legacy_names(tmp_path / "bin")
     assert sorted(p.name for p in links) == sorted(build.LEGACY_NAMES)
     for p in links:                                    # each name opens the one library

@@ -27,6 +27,24 @@ def test_cli_trains_saves_resumes(gpu, oracle_lib, tmp_path):
     assert W2.shape == (K, 2 * V) and W2.dtype == np.float32 and W2.flags.c_contiguous
     assert np.isfinite(W2).all()
 
+    # the checker over the same initial matrix and the same window orders (flyvec/train_flyvec.py:241, 253-263:
+    # normal(mu, sigma) weights, a reshuffle before every epoch, eps = lr0 (1 - ep / Nep)) gives the same checkpoints
+    from flyvec_amd import Trainer
+    to = oracle_lib
+    Wo = np.float32(np.random.default_rng(1).normal(0.0, 0.02, (K, 2 * V)))
+    t = Trainer(V, K, w, B)
+    t.set_corpus(tokens, offsets)
+    starts, invf = to.window_starts(offsets, w), to.inverse_frequency(tokens, V)
+    assert t.num_windows == len(starts) and len(starts) % B != 0
+    t.shuffle(1)
+    for ep in range(3):
+        t.shuffle(1 + 1 + ep)
+        to.train_steps(Wo, tokens, starts, t.get_permutation(), 0, B, len(starts) // B + 1, w, invf,
+                       to.epoch_eps(0.002, ep, 3))
+        if ep >= 1:
+            assert np.array_equal(np.load(out / names[ep - 1]).view(np.uint32), Wo.view(np.uint32)), f"epoch {ep}"
+    t.close()
+
     # same seed: same checkpoints
     out2 = tmp_path / "ckpt2"
     argv2 = list(argv)

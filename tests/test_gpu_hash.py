@@ -23,9 +23,10 @@ def test_config1_target_ids(gpu):
 
 
 def test_config3_window_batch(gpu):
-    """K = 400, V = 20000, 1,048,576 windows of w = 11, k = 32, 7 packed words per window.  The first
-    262,144 windows are compared with the numpy oracle bit for bit (CPU time bounds the sample); the
-    whole batch is checked through popcount, packed-vs-int8 agreement and repeatability."""
+    """K = 400, V = 20000, 1,048,576 windows of w = 11, k = 32, 7 packed words per window: every window of the
+    batch is compared with the numpy oracle bit for bit (the oracle's chunks are dealt over a few threads; numpy
+    releases the interpreter lock inside its loops)."""
+    from concurrent.futures import ThreadPoolExecutor
     from flyvec_amd import Hasher, synthetic
     from oracle import hash_oracle as ho
     K, V, w, k, n = 400, 20000, 11, 32, 1 << 20
@@ -34,9 +35,12 @@ def test_config3_window_batch(gpu):
     h = Hasher(W)
     bits = h.hash_windows(idx, k, packed=True)
     assert bits.shape == (n, 7) and bits.dtype == np.uint64
-    m = 1 << 18
-    want = ho.hash_windows(W, idx[:m], k)
-    assert np.array_equal(bits[:m], ho.pack_codes(want))
+    part = 1 << 15
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        want = list(pool.map(lambda s: ho.pack_codes(ho.hash_windows(W, idx[s:s + part], k)), range(0, n, part)))
+    want = np.concatenate(want)
+    assert want.shape == bits.shape
+    assert np.array_equal(bits, want)
     pop = np.unpackbits(bits.view(np.uint8), axis=1).sum(axis=1)
     assert pop.max() <= k and (pop == k).mean() > 0.999          # exactly k bits unless fp32 ties
     assert not (bits[:, 6] >> np.uint64(16)).any()                  # no bit beyond neuron 399
@@ -119,6 +123,72 @@ def test_normalize_matches_numpy(gpu):
         h.normalize()
         assert np.array_equal(h.weights(), ho.normalize_synapses(W)), (K, N)
         h.close()
+
+
+@pytest.mark.parametrize("p", [1, 2, 3, 4, 7])
+def test_normalize_with_another_exponent(gpu, p):
+    """flyvec/core.py:23 takes the exponent of the norm. p = 1 and p = 2 are numpy's fast paths (the value, the
+    fp32 product) and the device restates them exactly; from p = 3 on numpy's float32 power is the C library's
+    powf, whose last bit is not pinned by anything the reference holds (parity unpinned for that case): the device
+    takes the product in double, rounded once, and the normalised matrix agrees to rounding."""
+    from flyvec_amd import Hasher
+    from oracle import hash_oracle as ho
+    rng = np.random.default_rng(50 + p)
+    for K, N in ((37, 2 * 4097), (400, 2000)):
+        W = (rng.standard_normal((K, N)) * 10.0 ** rng.integers(-1, 2, size=(K, 1))).astype(f32)
+        if p % 2:
+            W = np.abs(W)                     # an odd power of a mixed-sign row sums to anything, its root to NaN
+        h = Hasher(W)
+        h.normalize(p=p)
+        got, want = h.weights(), ho.normalize_synapses(W, p=p)
+        assert np.isfinite(want).all()
+        if p <= 2:
+            assert np.array_equal(got, want), (K, N)
+        else:
+            assert np.allclose(got, want, rtol=2e-6, atol=0.0), (K, N)
+        h.close()
+    h = Hasher(W)
+    for bad in (0, -2, 1.5, 65):
+        with pytest.raises(ValueError):
+            h.normalize(p=bad)
+    h.close()
+
+
+def test_code_table_serves_the_per_word_calls(gpu):
+    """FlyVec.get_sparse_embedding reads a table of the whole vocabulary's codes, computed on the device by one
+    batched launch per hash length: its rows equal the launches per id and the numpy oracle's per-word path
+    (flyvec/core.py:153-158) bit for bit, and it is computed again when the resident matrix changes."""
+    from flyvec_amd import FlyVec
+    from oracle import hash_oracle as ho
+    rng = np.random.default_rng(12)
+    K, V = 400, 700
+    vocab = ["<UNK>"] + [f"t{i}" for i in range(1, V)]
+    W = rng.standard_normal((K, 2 * V)).astype(f32)
+    model = FlyVec(W, tokenizer=vocab, normalize_synapses=False)
+    for k in (50, 32, 1, 399):
+        table = model.code_table(k)
+        assert table.shape == (V, K) and table.dtype == np.int8 and not table.flags.writeable
+        assert model.code_table(k) is table                                    # kept, not computed again
+        assert np.array_equal(table, ho.hash_targets_loop(W, np.arange(V), k))
+        for i in (1, 2, 17, V - 1):
+            one = model.hasher.hash_targets([i], k)[0]                         # a launch of its own
+            emb = model.get_sparse_embedding(f"t{i}", k)
+            assert emb["id"] == i and emb["token"] == f"t{i}" and emb["embedding"].flags.writeable
+            assert np.array_equal(emb["embedding"], one) and np.array_equal(one, table[i])
+            assert np.array_equal(model.get_sparse_embedding(i, k)["embedding"], one)   # by id
+    with pytest.raises(IndexError):
+        model.code_table(K)                                                    # the reference reads act_sort[k]
+    with pytest.raises(IndexError):
+        model.get_sparse_embedding(V, 50)
+    assert len(model._code_tables) <= FlyVec.CODE_TABLES_KEPT
+    # a change of the resident matrix makes the tables stale
+    before = model.code_table(50)
+    model.hasher.normalize()
+    Wn = ho.normalize_synapses(W)
+    after = model.code_table(50)
+    assert after is not before and np.array_equal(after, ho.hash_targets_loop(Wn, np.arange(V), 50))
+    assert np.array_equal(model.synapses, Wn)
+    assert np.array_equal(model.get_sparse_embedding("t5")["embedding"], ho.sparse_code(Wn[:, V + 5], 50))
 
 
 def test_flyvec_wrapper_semantics(gpu, tmp_path):

@@ -4,6 +4,8 @@ The step is deterministic by construction (window-ordered xx, count-based sparse
 comparison is bit for bit: identical winners and identical W.  The bars the task states
 (winners >= 99.9 %, relative L2 of W <= 1e-4 after 100 steps) are asserted as well, at the
 benchmark's full size."""
+import functools
+
 import numpy as np
 import pytest
 
@@ -154,6 +156,16 @@ def test_single_dense_launch_gives_up_cleanly(gpu, oracle_lib, form):
     assert e.value.code == _lib.FV_ERR_STATE
     assert t.dense_launches == 2
     t.sync()                                   # reported once
+    assert np.array_equal(t.get_weights(), W0)
+    # the measurement hooks report it too: a figure over launches that neither waited nor updated is no figure
+    t.set_dense_launches(form)
+    with pytest.raises(_lib.FlyvecError) as e:
+        t.time_steps(0, 3, 1e-3, per_kernel=False)
+    assert e.value.code == _lib.FV_ERR_STATE
+    t.set_dense_launches(form)
+    with pytest.raises(_lib.FlyvecError) as e:
+        t.time_steps_graph(0, 2, 1e-3, 1)
+    assert e.value.code == _lib.FV_ERR_STATE
     assert np.array_equal(t.get_weights(), W0)
     starts, invf = oracle_inputs(to, tokens, offsets, V, w)
     for launches in (2, form):                 # usable afterwards, in either form
@@ -375,8 +387,11 @@ def test_steps_in_any_order_and_across_order_changes(gpu, oracle_lib, launches):
 
 
 def test_two_trainers_side_by_side(gpu, oracle_lib):
-    """The single dense launch wants every compute unit, so two trainers in one process both take two launches
-    (steps of both are enqueued without a synchronisation in between here); alone again, a trainer returns to one."""
+    """Where the single dense launch has to make the pass for max|ds| its blocks exchange their maxima inside the
+    launch and want every compute unit, so while a process holds two trainers a step enqueues the launch twice in
+    the form that waits for nobody (steps of both are enqueued without a synchronisation in between here). Both
+    trainers, the first steps on a new matrix (the pass) and the later ones (max|ds| known) included, train to the
+    checker's bits; alone again, a trainer returns to the one launch."""
     from flyvec_amd import synthetic
     to = oracle_lib
     V, K, w, B = 300, 64, 7, 128
@@ -386,11 +401,13 @@ def test_two_trainers_side_by_side(gpu, oracle_lib):
     a, perm_a = make_trainer(tokens, offsets, V, K, w, B, Wa, perm_seed=6)
     assert a.dense_launches == 1
     b, perm_b = make_trainer(tokens, offsets, V, K, w, B, Wb, perm_seed=7)
-    assert a.dense_launches == 2 and b.dense_launches == 2
+    assert a.dense_launches == 1 and b.dense_launches == 1
     for s in range(6):
         a.step(s * B, B, 1e-3)
         b.step(s * B, B, 1e-3)
     b.sync()
+    known, made = b.dense_path_counts
+    assert known + made == 6 and made >= 1 and known >= 3
     Wo = Wb.copy()
     to.train_steps(Wo, tokens, starts, perm_b, 0, B, 6, w, invf, 1e-3)
     assert np.array_equal(b.get_weights(), Wo)
@@ -401,7 +418,51 @@ def test_two_trainers_side_by_side(gpu, oracle_lib):
     Wo = Wa.copy()
     to.train_steps(Wo, tokens, starts, perm_a, 0, B, 9, w, invf, 1e-3)
     assert np.array_equal(a.get_weights(), Wo)
+    assert sum(a.dense_path_counts) == 9
     a.close()
+
+
+@pytest.mark.parametrize("launches", [1, 3])
+def test_second_trainer_alive_while_the_pass_for_the_maximum_is_needed(gpu, oracle_lib, launches):
+    """The form of the single dense launch that waits for nobody (a second trainer exists in the process), on
+    weights whose largest entries sit on the most frequent tokens: nearly every step has to make the pass for
+    max|ds|, which the first of the two launches then makes and the second follows with the update. Step by
+    step against the checker, in the register and in the streaming form, run_epoch's partial last minibatch
+    included."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    V, K, w, B = 800, 96, 9, 2000
+    tokens, offsets = small_corpus(80000, V, seed=2)
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    perm = np.random.default_rng(3).permutation(len(starts)).astype(np.uint64)
+    hot = np.argsort(-np.bincount(tokens[tokens >= 0], minlength=V))[:6]
+    planted = synthetic.synapses(K, V, seed=9)
+    planted[:, hot[:3]] = np.float32(7.0)
+    other = Trainer(50, 8, 3, 16)                    # idle, but alive
+    t = Trainer(V, K, w, B, initial_learning_rate=1e-3)
+    t.set_dense_launches(launches)
+    t.set_corpus(tokens, offsets)
+    t.set_permutation(perm)
+    t.set_weights(planted)
+    assert t.dense_launches == 1
+    Wo = planted.copy()
+    for s in range(8):
+        t.step(s * B, B, 1e-3)
+        ref = to.train_step(Wo, to.inflate(tokens, starts, perm, s * B, B, w, V), invf, 1e-3)
+        xx, nc = t.step_stats()
+        assert np.array_equal(t.winners(B), ref["winners"]) and np.array_equal(xx, ref["xx"]), s
+        assert nc == ref["nc"], s
+    assert np.array_equal(t.get_weights().view(np.uint32), Wo.view(np.uint32))
+    known, made = t.dense_path_counts
+    assert known + made == 8 and made >= 4
+    t.set_weights(planted)
+    t.run_epoch(3, 15)
+    Wo = planted.copy()
+    to.train_steps(Wo, tokens, starts, perm, 0, B, len(starts) // B + 1, w, invf, to.epoch_eps(1e-3, 3, 15))
+    assert len(starts) % B != 0 and np.array_equal(t.get_weights().view(np.uint32), Wo.view(np.uint32))
+    assert t.giveups_recovered == 0
+    t.close()
+    other.close()
 
 
 def test_device_shuffle_is_a_cumulative_bijection(gpu):
@@ -477,16 +538,27 @@ def test_row_norms(gpu):
     t.close()
 
 
+@functools.lru_cache(maxsize=1)
+def headline_corpus():
+    """The 10,000,000-token Zipf(1.07) corpus of the headline configuration (geometric chunks, mean 25), with what
+    the checker derives from it."""
+    from flyvec_amd import synthetic
+    from oracle import train_oracle as to
+    tokens, offsets = synthetic.corpus(10_000_000, 20000)
+    return tokens, offsets, to.window_starts(offsets, 11), to.inverse_frequency(tokens, 20000)
+
+
 def test_headline_config_100_steps(gpu, oracle_lib):
-    """K = 400, V = 20000, w = 11, B = 10000, 100 steps from one seed: the stated bars
+    """K = 400, V = 20000, w = 11, B = 10000 on the 10 M-token corpus, 100 steps from one seed: the stated bars
     (winners >= 99.9 %, relative L2 <= 1e-4) and, stronger, bit equality."""
     from flyvec_amd import synthetic
     to = oracle_lib
     V, K, w, B, steps = 20000, 400, 11, 10000, 100
-    tokens, offsets = synthetic.corpus(2_000_000, V)
+    tokens, offsets, starts, invf = headline_corpus()
+    assert len(tokens) == 10_000_000 and 6_500_000 < len(starts) < 6_800_000
     W0 = synthetic.synapses(K, V, seed=5)
     t, perm = make_trainer(tokens, offsets, V, K, w, B, W0)
-    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    assert t.num_windows == len(starts)
     eps = t.epoch_eps(0, 15)
     wins = []
     for s in range(steps):
@@ -505,14 +577,30 @@ def test_headline_config_100_steps(gpu, oracle_lib):
 
 
 def test_large_config_shape(gpu, oracle_lib):
-    """K = 1000, V = 50000, w = 15, B = 50000 (W = 400 MB): two steps, bit for bit."""
-    from flyvec_amd import synthetic
+    """K = 1000, V = 50000, w = 15, B = 50000 (W = 400 MB) on the 200 M-token Zipf(1.0) corpus the configuration
+    names: the most frequent token occurs more than 2^24 times, so its 1/frequency is the saturated one of the
+    reference's fp32 counter (flyvec/src/model_arrays.cu:396-424). Two steps, bit for bit."""
+    from flyvec_amd import Trainer, synthetic
     to = oracle_lib
     V, K, w, B, steps = 50000, 1000, 15, 50000, 2
-    tokens, offsets = synthetic.corpus(400_000, V, s=1.0, mean_chunk=40)
+    tokens, offsets = synthetic.corpus(200_000_000, V, s=1.0, mean_chunk=40)
+    head = int(np.count_nonzero(tokens == 1))
+    assert head > 1 << 24, head
     W0 = synthetic.synapses(K, V, seed=5, sigma=0.02)
-    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0)
+    t = Trainer(V, K, w, B, initial_learning_rate=2e-4)
+    t.set_corpus(tokens, offsets)
+    nwin = t.num_windows
+    # a bijection of [0, nwin) that is cheap to write down at this size: i -> (a i + b) mod nwin, gcd(a, nwin) = 1
+    a = 1_000_003
+    while np.gcd(a, nwin) != 1:
+        a += 2
+    perm = (np.arange(nwin, dtype=np.uint64) * np.uint64(a) + np.uint64(12345)) % np.uint64(nwin)
+    t.set_permutation(perm)
+    t.set_weights(W0)
     starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    assert nwin == len(starts) and 0.6 * len(tokens) < nwin < 0.75 * len(tokens)
+    assert invf[1] == np.float32(1.0) / np.float32(1 << 24) and invf[1] > 1.0 / head   # saturated, not 1 / count
+    assert np.array_equal(t.inverse_frequency(), invf)
     eps = t.epoch_eps(0, 15)
     wins = []
     for s in range(steps):
@@ -702,29 +790,42 @@ def test_duplicate_pruning_with_weights_and_epoch_driver(gpu, oracle_lib):
     t.close()
 
 
-def test_dense_launch_forms_agree_over_an_epoch_of_the_headline_shape(gpu):
-    """K = 400, V = 20000, w = 11, B = 10000: 1200 steps through run_epoch as one dense launch per step and as
-    three; every block exchange, slot record and ahead-sampled minibatch of the single launch has to
-    come out right for the two matrices to be equal bit for bit."""
+def test_an_epoch_of_the_headline_configuration_in_every_launch_form(gpu, oracle_lib):
+    """K = 400, V = 20000, w = 11, B = 10000 over the whole 10 M-token corpus: one epoch through run_epoch behind a
+    device shuffle (663 full minibatches and the partial one) equals the checker's epoch over the same order bit for
+    bit, as one dense launch per step, as separate launches, and with the grouping launch of its own; every block
+    exchange, slot record and ahead-sampled minibatch of the single launch has to come out right for that."""
     from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
     V, K, w, B = 20000, 400, 11, 10000
-    tokens, offsets = synthetic.corpus(18_000_000, V)
+    tokens, offsets, starts, invf = headline_corpus()
     W0 = synthetic.synapses(K, V, seed=5)
-    got = {}
+    got, perms = {}, []
     for launches, separate in ((1, False), (2, False), (1, True)):
         t = Trainer(V, K, w, B, initial_learning_rate=2e-4)
         t.set_dense_launches(launches)
         t.set_grouping_launch(separate)      # grouped inside the sparse launch, or by a launch of its own
         t.set_corpus(tokens, offsets)
-        assert t.num_windows // B >= 1100
+        nwin = t.num_windows
+        assert nwin == len(starts) and nwin // B >= 650 and nwin % B != 0
         t.set_weights(W0)
         t.shuffle(11)
+        perms.append(t.get_permutation())
         t.run_epoch(0, 15)
         got[launches, separate] = t.get_weights()
+        assert len(t.winners(nwin % B)) == nwin % B      # the last step took the remainder only
+        if launches == 1:
+            known, made = t.dense_path_counts
+            assert known + made == nwin // B + 1 and t.giveups_recovered == 0
         t.close()
-    assert np.isfinite(got[1, False]).all() and not np.array_equal(got[1, False], W0)
-    assert np.array_equal(got[1, False], got[2, False])
-    assert np.array_equal(got[1, False], got[1, True])
+    assert np.array_equal(perms[0], perms[1]) and np.array_equal(perms[0], perms[2])
+    assert np.array_equal(np.sort(perms[0]), np.arange(nwin, dtype=np.uint64))
+    Wo = W0.copy()
+    wo = to.train_steps(Wo, tokens, starts, perms[0], 0, B, nwin // B + 1, w, invf, to.epoch_eps(2e-4, 0, 15))
+    assert len(wo) == nwin
+    assert np.isfinite(Wo).all() and not np.array_equal(Wo, W0)
+    for form, Wg in got.items():
+        assert np.array_equal(Wg, Wo), form
 
 
 @pytest.mark.parametrize("V,K,w,B,steps", [

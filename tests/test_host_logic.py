@@ -59,6 +59,12 @@ def test_byte_model_matches_the_baseline_figures():
     six = sum(per[k] for k in ("gather_winner", "group_xx", "sparse_owners", "absmax_ds", "update", "slot_update"))
     assert 369_760_000 - 200_000 <= six <= 369_760_000 + 200_000
     assert per["dense_update"] == 8 * 400 * 40000 + 8 * 10000 * 11
+    # with the single dense launch the sparse launch is held to the model's whole sparse term, 16 B w
+    assert bench.kernel_bytes(400, 40000, 11, 10000, single_dense_launch=True)["sparse_owners"] == 16 * 10000 * 11 == 1_760_000
+    # the bytes the scheme has to move: the matrix once each way
+    assert bench.step_moved_model(400, 40000, 11, 10000) == 176_000_000 + 128_000_000 + 1_760_000 == 305_760_000
+    assert bench.frac_fields("x", 8.0e12, 2.0) == {"x_frac": 0.5}
+    assert bench.frac_fields("x", 8.0e12, 0.5) == {"x_frac": None, "x_byte_model_comparison": 2.0}
 
 
 def test_bench_reads_counters_from_the_profile_summaries():

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from flyvec_amd import engine
-from flyvec_amd._lib import DeviceBuffer, FlyvecError, FV_ERR_DATA, FV_ERR_INVALID, check, load
+from flyvec_amd._lib import DeviceBuffer, FlyvecError, FV_ERR_DATA, FV_ERR_INVALID, check, device_memory, load
 
 pytestmark = pytest.mark.gpu
 
@@ -46,6 +46,24 @@ def test_two_calls_in_a_row_match_the_allocating_entry_point(gpu, oracle_lib):
         assert np.array_equal(got, oracle_lib.inverse_frequency(tokens, vocab))
     # the small vocabulary's ids were the big corpus's most frequent ones: stale counters would show
     assert static_inverse_frequency(small, 700).max() <= 1.0
+
+
+def test_the_call_leaves_the_device_memory_as_it_found_it(gpu):
+    """Free device memory, as the runtime reports it, is the same before and after the call (its buffers are the
+    caller's, allocated before the first reading; the first call on a device has already happened above or happens
+    in the warm-up here, so that the library's code object and its array are resident)."""
+    tokens = zipf_corpus(300_000, 5_000, seed=13, masked=100)
+    d_corpus, d_out = DeviceBuffer.from_numpy(tokens), DeviceBuffer(4 * 5_000)
+    try:
+        check(load().fv_inverse_frequency_static(d_corpus.ptr, len(tokens), 5_000, d_out.ptr))   # warm-up
+        before = device_memory()[0]
+        for _ in range(3):
+            check(load().fv_inverse_frequency_static(d_corpus.ptr, len(tokens), 5_000, d_out.ptr))
+            assert device_memory()[0] == before
+        assert np.array_equal(d_out.to_numpy(np.float32, (5_000,)), engine.inverse_frequency(tokens, 5_000))
+    finally:
+        d_corpus.free()
+        d_out.free()
 
 
 def test_empty_corpus_and_absent_ids(gpu):
