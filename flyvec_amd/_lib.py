@@ -90,6 +90,7 @@ SIGNATURES = {
     "fv_trainer_set_wait_limit": [_vp, _u32],
     "fv_trainer_set_grouping_launch": [_vp, _u32],
     "fv_trainer_set_slot_regions": [_vp, _u32],
+    "fv_trainer_set_light_blocks": [_vp, _u32],
     "fv_trainer_set_sentinel_list": [_vp, _u32],
     "fv_trainer_get_grouping_launch": [_vp, C.POINTER(_u32)],
     "fv_trainer_get_winners": [_vp, _vp, _u32],

@@ -790,6 +790,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.row_top2 = t->row_top2;
   sp.row_hits = t->row_hits;
   sp.top2_known = top2_known ? 1u : 0u;
+  sp.light = t->no_light_blocks ? 0u : 1u;
   sp.slot_count = t->slot_count;
   sp.pad_row = t->B;
   sp.stride = t->idx_stride;
@@ -1097,6 +1098,13 @@ extern "C" int fv_trainer_set_sentinel_list(fv_trainer *t, uint32_t entries) {
 extern "C" int fv_trainer_set_slot_regions(fv_trainer *t, uint32_t per_block) {
   FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
   t->no_block_regions = per_block == 0;
+  return FV_OK;
+}
+
+extern "C" int fv_trainer_set_light_blocks(fv_trainer *t, uint32_t on) {
+  FV_REQUIRE(t, FV_ERR_INVALID, "null trainer");
+  FV_REQUIRE(on <= 1, FV_ERR_INVALID, "on must be 0 or 1");
+  t->no_light_blocks = on == 0;
   return FV_OK;
 }
 

@@ -97,6 +97,43 @@ __device__ __forceinline__ uint32_t fv_block_exclusive_scan(uint32_t v, uint32_t
   return before + incl - v;
 }
 
+// The sum of one value per lane over the balanced binary tree on the lane number: lanes 2i and 2i + 1 first, then
+// the pairs, ... The partner's value arrives by a DPP lane pattern inside a row of 16 lanes (addition is commutative,
+// so both partners form the same bits and every lane of an aligned group holds the group's sum), the four rows' sums
+// through v_readlane. All 64 lanes must be active. This is the order of the per-neuron totals xx: a lane's value is the
+// total of one group of 64 windows, and flyvec/src/cuda_funcs.cu:722-744 leaves the order to its atomics.
+__device__ __forceinline__ float fv_wave_tree_sum(float v) {
+#define FV_TREE_STEP(CTRL) v = __fadd_rn(v, __uint_as_float(fv_dpp<CTRL>(__float_as_uint(v))));
+  FV_TREE_STEP(FV_DPP_QUAD_XOR1)  // lane ^ 1
+  FV_TREE_STEP(FV_DPP_QUAD_XOR2)  // lane ^ 2
+  FV_TREE_STEP(0x141)             // row_half_mirror: lane 7 - i of each 8, which holds the other quad's sum
+  FV_TREE_STEP(0x140)             // row_mirror: lane 15 - i, which holds the other half's sum
+#undef FV_TREE_STEP
+  const float r0 = __uint_as_float(fv_readlane(__float_as_uint(v), 0)), r1 = __uint_as_float(fv_readlane(__float_as_uint(v), 16));
+  const float r2 = __uint_as_float(fv_readlane(__float_as_uint(v), 32)), r3 = __uint_as_float(fv_readlane(__float_as_uint(v), 48));
+  return __fadd_rn(__fadd_rn(r0, r1), __fadd_rn(r2, r3));
+}
+
+// The same tree continued over the waves of a block (wave w holds the lanes 64 w .. 64 w + 63 of the tree): the wave
+// sums meet in smem (16 floats) and every thread adds them up, the waves a block does not have counting as +0
+// (no value here is -0, so that changes no bit). LDS-only barriers.
+__device__ __forceinline__ void fv_lds_barrier();
+__device__ __forceinline__ float fv_block_tree_sum(float v, float *smem /*16*/) {
+  const float ws = fv_wave_tree_sum(v);
+  const uint32_t wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+  fv_lds_barrier();  // whoever still reads smem from an earlier use has done so
+  if ((threadIdx.x & 63u) == 0) smem[wave] = ws;
+  fv_lds_barrier();
+  float t[16];
+#pragma unroll
+  for (uint32_t i = 0; i < 16; ++i) t[i] = i < n_waves ? smem[i] : 0.0f;
+#pragma unroll
+  for (uint32_t stride = 1; stride < 16; stride <<= 1)
+#pragma unroll
+    for (uint32_t i = 0; i < 16; i += 2 * stride) t[i] = __fadd_rn(t[i], t[i + stride]);
+  return t[0];
+}
+
 // Barrier for data exchanged through LDS only: waits for the wave's LDS operations, not for its
 // global loads and stores still in flight.
 __device__ __forceinline__ void fv_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
@@ -120,8 +157,14 @@ __device__ __forceinline__ uint32_t fv_block_scan_total(uint32_t v, uint32_t *sm
   return before + incl - v;
 }
 
-// SMALL: a thread's run is at most 64 windows and the minibatch has fewer than 2^16. The run is then
-// fetched in one trip to memory (16 loads of 16 bytes in flight), the two counts travel through
+// The order of the additions behind xx[h] (the reference leaves it to its atomics, flyvec/src/cuda_funcs.cu:731): the
+// minibatch's rows in groups of 64; a neuron's values of a group are added in row order onto +0; the groups' sums
+// over the balanced binary tree on the group number (fv_wave_tree_sum, fv_block_tree_sum). A thread's run is one
+// group, or a power of two of them (its own subtree, which it adds up itself), so the thread number continues the
+// tree. The CPU checker states the same order.
+//
+// SMALL: a thread's run is one group and the minibatch has fewer than 2^16 windows. The run is then
+// fetched in one trip to memory (8 loads of 16 bytes in flight), the two counts travel through
 // one block scan as the halves of a word, and the scaled activations of a thread's first matches
 // are fetched while that scan runs.
 // Winner number q (0 .. 7) of a 16-byte load of 16-bit winners.
@@ -132,20 +175,28 @@ __device__ __forceinline__ uint32_t fv_winner_of(const int4 &v, int q) {
 
 typedef short fv_short2 __attribute__((ext_vector_type(2)));
 
+// Groups of 64 windows per thread of a block of T threads that takes n windows: the smallest power of two that covers them.
+__host__ __device__ __forceinline__ uint32_t fv_group_run_groups(uint32_t n, uint32_t T) {
+  uint32_t m = 1;
+  while ((uint64_t)64 * m * T < n) m <<= 1;
+  return m;
+}
+
 template <bool SMALL>
 __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_args a) {
-  __shared__ float scbuf[FV_NB_ROUND];
   __shared__ uint32_t red[17];
+  __shared__ float tree[16];
 
   const uint32_t h = blockIdx.x;
   const uint32_t tid = threadIdx.x, T = blockDim.x;
   const uint32_t n = a.n;
   const uint16_t *__restrict__ win = a.win;
 
-  // A thread's run is a multiple of 8 windows, read as 16-byte loads of 8 winners; matches among
+  // A thread's run is m groups of 64 windows (SMALL: one), read as 16-byte loads of 8 winners; matches among
   // its first 64 windows are kept as a bit mask.
-  const uint32_t seg = ((n + T - 1) / T + 7) & ~7u;
-  const uint32_t r0 = min(tid * seg, n), r1 = min(r0 + seg, n);
+  const uint32_t m_groups = SMALL ? 1u : fv_group_run_groups(n, T);
+  const uint32_t seg = 64u * m_groups;
+  const uint32_t r0 = (uint32_t)min((uint64_t)tid * seg, (uint64_t)n), r1 = (uint32_t)min((uint64_t)r0 + seg, (uint64_t)n);
   const uint32_t n_pad = (n + 63) & ~63u;
   uint32_t lt = 0, eq = 0;
   uint64_t mask = 0;
@@ -157,18 +208,13 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
 #pragma unroll
     for (int q = 0; q < 8; ++q) wv4[q] = *(const int4 *)(win + min(r0 + 8 * q, n_pad - 8));
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      if (g * 16 < (int)seg) {  // the same answer in the whole block
-#pragma unroll
-        for (int q = 16 * g; q < 16 * g + 16; ++q) {
-          const uint32_t wv = fv_winner_of(wv4[q >> 3], q & 7);
-          const bool in = r0 + q < r1;
-          lt += in && wv < h;
-          const bool hit = in && wv == h;
-          eq += hit;
-          mask |= (uint64_t)hit << q;
-        }
-      }
+    for (int q = 0; q < 64; ++q) {
+      const uint32_t wv = fv_winner_of(wv4[q >> 3], q & 7);
+      const bool in = r0 + q < r1;
+      lt += in && wv < h;
+      const bool hit = in && wv == h;
+      eq += hit;
+      mask |= (uint64_t)hit << q;
     }
     uint64_t mm = mask;
 #pragma unroll
@@ -206,75 +252,94 @@ __global__ __launch_bounds__(FV_NB_MAX_THREADS) void fv_group_kernel(fv_group_ar
     a.group_base[h] = base;
     a.group_count[h] = c_h;
   }
-  // SMALL and the neuron's values fit scbuf: they are placed by rank here, without a trip through order[]
-  const bool staged = SMALL && c_h <= FV_NB_ROUND;
+  // the neuron's windows, ascending, into order[]; the thread's own part of xx beside it
   uint32_t *order = a.order + base;
-  {
+  float part = 0.0f;
+  if (SMALL) {
     uint32_t rank = my_off;
     uint64_t mm = mask;
-    if (SMALL) {
 #pragma unroll
-      for (int q = 0; q < PF; ++q) {
+    for (int q = 0; q < PF; ++q) {
+      if (mm) {
+        order[rank++] = r0 + (uint32_t)__ffsll((long long)mm) - 1;
+        part = __fadd_rn(part, pf[q]);
+        mm &= mm - 1;
+      }
+    }
+    // a thread with more matches than it has fetched values for: the rest, eight loads at a time
+    while (__ballot(mm != 0ull)) {
+      uint32_t r[8];
+      float v[8];
+      uint64_t m2 = mm;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        r[q] = m2 ? r0 + (uint32_t)__ffsll((long long)m2) - 1 : r0;
+        m2 &= m2 - 1;
+        v[q] = __fmul_rn(a.scale, a.sc[min(r[q], n - 1)]);
+      }
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
         if (mm) {
-          order[rank] = r0 + (uint32_t)__ffsll((long long)mm) - 1;
-          if (staged) scbuf[rank] = pf[q];
-          ++rank;
+          order[rank++] = r[q];
+          part = __fadd_rn(part, v[q]);
           mm &= mm - 1;
         }
       }
     }
-    while (mm) {
-      const uint32_t r = r0 + (uint32_t)__ffsll((long long)mm) - 1;
-      order[rank] = r;
-      if (staged) scbuf[rank] = __fmul_rn(a.scale, a.sc[r]);
-      ++rank;
-      mm &= mm - 1;
-    }
+  } else {
+    // the matches of the thread's first 64 windows are in the mask, the others are found again in the winner array
+    uint32_t rank = my_off;
+    for (uint64_t mm = mask; mm; mm &= mm - 1) order[rank++] = r0 + (uint32_t)__ffsll((long long)mm) - 1;
     for (uint32_t r = r0 + 64; r < r1; ++r)
       if ((uint32_t)win[r] == h) order[rank++] = r;
-  }
-  __syncthreads();  // the neuron's part of order[] (and of scbuf) is now readable by the whole block
-
-  // xx[h]: lane l of the first wave adds the neuron's scaled activations number l, l + 64, l + 128, ...
-  // (window order) onto 0, then the 64 partial sums are added onto 0 in lane order. For up to 64
-  // windows that is the plain sum in window order.
-  float part = 0.0f;
-  if (staged) {
-    if (tid < 64) {
-      // four values fetched together, added one after the other
-      uint32_t j = tid;
-      for (; j + 192 < c_h; j += 256) {
-        const float v0 = scbuf[j], v1 = scbuf[j + 64], v2 = scbuf[j + 128], v3 = scbuf[j + 192];
-        part = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(part, v0), v1), v2), v3);
-      }
-      for (; j < c_h; j += 64) part = __fadd_rn(part, scbuf[j]);
-    }
-  } else {
-    for (uint32_t j0 = 0; j0 < c_h; j0 += FV_NB_ROUND) {
-      const uint32_t mr = min(c_h - j0, (uint32_t)FV_NB_ROUND);
-      for (uint32_t jb = tid; jb < mr; jb += 4 * T) {  // up to 4 independent loads per thread
+    // the thread's groups one after the other; their sums meet on a stack that is the thread's subtree: a finished
+    // node of level k waits in stack[k] for its right sibling (static indices: the stack stays in registers)
+    float stack[16];  // n < 2^30 windows and 1024 threads: at most 2^14 groups per thread
+#pragma unroll
+    for (int k = 0; k < 16; ++k) stack[k] = 0.0f;
+    uint32_t j = my_off;  // next match of the thread, by rank (its own writes to order[] above)
+    const uint32_t j_end = my_off + eq;
+    for (uint32_t g = 0; g < m_groups; ++g) {
+      const uint32_t g_end = r0 + 64u * (g + 1);
+      float p_g = 0.0f;
+      while (j < j_end) {  // up to four values of the group fetched together
         uint32_t r[4];
         float v[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) r[q] = order[j0 + min(jb + q * T, mr - 1)];
+        for (int q = 0; q < 4; ++q) r[q] = order[min(j + q, j_end - 1)];
 #pragma unroll
         for (int q = 0; q < 4; ++q) v[q] = __fmul_rn(a.scale, a.sc[r[q]]);
+        uint32_t took = 0;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          if (jb + q * T < mr) scbuf[jb + q * T] = v[q];
+          if (took == (uint32_t)q && j + q < j_end && r[q] < g_end) {
+            p_g = __fadd_rn(p_g, v[q]);
+            ++took;
+          }
+        j += took;
+        if (took < 4) break;
       }
-      __syncthreads();
-      if (tid < 64)
-        for (uint32_t j = tid; j < mr; j += 64) part = __fadd_rn(part, scbuf[j]);  // FV_NB_ROUND % 64 == 0
-      __syncthreads();
-    }
-  }
-  // The partial sums in lane order, read straight from the lanes of the first wave (a partial sum
-  // without values is +0, which changes nothing: the running total starts at +0 and so is never -0).
-  if (tid < 64) {
-    float xx = 0.0f;
+      float carry = p_g;
+      bool placed = false;
+      uint32_t i = g;
 #pragma unroll
-    for (int l = 0; l < 64; ++l) xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), l)));
-    if (tid == 0) a.xx[h] = a.accumulate ? __fadd_rn(a.xx[h], xx) : xx;
+      for (int k = 0; k < 16; ++k) {
+        if (!placed) {
+          if (i & 1u) {
+            carry = __fadd_rn(stack[k], carry);
+          } else {
+            stack[k] = carry;
+            placed = true;
+          }
+        }
+        i >>= 1;
+      }
+    }
+    // m_groups = 2^k: the last group's carry ended in stack[k], the root of the thread's subtree
+#pragma unroll
+    for (int k = 0; k < 16; ++k)
+      if (m_groups == (1u << k)) part = stack[k];
   }
+  const float xx = fv_block_tree_sum(part, tree);
+  if (tid == 0) a.xx[h] = a.accumulate ? __fadd_rn(a.xx[h], xx) : xx;
 }

@@ -54,6 +54,9 @@ struct fv_sparse_args {
   const float2 *row_top2;
   uint32_t *row_hits;
   uint32_t top2_known;
+  // grouping form with a slot region per block: a neuron whose window positions are no more than the block has
+  // threads is finished by its class-0 block alone, an entry per thread (fv_sparse_light); 0 switches that off
+  uint32_t light;
 };
 
 // Counting pass of one class block over the windows whose ids are staged in LDS: ord[0 .. n_staged),
@@ -126,14 +129,91 @@ __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uin
     fv_sparse_count<NARROW, FV_SP_LOADS, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid, behind_first_loads);
 }
 
+
+// A neuron with few windows (grouping form, a slot region per block): one of its four blocks takes all four column
+// classes, one window position per thread, and the other three end at once. The counter array and a pass over
+// 5120 words to find the few counters that are not zero would be most of such a block's time; here the thread
+// whose addition finds a counter at zero owns the element, reads the final count behind a barrier and clears the
+// counter again, so nothing is scanned. The classes share the counter array and are taken one after the other.
+// Every thread asks for its element's weight and 1/f as soon as it has the column, before ownership is settled: the
+// loads of the threads that turn out not to own an element are wasted, the owners' have arrived by the time they
+// are needed (one trip less in the chain). Records go to the region of the element's class, numbered in the order
+// the owners arrive; the results do not depend on that order.
+// Called by the whole block with the neuron's window ids staged by rank in ord[0 .. c_h) (c_h * stride <= the
+// block's threads), cnt[] zero and x_h = xx[h].
+template <typename Ord>
+__device__ __forceinline__ void fv_sparse_light(const fv_sparse_args &a, uint32_t h, uint32_t blk, uint32_t c_h, float x_h,
+                                                uint32_t *cnt, const Ord *ord, uint32_t *cls_n, uint32_t *sh_hits,
+                                                float *wave_max) {
+  const uint32_t tid = threadIdx.x;
+  const uint32_t n_cols = 2 * a.V;
+  if (tid < FV_NB_CLASSES) cls_n[tid] = 0;
+  if (tid == 0) sh_hits[0] = sh_hits[1] = 0;
+  fv_lds_barrier();
+  // the thread's window position: entry tid of the neuron's c_h rows of the index matrix
+  const uint32_t j = tid / a.stride, c = tid - j * a.stride;
+  const bool inside = j < c_h;
+  const int32_t iv = a.idx[(uint64_t)ord[inside ? j : 0u] * a.stride + c];
+  const bool real = inside && (uint32_t)iv < n_cols;
+  const uint32_t col = real ? (uint32_t)iv : 0u;
+  const uint32_t p = col * a.ldk + h;
+  const float wv = a.Wt[p];
+  const float f = a.invf[col >= a.V ? col - a.V : col];
+  const float l = col >= a.V ? a.lmid : a.lbase;
+  const float2 top2 = a.top2_known ? a.row_top2[h] : make_float2(0.0f, 0.0f);
+  const uint32_t cls = col & (FV_NB_CLASSES - 1), t = col >> FV_NB_CLASS_SHIFT;
+  const uint32_t shift = 16u * (t & 1u);
+  uint32_t hits1 = 0, hits2 = 0;  // the same in all lanes of a wave
+  float ds_max = 0.0f;
+  for (uint32_t q = 0; q < FV_NB_CLASSES; ++q) {
+    const bool mine = real && cls == q;
+    bool owner = false;
+    if (mine) owner = ((atomicAdd(&cnt[t >> 1], 1u << shift) >> shift) & 0xffffu) == 0u;
+    fv_lds_barrier();  // every occurrence of the class is counted
+    uint32_t n = 0, number = 0;
+    if (owner) {
+      n = (cnt[t >> 1] >> shift) & 0xffffu;
+      number = atomicAdd(&cls_n[q], 1u);
+    }
+    fv_lds_barrier();  // the counts are read
+    if (owner) {
+      atomicAnd(&cnt[t >> 1], 0xffff0000u >> shift);  // zero again for the next class
+      fv_slot rec;
+      rec.p = p;
+      rec.n = n;
+      rec.wv = wv;
+      rec.f = f;
+      a.slots[(uint64_t)((h << FV_NB_CLASS_SHIFT) | q) * a.slot_region + number] = rec;
+      a.Wt[p] = fv_sentinel(number);
+      if (x_h != 0.0f) ds_max = fv_absmax_keep(ds_max, fv_sparse_ds(x_h, wv, f, n, l));
+    }
+    const float aw = fabsf(wv);
+    hits1 += (uint32_t)__popcll(__ballot(owner && aw == top2.x));
+    hits2 += (uint32_t)__popcll(__ballot(owner && aw == top2.y && top2.y < top2.x));
+    fv_lds_barrier();  // the class's counters are zero again
+  }
+  if ((tid & 63u) == 0 && (hits1 | hits2)) {
+    atomicAdd(&sh_hits[0], hits1);
+    atomicAdd(&sh_hits[1], hits2);
+  }
+  const float bm = fv_block_max_nonneg(ds_max, wave_max);  // behind its barriers every wave's hits are counted
+  if (tid == 0) {
+    a.bmax_sparse[blk] = bm;
+    a.row_hits[blk] = min(sh_hits[0], 3u) | (min(sh_hits[1], 3u) << 2);
+  }
+  if (tid < FV_NB_CLASSES) a.slot_count[(h << FV_NB_CLASS_SHIFT) | tid] = cls_n[tid];
+}
+
 // DELTA: the neuron's elements are counted over two lists of windows, those it won and those in
 // which it came second, into two counter arrays; a record carries both counts.
 // GROUPING: no grouping launch has run. Every class block takes its neuron's windows from the bit row
-// the winner kernel has filled (a thread's two words are 64 windows: the step has no more than
-// 64 * FV_SP_THREADS), counts the windows of lower neurons in the 16-bit winner array, stages the
-// window ids in LDS by rank, and adds the neuron's scaled activations in the grouping kernel's order;
-// the block of class 0 leaves xx[h], the neuron's count and its base for the dense launch and clears
-// the neuron's row of the other bit-row buffer.
+// the winner kernel has filled (a thread's two words are one group of 64 windows: the step has no more than
+// 64 * FV_SP_THREADS), stages the window ids in LDS by rank, and adds the neuron's scaled activations in the
+// grouping kernel's order: every thread those of its group, in row order, then the threads' sums over the balanced
+// tree on the thread number (fv_block_tree_sum). The block of class 0 leaves xx[h], the neuron's count and its base
+// for the dense launch and clears the neuron's row of the other bit-row buffer. The blocks of this form go to the
+// device's eight XCDs in turn, so the class a block takes rotates with the neuron: every XCD gets its share of each
+// class (the class-0 blocks are the ones that finish a neuron with few windows alone, fv_sparse_light).
 // IDS16: the window ids staged in LDS are 16 bits wide (a batch below 65535 windows, so that the id of the padding
 // row behind the index matrix fits too): the smaller array lets one more block share a compute unit.
 // NW (GROUPING): 64-bit words of the neuron's bit row per thread; a step has up to 64 * NW * FV_SP_THREADS windows.
@@ -154,25 +234,28 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   typedef typename std::conditional<IDS16, uint16_t, uint32_t>::type ord_t;
   __shared__ ord_t ord[FV_SP_STAGE];
   __shared__ uint32_t sh_pos;
-  __shared__ float sh_xx;
   __shared__ uint32_t sh_hits[2];
-  __shared__ float sc64[GROUPING ? 64 : 1];  // activations of a neuron with up to 64 windows, by rank
   __shared__ float wave_max[16];
   __shared__ uint32_t red[17];
   constexpr uint32_t T = FV_SP_THREADS;
   const uint32_t h = blockIdx.x >> FV_NB_CLASS_SHIFT;
-  const uint32_t q = blockIdx.x & (FV_NB_CLASSES - 1);
+  const uint32_t q = GROUPING ? ((blockIdx.x & (FV_NB_CLASSES - 1)) + (blockIdx.x >> (FV_NB_CLASS_SHIFT + 1))) & (FV_NB_CLASSES - 1)
+                              : blockIdx.x & (FV_NB_CLASSES - 1);
+  const uint32_t blk = (h << FV_NB_CLASS_SHIFT) | q;  // the block's number in the arrays the other launches read
   const uint32_t tid = threadIdx.x;
   __shared__ uint32_t red2[GROUPING ? 17 : 1];
   uint32_t c_h, base, my_off = 0, r0 = 0;
-  bool sc_complete = true;  // every thread's matches have their activations in pf[]
   uint64_t mask[NW];
 #pragma unroll
   for (int i = 0; i < NW; ++i) mask[i] = 0;
   uint32_t eq = 0;  // the thread's matches
-  constexpr int PF = 4;
-  float pf[PF];
+  // scaled activations a thread fetches before it knows how many it needs: four, or sixteen in a wave with a
+  // thread that has more than four matches (a neuron that won a tenth of the minibatch has seven per thread)
+  constexpr int PF = 4, PF_BIG = 16;
+  float pf[PF_BIG];
+  float x_h = 0.0f;
   if (GROUPING) {
+    static_assert(NW == 1, "a thread's words are one group of 64 windows of the order of the totals xx");
     const uint32_t n = a.n;
     // thread t takes windows 64 NW t .. 64 NW (t + 1) - 1: 2 NW words of the neuron's row
     r0 = 64 * NW * tid;
@@ -192,44 +275,55 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
         if (word < a.won_words) *(uint2 *)(a.won_clear + (uint64_t)h * a.won_words + word) = make_uint2(0u, 0u);
       }
     }
-    // the scaled activations of a thread's first matches travel while the scan runs
+    // the scaled activations of a thread's matches travel while the scan runs
     {
-      uint64_t left[NW];
+      const bool wave_big = __ballot(eq > (uint32_t)PF) != 0ull;
+      uint64_t left = mask[0];
 #pragma unroll
-      for (int i = 0; i < NW; ++i) left[i] = mask[i];
+      for (int e = 0; e < PF_BIG; ++e) pf[e] = 0.0f;
+      // the lowest bit left (none left: the thread's first window, whose value is not used)
+#define FV_SP_FETCH(e)                                                                    \
+  {                                                                                       \
+    const uint32_t r = left ? r0 + (uint32_t)__ffsll((long long)left) - 1 : r0;           \
+    left &= left - 1;                                                                     \
+    pf[e] = a.sc[min(r, n - 1)];                                                          \
+  }
+      if (wave_big) {
 #pragma unroll
-      for (int e = 0; e < PF; ++e) {
-        // the first word with a bit left, its lowest bit taken (no word left: the thread's first window)
-        uint32_t r = r0;
-        bool taken = false;
+        for (int e = 0; e < PF_BIG; ++e) FV_SP_FETCH(e)
+      } else {
 #pragma unroll
-        for (int i = 0; i < NW; ++i) {
-          const bool here = !taken && left[i] != 0;
-          if (here) r = r0 + 64 * i + (uint32_t)__ffsll((long long)left[i]) - 1;
-          left[i] = here ? left[i] & (left[i] - 1) : left[i];
-          taken = taken || here;
-        }
-        pf[e] = a.sc[min(r, n - 1)];
+        for (int e = 0; e < PF; ++e) FV_SP_FETCH(e)
       }
+#undef FV_SP_FETCH
     }
-    // one block scan gives the ranks and the neuron's count, and tells whether any thread has more matches
-    // than it has fetched activations for
-    const bool wave_more = __ballot(eq > (uint32_t)PF) != 0ull;
+    // one block scan gives the ranks and the neuron's count
     const uint32_t incl = fv_wave_inclusive_scan_u32(eq);
-    if ((tid & 63u) == 63u) red[tid >> 6] = incl, red[8 + (tid >> 6)] = wave_more;
+    if ((tid & 63u) == 63u) red[tid >> 6] = incl;
     fv_lds_barrier();
     uint32_t before = 0, total = 0;
-    bool more = false;
 #pragma unroll
     for (uint32_t i = 0; i < T / 64; ++i) {
       const uint32_t t = red[i];
       before += i < (tid >> 6) ? t : 0u;
       total += t;
-      more = more || red[8 + i] != 0;
     }
     c_h = total;
     my_off = before + incl - eq;
-    sc_complete = !more;
+    // xx[h]: the thread's group first, in row order onto +0 (what was fetched, then, for a thread with more matches
+    // than that, the rest one by one), then the tree over the threads
+    {
+      float part = 0.0f;
+#pragma unroll
+      for (int e = 0; e < PF_BIG; ++e)
+        if ((uint32_t)e < eq) part = __fadd_rn(part, pf[e]);
+      if (eq > (uint32_t)PF_BIG) {
+        uint64_t left = mask[0];
+        for (int e = 0; e < PF_BIG; ++e) left &= left - 1;
+        for (; left; left &= left - 1) part = __fadd_rn(part, a.sc[r0 + (uint32_t)__ffsll((long long)left) - 1]);
+      }
+      x_h = fv_block_tree_sum(part, wave_max);
+    }
     base = 0;
     if (c_h != 0 && a.slot_region == 0) {
       // The number of windows won by lower neurons is the neuron's place in a class's slot region where the
@@ -265,7 +359,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     if (q == 0 && tid == 0) {
       a.group_base_out[h] = base;  // used where it was counted
       a.group_count_out[h] = c_h;
-      if (c_h == 0) a.xx_out[h] = 0.0f;
+      a.xx_out[h] = x_h;  // (+0 for a neuron without a window)
     }
   } else {
     c_h = a.group_count[h];
@@ -273,11 +367,34 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   const uint32_t c2_h = DELTA ? a.group_count2[h] : 0u;
   if (c_h == 0 && c2_h == 0) {
     if (tid == 0) {
-      a.bmax_sparse[blockIdx.x] = 0.0f;
-      a.slot_count[blockIdx.x] = 0;
-      a.row_hits[blockIdx.x] = 0;
+      a.bmax_sparse[blk] = 0.0f;
+      a.slot_count[blk] = 0;
+      a.row_hits[blk] = 0;
     }
     return;
+  }
+  if (GROUPING) {
+    // a neuron with no more window positions than the block has threads: all of it in the class-0 block
+    const uint32_t class_cols0 = (2 * a.V + FV_NB_CLASSES - 1) >> FV_NB_CLASS_SHIFT;
+    const bool light = a.light && a.slot_region != 0 && c_h * a.stride <= T &&
+                       class_cols0 <= 2u * CW;  // (the same answer in the neuron's four blocks)
+    if (light) {
+      if (q != 0) {
+        if (tid == 0) {
+          a.bmax_sparse[blk] = 0.0f;  // the neuron's records are counted by its class-0 block
+          a.row_hits[blk] = 0;
+        }
+        return;
+      }
+      {
+        uint32_t at = my_off;  // the window ids by rank
+#pragma unroll
+        for (int i = 0; i < NW; ++i)
+          for (uint64_t mm = mask[i]; mm; mm &= mm - 1) ord[at++] = (ord_t)(r0 + 64 * i + (uint32_t)__ffsll((long long)mm) - 1);
+      }
+      fv_sparse_light<ord_t>(a, h, blk, c_h, x_h, cnt, ord, red2, sh_hits, wave_max);
+      return;
+    }
   }
   // counts of the block's elements that hold the row's largest / second largest weight (every path to the
   // elements passes a barrier)
@@ -288,14 +405,14 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   if (c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
   if (!GROUPING) base = a.group_base[h];
   const uint32_t base2 = DELTA ? a.group_base2[h] : 0u;
-  float x_h = GROUPING ? 0.0f : a.xx[h];
+  if (!GROUPING) x_h = a.xx[h];
   float ds_max = 0.0f;
   const uint32_t *order = (GROUPING ? a.order_out : a.order) + base;  // GROUPING: also written here, through order_out
   const uint32_t n_cols = 2 * a.V;
   const uint32_t m_ent = max(c_h, c2_h) * a.w;
   // the block's records: no more than (c_h + c2_h) * w of them, behind those of the lower neurons
   const bool regions = GROUPING && a.slot_region != 0;
-  const uint64_t slot_first = regions ? (uint64_t)blockIdx.x * a.slot_region
+  const uint64_t slot_first = regions ? (uint64_t)blk * a.slot_region
                                       : (uint64_t)q * a.slot_stride + (uint64_t)(base + base2) * a.w;
   fv_slot *slots = a.slots + slot_first;
 
@@ -305,12 +422,6 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     if (DELTA)
       for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt2)[i] = make_uint4(0, 0, 0, 0);
   }
-  // xx[h] is added up in the grouping kernel's order: lane l of the first wave adds the values number
-  // l, l + 64, ... onto 0, then the partial sums are added onto 0 in lane order (those of the lanes
-  // from c_h on are +0 and change nothing). A neuron with up to 64 windows, each thread holding the
-  // activations of all its matches, does that behind the counting pass, where the value is first
-  // needed and the loads have long returned.
-  bool xx_pending = GROUPING && staged_once && sc_complete && c_h <= 64;
   // GROUPING: the window ids of ranks [j0, j0 + FV_SP_STAGE) into LDS, every thread those of its own matches (its
   // ranks start at my_off; a neuron with more windows than LDS stages is staged part by part, each time
   // from the bit row's words in registers)
@@ -325,56 +436,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   };
   if (GROUPING) {
     if (staged_once) stage_ids(0);
-    if (!xx_pending) {
-      // A neuron with many windows: the activations are fetched by rank into the counter array
-      // (cleared behind the block scan, and again by the first wave once it has added them).
-      static_assert(FV_SP_STAGE <= CW && FV_SP_STAGE % 64 == 0 && FV_SP_STAGE <= 8 * T,
-                    "a stage of activations fits the counters and one trip to memory");
-      float *scbuf = (float *)cnt;
-      float part = 0.0f;
-      for (uint32_t j0 = 0; j0 < c_h; j0 += FV_SP_STAGE) {
-        const uint32_t mr = min(c_h - j0, (uint32_t)FV_SP_STAGE);
-        if (!staged_once) stage_ids(j0);  // (the barrier that ends a part stands in front of this)
-        fv_lds_barrier();                 // the ids are in LDS
-        // eight loads in flight per thread: the ids first, all of them
-        uint32_t id8[8];
-        float v8[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) id8[u] = (uint32_t)ord[min(tid + u * T, mr - 1)];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v8[u] = a.sc[id8[u]];
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-          if (tid + u * T < mr) scbuf[tid + u * T] = v8[u];
-        fv_lds_barrier();
-        if (tid < 64) {
-          uint32_t j = tid;
-          for (; j + 192 < mr; j += 256) {  // four values fetched together, added one after the other
-            const float v0 = scbuf[j], v1 = scbuf[j + 64], v2 = scbuf[j + 128], v3 = scbuf[j + 192];
-            part = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(part, v0), v1), v2), v3);
-          }
-          for (; j < mr; j += 64) part = __fadd_rn(part, scbuf[j]);
-        }
-        if (j0 + FV_SP_STAGE < c_h) fv_lds_barrier();  // before the next stage overwrites this one
-      }
-      if (tid < 64) {
-        float xx = 0.0f;
-        if (c_h >= 64) {
-#pragma unroll
-          for (int l = 0; l < 64; ++l) xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), l)));
-        } else {
-          for (uint32_t l = 0; l < c_h; ++l)
-            xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), (int)l)));
-        }
-        if (tid == 0) {
-          sh_xx = xx;
-          if (q == 0) a.xx_out[h] = xx;
-        }
-        const uint32_t used = (min(c_h, (uint32_t)FV_SP_STAGE) + 3) / 4;
-        for (uint32_t i = tid; i < used; i += 64) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
-      }
-    }
-    // the counting pass starts behind a barrier; sh_xx is read behind that pass
+    // the counting pass starts behind a barrier
   } else {
     if (staged_once)
       for (uint32_t i = tid; i < c_h; i += T) ord[i] = (ord_t)order[i];
@@ -388,18 +450,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   const uint32_t class_cols = (n_cols + FV_NB_CLASSES - 1) >> FV_NB_CLASS_SHIFT;  // columns of a class
   uint32_t emitted = 0;
 
-  // The activations a thread fetched at the start go to LDS by rank as soon as they can be had without a wait
-  // of their own, behind the issue of the counting pass's first loads: held any longer they would sit in
-  // registers through the whole pass. (xx_pending implies a neuron with windows, so the pass has a first load.)
-  bool pf_staged = false;
-  auto stage_activations = [&]() {
-    if (GROUPING && xx_pending && !pf_staged) {
-#pragma unroll
-      for (int e = 0; e < PF; ++e)
-        if ((uint32_t)e < eq) sc64[my_off + e] = pf[e];  // a thread's matches have consecutive ranks
-      pf_staged = true;
-    }
-  };
+  auto nothing = []() {};
 
   for (uint32_t lo = 0; lo < class_cols; lo += span) {
     for (int l = 0; l < (DELTA ? 2 : 1); ++l) {
@@ -418,11 +469,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
           fv_lds_barrier();
         }
         if (narrow)
-          fv_sparse_count_any<true, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid,
-                                           stage_activations);
+          fv_sparse_count_any<true, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid, nothing);
         else
-          fv_sparse_count_any<false, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid,
-                                            stage_activations);
+          fv_sparse_count_any<false, ord_t>(counters, ord, n_staged, a.pad_row, a.idx, a.stride, q, lo, span, tid, nothing);
       }
     }
     // Every non-zero counter is one distinct element. Their positions are collected in LDS, up to
@@ -432,19 +481,6 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     do {
       if (tid == 0) sh_pos = 0;
       fv_lds_barrier();
-      if (GROUPING && xx_pending) {
-        if (tid < 64) {
-          const float part = tid < c_h ? __fadd_rn(0.0f, sc64[tid]) : 0.0f;
-          float xx = 0.0f;
-          for (uint32_t l = 0; l < c_h; ++l)
-            xx = __fadd_rn(xx, __uint_as_float(fv_readlane(__float_as_uint(part), (int)l)));
-          if (tid == 0) {
-            sh_xx = xx;
-            if (q == 0) a.xx_out[h] = xx;
-          }
-        }
-        xx_pending = false;
-      }
       {
         // bit 8 * i + u of `mine`: counter u of the thread's i-th group of four words is non-zero
         constexpr int n_groups = (CW / 4 + T - 1) / T;
@@ -494,7 +530,6 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       }
       fv_lds_barrier();
       found = sh_pos;
-      if (GROUPING) x_h = sh_xx;
       const uint32_t take = min(found, (uint32_t)FV_SP_LIST_CAP);
       // one element per thread (four in flight): save its weight and its count in a slot record,
       // plant the sentinel, take |ds| (the dense term plus count additions of 1/f; a row with
@@ -562,9 +597,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   }
   const float bm = fv_block_max_nonneg(ds_max, wave_max);  // behind its barriers every wave's hits are counted
   if (tid == 0) {
-    a.bmax_sparse[blockIdx.x] = bm;
-    a.slot_count[blockIdx.x] = emitted;
-    a.row_hits[blockIdx.x] = min(sh_hits[0], 3u) | (min(sh_hits[1], 3u) << 2);
+    a.bmax_sparse[blk] = bm;
+    a.slot_count[blk] = emitted;
+    a.row_hits[blk] = min(sh_hits[0], 3u) | (min(sh_hits[1], 3u) << 2);
   }
 }
 

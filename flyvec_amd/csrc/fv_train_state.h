@@ -81,6 +81,7 @@ struct fv_trainer {
   fv_slot *slots_blocks;
   uint32_t slot_region;
   bool no_block_regions;  // fv_trainer_set_slot_regions(0): the class regions are used all the same
+  bool no_light_blocks;   // fv_trainer_set_light_blocks(0): a neuron with few windows keeps its four class blocks
   uint32_t *slot_count;  // K * FV_NB_CLASSES
   float *xx;        // ldk
   float *bmax;      // max|ds| of each block of the absmax launch, then of each block of the sparse launch

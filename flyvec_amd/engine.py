@@ -192,6 +192,12 @@ class Trainer:
         Same results either way."""
         check(self.lib.fv_trainer_set_slot_regions(self.handle, 1 if per_block else 0))
 
+    def set_light_blocks(self, on):
+        """True (the default): a neuron with few windows is finished by one block of the sparse-element launch
+        that groups for itself, an entry per thread; False: by its four class blocks like the others.
+        Same results either way."""
+        check(self.lib.fv_trainer_set_light_blocks(self.handle, 1 if on else 0))
+
     def set_sentinel_list(self, entries):
         """Test hook: the single dense launch's LDS list of sparse elements counts as full after `entries`
         (0: its real size); the elements beyond are finished where they are met.  Same results."""

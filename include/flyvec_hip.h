@@ -237,6 +237,12 @@ int fv_trainer_get_grouping_launch(fv_trainer *t, uint32_t *out_separate); /* th
  * blocks share one region per class, each behind the records of the neurons before it, as the other launch
  * forms do. Results are bit-identical either way. No counterpart in the reference. */
 int fv_trainer_set_slot_regions(fv_trainer *t, uint32_t per_block);
+/* In that launch form (blocks with regions of their own) a neuron that won so few windows that a block has a thread
+ * for each of their positions (21 windows of 11 at 256 threads) is finished by one of its four blocks alone, an
+ * entry per thread, and the other three end at once: most neurons of a Zipf minibatch are such. on = 1, the
+ * default; 0 keeps the four class blocks for every neuron. Results are bit-identical either way. No counterpart
+ * in the reference. */
+int fv_trainer_set_light_blocks(fv_trainer *t, uint32_t on);
 /* Test hook. A block of the single dense launch notes the sparse elements it meets (their sentinels) in an LDS
  * list and finishes them when its dense elements are done; an element that finds the list full is finished on
  * the spot. entries > 0 makes the list count as full after that many (no more than it holds: 2048, or 8192 in

@@ -30,11 +30,13 @@
  * Order-dependent fp32 sums (the reference uses atomics whose order is not
  * defined) are given a fixed order here.  The sparse term of ds: increasing
  * window order, then increasing position inside the window.  The per-neuron
- * totals xx: see fvo_xx_sums (64 interleaved partial sums in window order,
- * then the partials in index order; for a neuron with at most 64 windows that
- * is the plain sum in window order).  fvo_xx_sums is pinned by a numpy
- * restatement of that order and by its agreement with plain window order (to
- * rounding) in tests/test_oracle_train.py.
+ * totals xx: see fvo_xx_sums (the minibatch's rows in groups of 64: a
+ * neuron's values of a group are added in row order, the groups' sums over the
+ * balanced binary tree on the group number).  fvo_xx_sums is pinned by a numpy
+ * restatement of that order (halving an array of group sums), by the cases in
+ * which it is the plain sum in row order (one group; two groups; one value per
+ * group and a power-of-two alignment) and by its agreement with plain row
+ * order to rounding, in tests/test_oracle_train.py.
  *
  * Parity unpinned against the reference BINARY in one rounding: the update
  * W += (eps / max|ds|) * ds is written as a multiply and then an add in
@@ -238,32 +240,49 @@ float fvo_epoch_eps(float lr0, uint64_t epoch, uint64_t n_epochs) {
 
 /*
  * xx[h] = sum of sc[r] over the windows r won by h (flyvec/src/cuda_funcs.cu:722-744, fp32 atomics
- * there).  order_kind 0: the j-th window of neuron h, counted in increasing window order, is added
- * onto partial sum j mod 64 (each starting at 0); the partials that received a value are then
- * added onto 0 in index order.  order_kind 1: every window added onto xx[h] in increasing window
- * order.  The two agree for neurons with at most 64 windows.
+ * there: the reference's order of additions is not defined).  order_kind 0, the step's order: the rows
+ * of the minibatch are taken in groups of 64 consecutive rows; P_g is the sum, onto 0 and in row order,
+ * of sc[r] over the rows of group g that h won (0 if none); xx[h] is the sum of P_0, P_1, ... over the
+ * balanced binary tree on the group number: node(0, g) = P_g, node(k, i) = node(k-1, 2i) + node(k-1, 2i+1),
+ * groups past the last one counting as 0 (a sum onto +0 is never -0, so adding such a 0 changes no bit and
+ * the result does not depend on how far the tree is padded).  order_kind 1: every window added onto xx[h]
+ * in increasing row order.
  */
-#define FVO_XX_LANES 64
+#define FVO_XX_GROUP 64
+#define FVO_XX_LEVELS 64
 void fvo_xx_sums(const int32_t *win, const float *sc, uint64_t n, int K, int order_kind, float *xx) {
   for (int h = 0; h < K; ++h) xx[h] = 0.0f;
   if (order_kind == 1) {
     for (uint64_t r = 0; r < n; ++r) xx[win[r]] = xx[win[r]] + sc[r];
     return;
   }
-  float *part = (float *)calloc((size_t)K * FVO_XX_LANES, sizeof(float));
-  uint64_t *cnt = (uint64_t *)calloc((size_t)K, sizeof(uint64_t));
-  for (uint64_t r = 0; r < n; ++r) {
-    const int h = win[r];
-    float *p = part + (size_t)h * FVO_XX_LANES + (cnt[h] % FVO_XX_LANES);
-    *p = *p + sc[r];
-    cnt[h]++;
+  /* the tree is evaluated as the groups arrive: stack[h][k] holds a finished node of level k that waits for
+   * its right sibling; a neuron's stack after G groups holds the nodes the set bits of G name */
+  float *stack = (float *)calloc((size_t)K * FVO_XX_LEVELS, sizeof(float));
+  float *part = (float *)calloc((size_t)K, sizeof(float));
+  const uint64_t G = (n + FVO_XX_GROUP - 1) / FVO_XX_GROUP;
+  for (uint64_t g = 0; g < G; ++g) {
+    const uint64_t r1 = (g + 1) * FVO_XX_GROUP < n ? (g + 1) * FVO_XX_GROUP : n;
+    for (int h = 0; h < K; ++h) part[h] = 0.0f;
+    for (uint64_t r = g * FVO_XX_GROUP; r < r1; ++r) part[win[r]] = part[win[r]] + sc[r];
+    for (int h = 0; h < K; ++h) {
+      float carry = part[h];
+      int level = 0;
+      for (uint64_t i = g; i & 1; i >>= 1, ++level) carry = stack[(size_t)h * FVO_XX_LEVELS + level] + carry;
+      stack[(size_t)h * FVO_XX_LEVELS + level] = carry;
+    }
   }
   for (int h = 0; h < K; ++h) {
-    const uint64_t used = cnt[h] < FVO_XX_LANES ? cnt[h] : FVO_XX_LANES;
-    for (uint64_t l = 0; l < used; ++l) xx[h] = xx[h] + part[(size_t)h * FVO_XX_LANES + l];
+    /* the groups from G on are 0: what is left on the stack is added from the lowest level up, each node
+     * as the left operand of the partial node to its right */
+    float acc = 0.0f;
+    int level = 0;
+    for (uint64_t i = G; i; i >>= 1, ++level)
+      if (i & 1) acc = stack[(size_t)h * FVO_XX_LEVELS + level] + acc;
+    xx[h] = acc;
   }
+  free(stack);
   free(part);
-  free(cnt);
 }
 
 /*

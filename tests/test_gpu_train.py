@@ -1004,6 +1004,48 @@ def test_minibatches_beyond_16384_windows(gpu, oracle_lib, K, w, V, B):
         assert np.array_equal(Wg.view(np.uint32), Wo.view(np.uint32)), f"W, launches {launches}"
 
 
+@pytest.mark.parametrize("launches", [1, 2, 3])
+@pytest.mark.parametrize("V,K,w,B", [(20000, 400, 11, 3000), (700, 130, 9, 2500), (300, 500, 64, 600), (900, 40, 1, 900),
+                                     (60, 300, 15, 200), (5000, 7, 5, 4000), (3000, 2048, 3, 1000)])
+def test_neurons_with_few_windows_are_finished_by_one_block(gpu, oracle_lib, V, K, w, B, launches):
+    """The sparse-element launch that groups for itself gives a neuron with no more window positions than a block
+    has threads to one block, an entry per thread, for all four column classes (the other three blocks end at
+    once). With that form and without it, against the checker step by step: many neurons (most are such), few
+    (every neuron heavy), w = 64 (four windows fill a block) and w = 1, repeated tokens inside a window, ties."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    tokens, offsets = small_corpus(max(40000, 12 * B), V, seed=V % 7, mean_chunk=max(25, w + 8))
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    perm = np.random.default_rng(V).permutation(len(starts)).astype(np.uint64)
+    W0 = synthetic.synapses(K, V, seed=3, sigma=0.02)
+    if K == 300:
+        W0 = np.round(W0 * 100) / np.float32(100)            # a coarse grid: ties among the activations
+    steps = min(4, len(starts) // B)
+    assert steps >= 2
+    Wo, ref = W0.copy(), []
+    for s in range(steps):
+        ref.append(to.train_step(Wo, to.inflate(tokens, starts, perm, s * B, B, w, V), invf, 1e-3))
+    counts = np.bincount(ref[0]["winners"], minlength=K)
+    stride = (w + 3) & ~3
+    few = np.count_nonzero((counts > 0) & (counts * stride <= 256))
+    assert few > 0 or K <= 7, "no neuron of this case takes the form under test"
+    for light in (True, False):
+        t = Trainer(V, K, w, B, initial_learning_rate=1e-3)
+        t.set_dense_launches(launches)
+        t.set_light_blocks(light)
+        t.set_corpus(tokens, offsets)
+        t.set_permutation(perm)
+        t.set_weights(W0)
+        assert t.grouping_launch is False
+        for s in range(steps):
+            t.step(s * B, B, 1e-3)
+            assert np.array_equal(t.winners(B), ref[s]["winners"]), (light, s)
+            xx, nc = t.step_stats()
+            assert np.array_equal(xx, ref[s]["xx"]) and nc == ref[s]["nc"], (light, s)
+        assert np.array_equal(t.get_weights().view(np.uint32), Wo.view(np.uint32)), light
+        t.close()
+
+
 @pytest.mark.parametrize("launches,entries", [(1, 1), (1, 37), (3, 1), (3, 300)])
 def test_sparse_elements_beyond_the_sentinel_list_are_finished_where_they_are_met(gpu, oracle_lib, launches, entries):
     """The single dense launch with a sentinel list that counts as full after a few entries: nearly every sparse

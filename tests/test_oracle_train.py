@@ -334,19 +334,29 @@ def test_multi_step_driver_matches_single_steps():
 # ---- order of the per-neuron totals ---------------------------------------------------------------
 
 def xx_numpy(winners, sc, K):
-    """The step's order, restated: value j of a neuron (window order) joins partial j mod 64; the
-    partials in use are then added in index order. np.cumsum in float32 adds strictly left to right."""
+    """The step's order, restated: the rows in groups of 64; a neuron's values of a group are added in row order
+    (np.cumsum in float32 adds strictly left to right), and the array of group sums, padded with zeros to a power
+    of two, is halved by adding neighbours until one value is left."""
+    n = len(winners)
+    G = max(1, -(-n // 64))
+    size = 1
+    while size < G:
+        size *= 2
     out = np.zeros(K, dtype=f32)
     for h in range(K):
-        v = sc[winners == h]
-        if len(v) == 0:
-            continue
-        parts = [np.cumsum(v[l::64], dtype=f32)[-1] for l in range(min(64, len(v)))]
-        out[h] = np.cumsum(np.array(parts, dtype=f32), dtype=f32)[-1]
+        P = np.zeros(size, dtype=f32)
+        for g in range(G):
+            rows = slice(64 * g, min(64 * g + 64, n))
+            v = sc[rows][winners[rows] == h]
+            if len(v):
+                P[g] = np.cumsum(v, dtype=f32)[-1]
+        while len(P) > 1:
+            P = (P[0::2] + P[1::2]).astype(f32)
+        out[h] = P[0]
     return out
 
 
-@pytest.mark.parametrize("n,K", [(1, 3), (50, 4), (64, 1), (65, 1), (129, 2), (5000, 7), (40000, 3)])
+@pytest.mark.parametrize("n,K", [(1, 3), (50, 4), (64, 1), (65, 1), (129, 2), (5000, 7), (10000, 400), (40000, 3), (65537, 2)])
 def test_xx_order_against_numpy(n, K):
     rng = np.random.default_rng(n + K)
     winners = rng.integers(0, K, size=n).astype(np.int32)
@@ -358,13 +368,38 @@ def test_xx_order_against_numpy(n, K):
     assert np.array_equal(to.xx_sums(winners, sc, K, 1), seq)
 
 
-def test_xx_order_is_window_order_up_to_64_windows_and_close_beyond():
+def test_xx_order_is_row_order_where_the_tree_is_a_chain_and_close_elsewhere():
     rng = np.random.default_rng(5)
-    K = 40
-    winners = np.repeat(np.arange(K), 64).astype(np.int32)      # exactly 64 windows each
-    rng.shuffle(winners)
+    # one group: the plain sum in row order
+    winners = rng.integers(0, 5, size=64).astype(np.int32)
+    sc = rng.standard_normal(64).astype(f32)
+    assert np.array_equal(to.xx_sums(winners, sc, 5, 0), to.xx_sums(winners, sc, 5, 1))
+    # two groups, and a neuron that wins the whole first group and one window of the second: P_0 + P_1 is the sum
+    # in row order
+    winners = np.ones(128, dtype=np.int32)
+    winners[:64] = 0
+    winners[64 + 5] = 0
+    sc = rng.standard_normal(128).astype(f32)
+    assert to.xx_sums(winners, sc, 2, 0)[0] == to.xx_sums(winners, sc, 2, 1)[0]
+    # one value per group in groups 0, 1, 2, 4: ((a + b) + (c + 0)) + ((d + 0) + 0) = ((a + b) + c) + d
+    winners = np.ones(5 * 64, dtype=np.int32)
+    winners[[3, 64 + 9, 128 + 63, 256]] = 0
     sc = rng.standard_normal(len(winners)).astype(f32)
-    assert np.array_equal(to.xx_sums(winners, sc, K, 0), to.xx_sums(winners, sc, K, 1))
+    a, b, c, d = sc[[3, 64 + 9, 128 + 63, 256]]
+    want = f32(f32(f32(a + b) + c) + d)
+    assert to.xx_sums(winners, sc, 2, 0)[0] == want == to.xx_sums(winners, sc, 2, 1)[0]
+    # one value per group in groups 1, 2, 3: (0 + a) + (b + c), which is not the sum in row order
+    winners = np.ones(4 * 64, dtype=np.int32)
+    winners[[64, 128, 192]] = 0
+    sc = np.array([0.1] * 256, dtype=f32)
+    sc[[64, 128, 192]] = [f32(1.0), f32(2.0 ** -24), f32(2.0 ** -24)]
+    assert to.xx_sums(winners, sc, 2, 0)[0] == f32(f32(1.0) + f32(2.0 ** -23))       # b + c first: it survives
+    assert to.xx_sums(winners, sc, 2, 1)[0] == f32(1.0)                               # one by one both are lost
+    # a sum that starts at +0 is never -0, whatever it adds
+    winners = np.zeros(70, dtype=np.int32)
+    sc = np.full(70, -0.0, dtype=f32)
+    assert not np.signbit(to.xx_sums(winners, sc, 1, 0)[0])
+    # many windows: the two orders differ, by rounding only
     winners = rng.integers(0, 3, size=30000).astype(np.int32)
     sc = np.abs(rng.standard_normal(30000)).astype(f32)
     a, b = to.xx_sums(winners, sc, 3, 0), to.xx_sums(winners, sc, 3, 1)
@@ -374,7 +409,7 @@ def test_xx_order_is_window_order_up_to_64_windows_and_close_beyond():
     assert np.all(np.abs(b - exact) <= 2e-5 * exact)
 
 
-def test_step_uses_the_interleaved_order():
+def test_step_uses_the_grouped_order():
     rng = np.random.default_rng(8)
     K, V, w, n = 3, 30, 5, 2000
     W = rng.standard_normal((K, 2 * V)).astype(f32)
