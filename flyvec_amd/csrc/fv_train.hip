@@ -303,6 +303,22 @@ static void fv_choose_onepass(fv_trainer *t, uint64_t cu) {
   if (need <= FV_ONEPASS_MAX_UNROLL) {
     unroll = need <= 8 ? 8 : 16;
     const size_t smem = fv_onepass_smem(t);
+    {
+      // its sentinel lists take more LDS than a launch may have without asking
+      bool set = true;
+#define FV_SET(KERNEL)                                                                                              \
+  set = set && hipFuncSetAttribute((const void *)KERNEL, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess;
+#define FV_SET_PHASES(U, DELTA) \
+  FV_SET((fv_dense_onepass_kernel<U, DELTA, 0>)) FV_SET((fv_dense_onepass_kernel<U, DELTA, 1>)) FV_SET((fv_dense_onepass_kernel<U, DELTA, 2>))
+      if (unroll == 8) { FV_SET_PHASES(8, false) FV_SET_PHASES(8, true) } else { FV_SET_PHASES(16, false) FV_SET_PHASES(16, true) }
+#undef FV_SET_PHASES
+#undef FV_SET
+      if (!set) {
+        (void)hipGetLastError();
+        unroll = 0;
+      }
+    }
+    if (unroll)
     if (!(unroll == 8 ? fv_onepass_fits<8>(smem) : fv_onepass_fits<16>(smem))) unroll = 0;
   }
   if (!unroll && !t->stream_ok) return;
@@ -838,7 +854,8 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.slots = anti ? t->slots2 : slot_region ? t->slots_blocks : t->slots;
   d.slot_region = slot_region;
   {
-    const uint32_t holds = t->onepass_stream ? FV_STREAM_HIT_CAP : FV_ONEPASS_HIT_CAP;
+    // (the register form keeps a list per wave, the streaming form one per block)
+    const uint32_t holds = t->onepass_stream ? FV_STREAM_HIT_CAP : FV_ONEPASS_WAVE_HITS;
     d.hit_cap = t->hit_cap_limit && t->hit_cap_limit < holds ? t->hit_cap_limit : holds;
   }
   d.slot_count = t->slot_count;

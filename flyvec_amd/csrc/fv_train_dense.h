@@ -329,10 +329,12 @@ __global__ __launch_bounds__(TB) void fv_update_kernel(fv_dense_args a) {
 // give up as well, sets the status word and leaves its part of W as it is.
 //
 // The sparse elements are finished here as well, by the block that owns them: a thread that meets a
-// sentinel leaves it alone and notes (sentinel, element) in an LDS list; when the block has updated its
-// dense elements the list is dealt over its threads, each of which finds the record through the
-// sentinel's number, forms ds and writes the element. No other block ever reads or writes that element
-// in this launch.
+// sentinel leaves it alone and notes (sentinel, element) in its wave's LDS list; when the wave has updated its
+// dense elements it deals its list over its lanes, each of which finds the record through the sentinel's
+// number, forms ds and writes the element. No other block ever reads or writes that element in this launch.
+// (A list per wave, not per block: the wave asks for its records as soon as its own last store is issued,
+// without a barrier, so the records travel while the stores drain -- a wave's loads and stores share one
+// counter, and a load asked for behind the block's barrier would begin its trip only when the drain is over.)
 #ifndef FV_ONEPASS_THREADS
 #define FV_ONEPASS_THREADS 1024
 #endif
@@ -345,7 +347,9 @@ __global__ __launch_bounds__(TB) void fv_update_kernel(fv_dense_args a) {
 #endif
 #define FV_ONEPASS_SPIN_LIMIT (1u << 14)  // rounds of a few microseconds each: tens of milliseconds
 #define FV_ONEPASS_ABANDONED 0xffffffffu  // in place of a block's maximum (no maximum is a NaN): it gave up
-#define FV_ONEPASS_HIT_CAP 2048           // sentinels a block notes in LDS; one beyond that is finished on the spot
+#define FV_ONEPASS_HIT_CAP 4096           // sentinels a block notes in LDS, a list of its own for every wave; one
+                                          // that finds its wave's list full is finished by its thread, from memory
+#define FV_ONEPASS_WAVE_HITS (FV_ONEPASS_HIT_CAP / (FV_ONEPASS_THREADS / 64))
 
 // The same on two LDS words per neuron, from many threads at once: the value that loses at the first
 // word -- the newcomer, or the value it displaced -- goes on to the second; every value but the
@@ -382,6 +386,58 @@ __device__ __forceinline__ void fv_finish_sparse_element(const fv_dense_args &a,
   }
   ((float *)a.Wt4)[p] = out;
   fv_top2_insert_lds(sp1, sp2, h, fv_abs_or_zero(out));
+}
+
+// The sentinels of a list, dealt over `width` threads (this one is number `me` of them), four records in flight per
+// thread: a wave that has met a row of a frequent token holds a few hundred of them, and one after the other each
+// would be a trip to memory of its own.
+template <bool DELTA>
+__device__ __forceinline__ void fv_finish_sparse_elements(const fv_dense_args &a, const uint2 *list, uint32_t n, uint32_t me,
+                                                          uint32_t width, float s, bool ok, const float *xs, uint32_t *sp1,
+                                                          uint32_t *sp2) {
+  for (uint32_t i0 = me; i0 < n; i0 += 4 * width) {
+    uint2 hit[4];
+    fv_slot sl[4];
+    uint32_t n2[4];
+    bool mine[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      hit[u] = list[min(i0 + u * width, n - 1)];
+      const uint32_t number = (hit[u].x & FV_SENTINEL_MAX) - 1u;
+      mine[u] = i0 + u * width < n && number < a.n_slots;  // a NaN of another origin stays what it is
+      const uint32_t p = hit[u].y, col = p / a.ldk, h = p - col * a.ldk;
+      const uint64_t at = a.slot_region
+                              ? (uint64_t)((h << FV_NB_CLASS_SHIFT) | (col & (FV_NB_CLASSES - 1))) * a.slot_region + number
+                              : number;
+      sl[u] = a.slots[mine[u] ? at : 0];
+      n2[u] = DELTA ? a.slot_n2[mine[u] ? at : 0] : 0u;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t p = hit[u].y;
+      if (!mine[u] || sl[u].p != p) continue;
+      const uint32_t h = p % a.ldk;
+      const float x = xs[h];
+      float out = sl[u].wv;
+      if (ok && x != 0.0f) {
+        const float l = p >= a.V * a.ldk ? a.lmid : a.lbase;
+        const float ds = DELTA ? fv_sparse_ds2(x, sl[u].wv, sl[u].f, sl[u].n, a.delta, n2[u], l)
+                               : fv_sparse_ds(x, sl[u].wv, sl[u].f, sl[u].n, l);
+        const float d = __fmul_rn(s, ds);
+        if (fabsf(d) > a.update_cut) out = __fadd_rn(sl[u].wv, d);
+      }
+      ((float *)a.Wt4)[p] = out;
+      fv_top2_insert_lds(sp1, sp2, h, fv_abs_or_zero(out));
+    }
+  }
+}
+
+// s_setprio takes its level as an immediate.
+__device__ __forceinline__ void fv_set_wave_priority(uint32_t level) {
+  if (level == 0) __builtin_amdgcn_s_setprio(0);
+  else if (level == 1) __builtin_amdgcn_s_setprio(1);
+  else if (level == 2) __builtin_amdgcn_s_setprio(2);
+  else __builtin_amdgcn_s_setprio(3);
 }
 
 // The next minibatch's column indices, by all waves but the first (which polls in the exchange): the
@@ -552,7 +608,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   constexpr uint32_t T = FV_ONEPASS_THREADS;
   constexpr int DEPTH = FV_ONEPASS_DEPTH < U ? FV_ONEPASS_DEPTH : U;
   // xx (ldk floats); the two largest finished sparse elements of every neuron (2 x ldk words); the
-  // sentinels met (FV_ONEPASS_HIT_CAP pairs); the threads' two largest weights (4 x active pairs)
+  // sentinels met (FV_ONEPASS_WAVE_HITS pairs per wave); the threads' two largest weights (4 x active pairs)
   extern __shared__ float4 dyn4[];
   float *xs = (float *)dyn4;
   uint32_t *sp1 = (uint32_t *)(xs + a.ldk);
@@ -562,7 +618,9 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   __shared__ uint32_t red3[T / 64][3];
   __shared__ float smem16[16];
   __shared__ float sh_s;
-  __shared__ uint32_t sh_ok, sh_hits;
+  __shared__ uint32_t sh_ok, sh_hits[T / 64];
+  uint2 *wave_list = hit_list + (threadIdx.x >> 6) * FV_ONEPASS_WAVE_HITS;
+  uint32_t *wave_hits = &sh_hits[threadIdx.x >> 6];
   const uint32_t tid = threadIdx.x;
   const bool active = tid < a.active;
   const uint32_t q = tid % a.ldk4, r = tid / a.ldk4;
@@ -619,7 +677,7 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
     }
     if (h < a.K) fv_row_candidate(xh[j], rm[j], hit4[j], smx[j], S, E, F);
   }
-  if (tid == 0) sh_hits = 0;
+  if (tid < T / 64) sh_hits[tid] = 0;
   {
     const uint32_t ws = fv_wave_max_u32(S), we = fv_wave_max_u32(E), wf = fv_wave_max_u32(F);
     if ((tid & 63) == 0) {
@@ -699,15 +757,19 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   if (v.member == v.member) {                                                                  \
     if (changed) e[lane4] = v.member;                                                          \
   } else {                                                                                     \
-    const uint32_t k = atomicAdd(&sh_hits, 1u);                                                \
+    const uint32_t k = atomicAdd(wave_hits, 1u);                                               \
     if (k < a.hit_cap)                                                                         \
-      hit_list[k] = make_uint2(__float_as_uint(v.member), 4u * p4 + lane4);                    \
+      wave_list[k] = make_uint2(__float_as_uint(v.member), 4u * p4 + lane4);                   \
     else                                                                                       \
       beyond_list |= 1ull << (4 * u + lane4);                                                  \
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const uint32_t row = row0 + u * row_step;
+    // The four waves that share a SIMD take turns at going first. Left to the age of the waves, the youngest ones
+    // of every block are served last throughout and end their stream 3 to 4 us behind the median wave, and the
+    // block ends with them.
+    fv_set_wave_priority(((tid >> 8) + (uint32_t)u) & 3u);
     if (active && row < a.n_rows) {
       const uint32_t p4 = row * a.ldk4 + q;
       float4 v = w[u];
@@ -734,6 +796,12 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
     if (samples0) a.idx_ahead[e0] = c0 < a.w ? fv_column_index(tok0, c0, a.w, a.V) : -1;
     fv_sample_ahead(a, false, e0, er0, start0, ahead_entries, TS);  // the entries beyond the first, if any
   }
+  // the sentinels the wave has met, dealt over its lanes (the list and its count are the wave's own: no barrier)
+  __builtin_amdgcn_s_setprio(0);
+  {
+    const uint32_t n_hits = min(*wave_hits, a.hit_cap);
+    fv_finish_sparse_elements<DELTA>(a, wave_list, n_hits, tid & 63u, 64u, s, ok, xs, sp1, sp2);
+  }
   while (beyond_list) {
     const uint32_t b = (uint32_t)__ffsll((long long)beyond_list) - 1u;
     beyond_list &= beyond_list - 1;
@@ -743,13 +811,6 @@ __global__ __launch_bounds__(FV_ONEPASS_THREADS) void fv_dense_onepass_kernel(fv
   if (active) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) pairs[(e * rows_per_round + r) * a.ldk4 + q] = make_float2(t1[e], t2[e]);
-  }
-  __syncthreads();
-  // the sentinels the block has met, dealt over its threads
-  const uint32_t n_hits = min(sh_hits, a.hit_cap);
-  for (uint32_t i = tid; i < n_hits; i += T) {
-    const uint2 hit = hit_list[i];
-    fv_finish_sparse_element<DELTA>(a, hit.x, hit.y, s, ok, xs, sp1, sp2);
   }
   __syncthreads();
   // the block's share of every row's two largest weights: its threads' pairs and the finished sparse elements

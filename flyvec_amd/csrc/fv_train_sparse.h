@@ -60,14 +60,15 @@ struct fv_sparse_args {
 };
 
 // Counting pass of one class block over the windows whose ids are staged in LDS: ord[0 .. n_staged),
-// followed up to the next multiple of FV_SP_WPS * LOADS by the id of the padding row behind the
-// index matrix (all -1). A row of idx is `stride` entries, a multiple of 4, those past w holding -1;
-// four consecutive lanes read the sixteen positions of a chunk of one window 16 bytes each, so a
-// wave's load covers sixteen windows. A lane issues LOADS loads back to back with no branch between
-// them (the compiler waits for every load in flight at a branch target), then counts. With the
-// class in the top bits and the column of the class below, one subtraction and one comparison tell
-// whether an entry is this block's: of class q, inside [lo, lo + span), not masked, not padding.
-#define FV_SP_WPS (FV_SP_THREADS / 4)  // windows the block takes per step
+// followed up to the next multiple of the windows a batch of loads takes by the id of the padding row behind the
+// index matrix (all -1). A row of idx is `stride` entries, a multiple of 4, those past w holding -1; a lane
+// reads four positions of one window, 16 bytes, and a window takes as many neighbouring lanes as its row has
+// such pieces, up to four (fv_sparse_lanes: three for the eleven positions of the reference's window, so that a
+// block's load covers 85 windows, not 64; a longer row is read in chunks of sixteen positions). A lane issues
+// LOADS loads back to back with no branch between them (the compiler waits for every load in flight at a
+// branch target), then counts. With the class in the top bits and the column of the class below, one
+// subtraction and one comparison tell whether an entry is this block's: of class q, inside [lo, lo + span),
+// not masked, not padding.
 #define FV_SLOT_REGIONS_MAX_BYTES (1ull << 30)  // most memory spent on slot regions per block
 template <bool NARROW>
 __device__ __forceinline__ void fv_sparse_count_entry(uint32_t *cnt, int32_t iv, uint32_t drop, uint32_t origin,
@@ -81,24 +82,38 @@ __device__ __forceinline__ void fv_sparse_count_entry(uint32_t *cnt, int32_t iv,
   }
 }
 
+// Lanes that share a window in the counting pass, and the windows a block of FV_SP_THREADS then takes per load.
+__host__ __device__ __forceinline__ uint32_t fv_sparse_lanes(uint32_t stride) { return stride >= 16 ? 4u : stride >> 2; }
+__host__ __device__ __forceinline__ uint32_t fv_sparse_wps(uint32_t stride) { return FV_SP_THREADS / fv_sparse_lanes(stride); }
+// Window ids staged in LDS at a time: whole batches of FV_SP_LOADS loads, so that the padding stays inside ord[].
+__host__ __device__ __forceinline__ uint32_t fv_sparse_stage_cap(uint32_t stride) {
+  const uint32_t per = fv_sparse_wps(stride) * FV_SP_LOADS;
+  return FV_SP_STAGE / per * per;
+}
+
 // behind_first_loads() runs once, between the issue of the first loads and the counting of what they bring: the
 // place for work on values whose own loads were issued earlier and so have returned by then.
 template <bool NARROW, int LOADS, typename Ord, typename Hook>
 __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const Ord *ord, uint32_t n_staged,
                                                 const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
                                                 uint32_t lo, uint32_t span, uint32_t tid, Hook &behind_first_loads) {
-  const uint32_t c4 = 4u * (tid & 3u), slot = tid >> 2;
-  const uint32_t steps = (n_staged + FV_SP_WPS - 1) / FV_SP_WPS;
+  const uint32_t lanes = fv_sparse_lanes(stride), wps = FV_SP_THREADS / lanes;
+  // tid / lanes without a division: exact for tid < 2^16 / lanes
+  const uint32_t slot_of = (tid * ((65536u + lanes - 1) / lanes)) >> 16;
+  const bool alive = slot_of < wps;  // (255 of 256 threads with three lanes per window)
+  const uint32_t slot = alive ? slot_of : 0u;
+  const uint32_t c4 = 4u * (tid - slot_of * lanes);
+  const uint32_t steps = (n_staged + wps - 1) / wps;
   const uint32_t origin = (q << (32 - FV_NB_CLASS_SHIFT)) | lo;
   for (uint32_t c0 = 0; c0 < stride; c0 += FV_SP_CHUNK) {
-    const bool live = c0 + c4 < stride;  // a row shorter than the chunk: the lanes past its end read its start again
+    const bool live = alive && c0 + c4 < stride;  // a row shorter than the chunk: the lanes past its end read its start again
     const uint32_t cc = live ? c0 + c4 : 0u;
     const uint32_t drop = live ? 0u : 0xffffffffu;
     for (uint32_t s0 = 0; s0 < steps; s0 += LOADS) {
       int4 iv[LOADS];
 #pragma unroll
       for (int b = 0; b < LOADS; ++b)
-        iv[b] = *(const int4 *)(idx + (uint64_t)ord[(s0 + b) * FV_SP_WPS + slot] * stride + cc);
+        iv[b] = *(const int4 *)(idx + (uint64_t)ord[(s0 + b) * wps + slot] * stride + cc);
       if (c0 == 0 && s0 == 0) behind_first_loads();
 #pragma unroll
       for (int b = 0; b < LOADS; ++b) {
@@ -111,24 +126,25 @@ __device__ __forceinline__ void fv_sparse_count(uint32_t *cnt, const Ord *ord, u
   }
 }
 
-// The same with the number of loads in flight fitted to the number of windows; pads ord[].
+// The same with the number of loads in flight fitted to the number of windows; pads ord[] (n_staged is at most
+// fv_sparse_stage_cap).
 template <bool NARROW, typename Ord, typename Hook>
 __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uint32_t n_staged, uint32_t pad_row,
                                                     const int32_t *__restrict__ idx, uint32_t stride, uint32_t q,
                                                     uint32_t lo, uint32_t span, uint32_t tid, Hook &behind_first_loads) {
-  static_assert(FV_SP_STAGE % (FV_SP_WPS * FV_SP_LOADS) == 0 && FV_SP_LOADS % 4 == 0, "padding of ord[] stays inside it");
-  const uint32_t per = FV_SP_WPS * (n_staged <= FV_SP_WPS ? 1 : n_staged <= FV_SP_WPS * 4 ? 4 : FV_SP_LOADS);
+  static_assert(FV_SP_LOADS % 4 == 0 && FV_SP_STAGE >= FV_SP_THREADS * FV_SP_LOADS, "padding of ord[] stays inside it");
+  const uint32_t wps = fv_sparse_wps(stride);
+  const uint32_t per = wps * (n_staged <= wps ? 1 : n_staged <= wps * 4 ? 4 : FV_SP_LOADS);
   const uint32_t padded = (n_staged + per - 1) / per * per;
   for (uint32_t i = n_staged + tid; i < padded; i += FV_SP_THREADS) ord[i] = (Ord)pad_row;
   fv_lds_barrier();
-  if (per == FV_SP_WPS)
+  if (per == wps)
     fv_sparse_count<NARROW, 1, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid, behind_first_loads);
-  else if (per == FV_SP_WPS * 4)
+  else if (per == wps * 4)
     fv_sparse_count<NARROW, 4, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid, behind_first_loads);
   else
     fv_sparse_count<NARROW, FV_SP_LOADS, Ord>(cnt, ord, n_staged, idx, stride, q, lo, span, tid, behind_first_loads);
 }
-
 
 // A neuron with few windows (grouping form, a slot region per block): one of its four blocks takes all four column
 // classes, one window position per thread, and the other three end at once. The counter array and a pass over
@@ -257,6 +273,8 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   if (GROUPING) {
     static_assert(NW == 1, "a thread's words are one group of 64 windows of the order of the totals xx");
     const uint32_t n = a.n;
+    // (the counters are cleared while the bit row travels)
+    for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
     // thread t takes windows 64 NW t .. 64 NW (t + 1) - 1: 2 NW words of the neuron's row
     r0 = 64 * NW * tid;
 #pragma unroll
@@ -278,6 +296,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     // the scaled activations of a thread's matches travel while the scan runs
     {
       const bool wave_big = __ballot(eq > (uint32_t)PF) != 0ull;
+      // such a wave belongs to one of the few blocks the launch waits for: it goes first from here on wherever
+      // it shares a SIMD with the waves of other blocks
+      if (wave_big) __builtin_amdgcn_s_setprio(3);
       uint64_t left = mask[0];
 #pragma unroll
       for (int e = 0; e < PF_BIG; ++e) pf[e] = 0.0f;
@@ -310,6 +331,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     }
     c_h = total;
     my_off = before + incl - eq;
+    // The launch lasts as long as its few heaviest blocks: their waves go first wherever they share a
+    // SIMD with the waves of light blocks.
+    if (c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
     // xx[h]: the thread's group first, in row order onto +0 (what was fetched, then, for a thread with more matches
     // than that, the rest one by one), then the tree over the threads
     {
@@ -317,10 +341,24 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
 #pragma unroll
       for (int e = 0; e < PF_BIG; ++e)
         if ((uint32_t)e < eq) part = __fadd_rn(part, pf[e]);
-      if (eq > (uint32_t)PF_BIG) {
-        uint64_t left = mask[0];
+      if (__ballot(eq > (uint32_t)PF_BIG)) {  // (a neuron that won more than a quarter of some group of 64 windows)
+        uint64_t left = eq > (uint32_t)PF_BIG ? mask[0] : 0ull;
         for (int e = 0; e < PF_BIG; ++e) left &= left - 1;
-        for (; left; left &= left - 1) part = __fadd_rn(part, a.sc[r0 + (uint32_t)__ffsll((long long)left) - 1]);
+        while (__ballot(left != 0ull)) {  // eight loads in flight, then their additions in row order
+          float v[8];
+          uint64_t l2 = left;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const uint32_t r = l2 ? r0 + (uint32_t)__ffsll((long long)l2) - 1 : r0;
+            l2 &= l2 - 1;
+            v[e] = a.sc[min(r, n - 1)];
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            if (left) part = __fadd_rn(part, v[e]);
+            left &= left - 1;
+          }
+        }
       }
       x_h = fv_block_tree_sum(part, wave_max);
     }
@@ -355,7 +393,6 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       }
       base = fv_block_sum_u32((uint32_t)(-((int)below.x + (int)below.y)), red2);
     }
-    for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
     if (q == 0 && tid == 0) {
       a.group_base_out[h] = base;  // used where it was counted
       a.group_count_out[h] = c_h;
@@ -400,9 +437,8 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   // elements passes a barrier)
   if (tid == 0) sh_hits[0] = sh_hits[1] = 0;
   uint32_t hits1 = 0, hits2 = 0;  // the same in all lanes of a wave
-  // The launch lasts as long as its few heaviest blocks: their waves go first wherever they share a
-  // SIMD with the waves of light blocks.
-  if (c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
+  // (GROUPING: done as soon as the count was known) the waves of the few heaviest blocks go first
+  if (!GROUPING && c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
   if (!GROUPING) base = a.group_base[h];
   const uint32_t base2 = DELTA ? a.group_base2[h] : 0u;
   if (!GROUPING) x_h = a.xx[h];
@@ -416,7 +452,8 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
                                       : (uint64_t)q * a.slot_stride + (uint64_t)(base + base2) * a.w;
   fv_slot *slots = a.slots + slot_first;
 
-  const bool staged_once = !DELTA && c_h <= FV_SP_STAGE;  // the usual case: the neuron's window ids are staged here
+  const uint32_t stage_cap = fv_sparse_stage_cap(a.stride);  // window ids staged in LDS at a time
+  const bool staged_once = !DELTA && c_h <= stage_cap;  // the usual case: the neuron's window ids are staged here
   if (!GROUPING) {
     for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
     if (DELTA)
@@ -427,12 +464,24 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   // from the bit row's words in registers)
   auto stage_ids = [&](uint32_t j0) {
     uint32_t at = my_off - j0;  // wraps below 0 for the ranks in front of the part
+    // the two halves of a word one after the other, four matches between two branches, as many rounds as the
+    // wave's busiest thread needs (a taken branch costs a lone wave as much as four or five instructions)
 #pragma unroll
-    for (int i = 0; i < NW; ++i)
-      for (uint64_t mm = mask[i]; mm; mm &= mm - 1) {
-        if (at < (uint32_t)FV_SP_STAGE) ord[at] = (ord_t)(r0 + 64 * i + (uint32_t)__ffsll((long long)mm) - 1);
-        ++at;
+    for (int half = 0; half < 2 * NW; ++half) {
+      uint32_t mm = (uint32_t)(mask[half >> 1] >> (32 * (half & 1)));
+      const uint32_t first = r0 + 32u * half;
+      const uint32_t rounds = (fv_wave_max_u32((uint32_t)__popc(mm)) + 3u) >> 2;
+      for (uint32_t it = 0; it < rounds; ++it) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (mm) {
+            if (at < stage_cap) ord[at] = (ord_t)(first + (uint32_t)__ffs((int)mm) - 1u);
+            ++at;
+            mm &= mm - 1;
+          }
+        }
       }
+    }
   };
   if (GROUPING) {
     if (staged_once) stage_ids(0);
@@ -457,8 +506,8 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       const uint32_t *ids = l == 0 ? order : a.order2 + base2;
       const uint32_t n_ids = l == 0 ? c_h : c2_h;
       uint32_t *counters = l == 0 ? cnt : cnt2;
-      for (uint32_t j0 = 0; j0 < n_ids; j0 += FV_SP_STAGE) {
-        const uint32_t n_staged = min(n_ids - j0, (uint32_t)FV_SP_STAGE);
+      for (uint32_t j0 = 0; j0 < n_ids; j0 += stage_cap) {
+        const uint32_t n_staged = min(n_ids - j0, stage_cap);
         if (!staged_once) {
           fv_lds_barrier();  // the previous part has been counted
           if (GROUPING) {
