@@ -281,6 +281,34 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, which="step", dense_launche
     return out
 
 
+def bench_delta_step(steps, warmup, plain_ms_per_step, c=TRAIN, delta=0.4):
+    """The same step with the anti-Hebbian term of the reference switched on (delta != 0 at
+    flyvec/src/cuda_funcs.cu:870-935: the neuron that came second in a window is pushed away from it), which the
+    reference's driver leaves at 0: the second neuron's window lists are grouped and summed beside the winner's."""
+    from flyvec_amd import Trainer, synthetic
+    tokens, offsets = synthetic.corpus(c["n_tokens"], c["V"], s=c["zipf_s"], mean_chunk=c["mean_chunk"])
+    t = Trainer(c["V"], c["K"], c["w"], c["B"], initial_learning_rate=c["lr0"], prec=c["prec"])
+    t.set_corpus(tokens, offsets)
+    t.set_permutation(np.random.default_rng(6).permutation(t.num_windows).astype(np.uint64))
+    t.set_weights(synthetic.synapses(c["K"], c["V"], seed=5))
+    eps = t.epoch_eps(0, c["n_epochs"])
+    for s in range(warmup):
+        t.step(s * c["B"], c["B"], eps, delta=delta)
+    t.sync()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        t.step((warmup + s) * c["B"], c["B"], eps, delta=delta)
+    t.sync()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    kern_ms = {k: v for k, v in t.time_kernels(reps=20).items() if v > 1e-3}  # empty launches take 0.2 us
+    t.close()
+    return {"delta": delta, "value": c["B"] / (ms * 1e-3), "unit": "windows/s", "steps": steps, "warmup": warmup,
+            "ms_per_step": ms, "us_over_the_step_without_the_term": (ms - plain_ms_per_step) * 1e3,
+            "kernel_ms": kern_ms,
+            "note": "same corpus, order, matrix and batch as the headline step; wall clock over the timed steps, device "
+                    "idle before and after; kernel_ms from replays of the last step's launches between HIP events"}
+
+
 def bench_epoch(c=EPOCH):
     """One full epoch as flyvec_train runs it (flyvec/train_flyvec.py:253-263): reshuffle, every
     minibatch of the corpus, then one checkpoint written as .npy; set-up is timed beside it."""
@@ -512,6 +540,7 @@ def main():
         line["hash"], line["hash_host"] = bench_hash(reps=10, cpu_seconds=min(args.cpu_seconds, 5.0),
                                                      host=not args.no_hash_host)
     if args.workload == "all":
+        line["delta_step"] = bench_delta_step(args.steps, args.warmup, tr["ms_per_step"])
         if not args.no_large:
             steps, warmup = min(args.steps, 30), min(args.warmup, 5)
             lt = bench_train(steps, warmup, 0.0, LARGE, "large", args.dense_launches, args.separate_grouping)

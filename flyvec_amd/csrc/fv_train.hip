@@ -632,6 +632,12 @@ static void fv_trainer_free_delta(fv_trainer *t) {
   (void)hipFree(t->group_count2);
   (void)hipFree(t->slots2);
   (void)hipFree(t->slot_n2);
+  (void)hipFree(t->won2[0]);
+  (void)hipFree(t->slots2_blocks);
+  (void)hipFree(t->slot_n2_blocks);
+  t->won2[0] = t->won2[1] = nullptr;
+  t->slots2_blocks = nullptr;
+  t->slot_n2_blocks = nullptr;
   t->win2 = nullptr;
   t->win2_16 = nullptr;
   t->sc2 = nullptr;
@@ -651,6 +657,19 @@ static int fv_trainer_alloc_delta(fv_trainer *t) {
   FV_HIP(hipMalloc((void **)&t->group_base2, (size_t)t->K * sizeof(uint32_t)));
   FV_HIP(hipMalloc((void **)&t->group_count2, (size_t)t->K * sizeof(uint32_t)));
   FV_HIP(hipMalloc((void **)&t->slots2, 2 * FV_NB_CLASSES * bw * sizeof(fv_slot)));
+  // The form that groups inside the sparse launch: bit rows for the second neurons, and a slot region per block. A
+  // block writes at most one record per column of its class; the regions are that long only where a class has no
+  // more columns than the minibatch has window positions (fv_trainer_alloc), else this form is not taken.
+  const uint64_t class_cols = (t->N + FV_NB_CLASSES - 1) / FV_NB_CLASSES;
+  if (t->won[0] && t->slot_region && t->slot_region == class_cols) {
+    const size_t row_words = (size_t)t->K * t->won_words;
+    const size_t records = (size_t)t->slot_region * t->K * FV_NB_CLASSES;
+    FV_HIP(hipMalloc((void **)&t->won2[0], 2 * row_words * sizeof(uint32_t)));
+    t->won2[1] = t->won2[0] + row_words;
+    FV_HIP(hipMemsetAsync(t->won2[0], 0, 2 * row_words * sizeof(uint32_t), t->stream));
+    FV_HIP(hipMalloc((void **)&t->slots2_blocks, records * sizeof(fv_slot)));
+    FV_HIP(hipMalloc((void **)&t->slot_n2_blocks, records * sizeof(uint32_t)));
+  }
   FV_HIP(hipMalloc((void **)&t->slot_n2, 2 * FV_NB_CLASSES * bw * sizeof(uint32_t)));
   return FV_OK;
 }
@@ -712,8 +731,9 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   // on the last step's pair, cleared here first unless it repeats the launch before it.
   // (beyond 64 windows per thread of a class block only with a slot region per block: without one every block
   // would count the lower neurons' windows in the whole winner array)
-  const bool grouping_in_sparse = which == 0x3f ? !anti && fv_groups_in_sparse(t) : t->last_grouped_in_sparse;
-  if (which == 0x3f) t->last_grouped_in_sparse = grouping_in_sparse;
+  const bool can_group = fv_groups_in_sparse(t) && (!anti || (t->slot_n2_blocks && !t->no_block_regions));
+  const bool grouping_in_sparse = which == 0x3f ? can_group : (anti ? t->last_delta_grouped : t->last_grouped_in_sparse);
+  if (which == 0x3f) (anti ? t->last_delta_grouped : t->last_grouped_in_sparse) = grouping_in_sparse;
   // the blocks of a sparse launch that groups for itself write their records to regions of their own, where
   // the trainer has them, and a sentinel names a record inside its block's region
   const uint32_t slot_region = grouping_in_sparse && !t->no_block_regions ? t->slot_region : 0u;
@@ -721,14 +741,19 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   const bool onepass = t->onepass && n_slots + 1 < FV_SENTINEL_MAX;
   const bool alone = fv_trainers_alive.load() == 1;
   g.won = nullptr;
+  g.won2 = nullptr;
   g.won_words = t->won_words;
   if (grouping_in_sparse) {
     if (which == 0x3f) {
       t->won_parity ^= 1u;
+      if (anti) t->won2_parity ^= 1u;
     } else if ((which & 1u) && !repeated) {
       FV_HIP(hipMemsetAsync(t->won[t->won_parity], 0, (size_t)t->K * t->won_words * sizeof(uint32_t), t->stream));
+      if (anti)
+        FV_HIP(hipMemsetAsync(t->won2[t->won2_parity], 0, (size_t)t->K * t->won_words * sizeof(uint32_t), t->stream));
     }
     g.won = t->won[t->won_parity];
+    if (anti) g.won2 = t->won2[t->won2_parity];
   }
   // a whole step whose windows the previous one has sampled ahead takes that buffer
   g.sampled = 0;
@@ -790,13 +815,13 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.group_count = t->group_count;
   sp.idx = t->idx;
   sp.Wt = t->Wt;
-  sp.slots = anti ? t->slots2 : slot_region ? t->slots_blocks : t->slots;
+  sp.slots = anti ? (slot_region ? t->slots2_blocks : t->slots2) : slot_region ? t->slots_blocks : t->slots;
   sp.slot_region = slot_region;
   sp.slot_stride = (uint64_t)t->B * t->w * (anti ? 2 : 1);
   sp.order2 = t->order2;
   sp.group_base2 = t->group_base2;
   sp.group_count2 = t->group_count2;
-  sp.slot_n2 = t->slot_n2;
+  sp.slot_n2 = anti && slot_region ? t->slot_n2_blocks : t->slot_n2;
   sp.delta = delta;
   sp.lmid = t->cfg.lmid;
   sp.lbase = t->cfg.lbase;
@@ -817,6 +842,11 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.win = t->win16;
   sp.won_words = t->won_words;
   sp.won_clear = t->won[t->won_parity ^ 1u];
+  sp.won2 = anti && grouping_in_sparse ? t->won2[t->won2_parity] : nullptr;
+  sp.won2_clear = anti && grouping_in_sparse ? t->won2[t->won2_parity ^ 1u] : nullptr;
+  sp.sc2 = t->sc2;
+  sp.group_base2_out = t->group_base2;
+  sp.group_count2_out = t->group_count2;
   sp.sc = t->sc;
   sp.n = n;
   sp.order_out = t->order;
@@ -831,7 +861,9 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
     const auto passes = [&](uint32_t words) { return (class_cols + 2 * words - 1) / (2 * words); };
     const bool wide = passes(FV_NB_CNT_WORDS_WIDE) < passes(FV_NB_CNT_WORDS);
 #define FV_LAUNCH_SPARSE(CW, GROUPING_KERNEL)                                                       \
-  if (anti)                                                                                         \
+  if (anti && grouping_in_sparse)                                                                   \
+    hipLaunchKernelGGL((fv_sparse_grouping_delta_kernel<CW>), sp_grid, sp_block, 0, t->stream, sp); \
+  else if (anti)                                                                                    \
     hipLaunchKernelGGL((fv_sparse_kernel<true, CW>), sp_grid, sp_block, 0, t->stream, sp);          \
   else if (grouping_in_sparse)                                                                      \
     hipLaunchKernelGGL(GROUPING_KERNEL, sp_grid, sp_block, 0, t->stream, sp);                       \
@@ -851,7 +883,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.Wt4 = (float4 *)t->Wt;
   d.xx = t->xx;
   d.invf = t->invf;
-  d.slots = anti ? t->slots2 : slot_region ? t->slots_blocks : t->slots;
+  d.slots = anti ? (slot_region ? t->slots2_blocks : t->slots2) : slot_region ? t->slots_blocks : t->slots;
   d.slot_region = slot_region;
   {
     // (the register form keeps a list per wave, the streaming form one per block)
@@ -861,7 +893,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   d.slot_count = t->slot_count;
   d.group_base = t->group_base;
   d.group_base2 = t->group_base2;
-  d.slot_n2 = t->slot_n2;
+  d.slot_n2 = anti && slot_region ? t->slot_n2_blocks : t->slot_n2;
   d.delta = delta;
   d.w = t->w;
   d.arrive = nullptr;

@@ -14,6 +14,7 @@ struct fv_gather_args {
   int32_t *win;
   uint16_t *win16;  // the same winners as 16-bit values, for the grouping kernel
   uint32_t *won;        // not null: bit r of row hstar is set (atomic OR; the rows are zero before)
+  uint32_t *won2;       // not null (anti-Hebbian form): the same for the window's second neuron
   uint32_t won_words;
   float *sc;
   // anti-Hebbian form only: the second neuron of every window and its scaled activation
@@ -200,6 +201,7 @@ __device__ __forceinline__ void fv_gather_one_window(const fv_gather_args &a, ui
       a.win2[r] = (int32_t)second;
       a.win2_16[r] = (uint16_t)second;
       a.sc2[r] = s2;
+      if (a.won2 && second < a.K) atomicOr(&a.won2[(uint64_t)second * a.won_words + (r >> 5)], 1u << (r & 31u));
     }
   }
 }

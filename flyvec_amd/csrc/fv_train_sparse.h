@@ -42,6 +42,12 @@ struct fv_sparse_args {
   const uint16_t *win;        // 16-bit winners; behind the last one, up to a multiple of 64 entries, 0x7fff
   uint32_t won_words;
   uint32_t *won_clear;  // the other buffer: the class-0 block of neuron h clears row h
+  // anti-Hebbian form that groups for itself: the same pair of bit rows for the second neurons, their scaled
+  // activations, and where the class-0 block leaves the second count
+  const uint32_t *won2;
+  uint32_t *won2_clear;
+  const float *sc2;
+  uint32_t *group_base2_out, *group_count2_out;
   const float *sc;      // scaled activations of the windows
   uint32_t n;           // windows of the step
   uint32_t *order_out;  // a neuron's window ids beyond what LDS stages go through here
@@ -157,9 +163,11 @@ __device__ __forceinline__ void fv_sparse_count_any(uint32_t *cnt, Ord *ord, uin
 // the owners arrive; the results do not depend on that order.
 // Called by the whole block with the neuron's window ids staged by rank in ord[0 .. c_h) (c_h * stride <= the
 // block's threads), cnt[] zero and x_h = xx[h].
-template <typename Ord>
-__device__ __forceinline__ void fv_sparse_light(const fv_sparse_args &a, uint32_t h, uint32_t blk, uint32_t c_h, float x_h,
-                                                uint32_t *cnt, const Ord *ord, uint32_t *cls_n, uint32_t *sh_hits,
+// DELTA: ord[c_h .. c_h + c2_h) holds the windows in which the neuron came second; a column's two counts share a
+// 32-bit counter (cnt[] then has a word for every column of a class), the first in the low half.
+template <bool DELTA, typename Ord>
+__device__ __forceinline__ void fv_sparse_light(const fv_sparse_args &a, uint32_t h, uint32_t blk, uint32_t c_h, uint32_t c2_h,
+                                                float x_h, uint32_t *cnt, const Ord *ord, uint32_t *cls_n, uint32_t *sh_hits,
                                                 float *wave_max) {
   const uint32_t tid = threadIdx.x;
   const uint32_t n_cols = 2 * a.V;
@@ -168,7 +176,8 @@ __device__ __forceinline__ void fv_sparse_light(const fv_sparse_args &a, uint32_
   fv_lds_barrier();
   // the thread's window position: entry tid of the neuron's c_h rows of the index matrix
   const uint32_t j = tid / a.stride, c = tid - j * a.stride;
-  const bool inside = j < c_h;
+  const bool inside = j < c_h + c2_h;
+  const bool second = DELTA && j >= c_h;  // a position of a window in which the neuron came second
   const int32_t iv = a.idx[(uint64_t)ord[inside ? j : 0u] * a.stride + c];
   const bool real = inside && (uint32_t)iv < n_cols;
   const uint32_t col = real ? (uint32_t)iv : 0u;
@@ -178,30 +187,42 @@ __device__ __forceinline__ void fv_sparse_light(const fv_sparse_args &a, uint32_
   const float l = col >= a.V ? a.lmid : a.lbase;
   const float2 top2 = a.top2_known ? a.row_top2[h] : make_float2(0.0f, 0.0f);
   const uint32_t cls = col & (FV_NB_CLASSES - 1), t = col >> FV_NB_CLASS_SHIFT;
-  const uint32_t shift = 16u * (t & 1u);
+  // the element's counter: half of word t / 2, or, with two counts to keep, word t
+  const uint32_t shift = DELTA ? 0u : 16u * (t & 1u), at = DELTA ? t : t >> 1;
   uint32_t hits1 = 0, hits2 = 0;  // the same in all lanes of a wave
   float ds_max = 0.0f;
   for (uint32_t q = 0; q < FV_NB_CLASSES; ++q) {
     const bool mine = real && cls == q;
     bool owner = false;
-    if (mine) owner = ((atomicAdd(&cnt[t >> 1], 1u << shift) >> shift) & 0xffffu) == 0u;
+    if (mine) {
+      const uint32_t old = atomicAdd(&cnt[at], second ? 0x10000u : 1u << shift);
+      owner = DELTA ? old == 0u : ((old >> shift) & 0xffffu) == 0u;
+    }
     fv_lds_barrier();  // every occurrence of the class is counted
-    uint32_t n = 0, number = 0;
+    uint32_t n = 0, n2 = 0, number = 0;
     if (owner) {
-      n = (cnt[t >> 1] >> shift) & 0xffffu;
+      const uint32_t word = cnt[at];
+      n = (word >> shift) & 0xffffu;
+      n2 = DELTA ? word >> 16 : 0u;
       number = atomicAdd(&cls_n[q], 1u);
     }
     fv_lds_barrier();  // the counts are read
     if (owner) {
-      atomicAnd(&cnt[t >> 1], 0xffff0000u >> shift);  // zero again for the next class
+      if (DELTA)
+        cnt[at] = 0;  // zero again for the next class
+      else
+        atomicAnd(&cnt[at], 0xffff0000u >> shift);
       fv_slot rec;
       rec.p = p;
       rec.n = n;
       rec.wv = wv;
       rec.f = f;
-      a.slots[(uint64_t)((h << FV_NB_CLASS_SHIFT) | q) * a.slot_region + number] = rec;
+      const uint64_t place = (uint64_t)((h << FV_NB_CLASS_SHIFT) | q) * a.slot_region + number;
+      a.slots[place] = rec;
+      if (DELTA) a.slot_n2[place] = n2;
       a.Wt[p] = fv_sentinel(number);
-      if (x_h != 0.0f) ds_max = fv_absmax_keep(ds_max, fv_sparse_ds(x_h, wv, f, n, l));
+      if (x_h != 0.0f)
+        ds_max = fv_absmax_keep(ds_max, DELTA ? fv_sparse_ds2(x_h, wv, f, n, a.delta, n2, l) : fv_sparse_ds(x_h, wv, f, n, l));
     }
     const float aw = fabsf(wv);
     hits1 += (uint32_t)__popcll(__ballot(owner && aw == top2.x));
@@ -238,9 +259,8 @@ __device__ __forceinline__ void fv_sparse_light(const fv_sparse_args &a, uint32_
 // as the grouping launch it replaces lasts; only the one-word form is instantiated.)
 template <bool DELTA, bool GROUPING, int CW, bool IDS16 = GROUPING, int NW = 1>
 __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
-  static_assert(!(DELTA && GROUPING), "the anti-Hebbian form has its two lists grouped by launches of their own");
-  __shared__ uint32_t cnt[CW];
-  __shared__ uint32_t cnt2[DELTA ? CW : 4];
+  __shared__ uint32_t cnt_all[DELTA ? 2 * CW : CW];  // (one array: the form for neurons with few windows uses all of it)
+  uint32_t *const cnt = cnt_all, *const cnt2 = cnt_all + (DELTA ? CW : 0);
   __shared__ uint16_t list[FV_SP_LIST_CAP];
   // window ids of a grouping step (at most 64 * FV_SP_THREADS windows, and the padding row behind them)
   // fit 16 bits: the smaller array lets one more block share a compute unit
@@ -265,6 +285,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
 #pragma unroll
   for (int i = 0; i < NW; ++i) mask[i] = 0;
   uint32_t eq = 0;  // the thread's matches
+  // anti-Hebbian form: the windows in which the neuron came second, likewise
+  uint64_t mask2 = 0;
+  uint32_t eq2 = 0, my_off2 = 0, c2_grouped = 0;
   // scaled activations a thread fetches before it knows how many it needs: four, or sixteen in a wave with a
   // thread that has more than four matches (a neuron that won a tenth of the minibatch has seven per thread)
   constexpr int PF = 4, PF_BIG = 16;
@@ -275,6 +298,8 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     const uint32_t n = a.n;
     // (the counters are cleared while the bit row travels)
     for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt)[i] = make_uint4(0, 0, 0, 0);
+    if (DELTA)
+      for (uint32_t i = tid; i < CW / 4; i += T) ((uint4 *)cnt2)[i] = make_uint4(0, 0, 0, 0);
     // thread t takes windows 64 NW t .. 64 NW (t + 1) - 1: 2 NW words of the neuron's row
     r0 = 64 * NW * tid;
 #pragma unroll
@@ -286,11 +311,21 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     }
 #pragma unroll
     for (int i = 0; i < NW; ++i) eq += (uint32_t)__popcll(mask[i]);
+    if (DELTA) {
+      const uint32_t word = 2 * tid;
+      uint2 mw = make_uint2(0u, 0u);
+      if (word < a.won_words) mw = *(const uint2 *)(a.won2 + (uint64_t)h * a.won_words + word);
+      mask2 = (uint64_t)mw.x | ((uint64_t)mw.y << 32);
+      eq2 = (uint32_t)__popcll(mask2);
+    }
     if (q == 0) {
 #pragma unroll
       for (int i = 0; i < NW; ++i) {
         const uint32_t word = 2 * (NW * tid + i);
-        if (word < a.won_words) *(uint2 *)(a.won_clear + (uint64_t)h * a.won_words + word) = make_uint2(0u, 0u);
+        if (word < a.won_words) {
+          *(uint2 *)(a.won_clear + (uint64_t)h * a.won_words + word) = make_uint2(0u, 0u);
+          if (DELTA) *(uint2 *)(a.won2_clear + (uint64_t)h * a.won_words + word) = make_uint2(0u, 0u);
+        }
       }
     }
     // the scaled activations of a thread's matches travel while the scan runs
@@ -318,8 +353,31 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       }
 #undef FV_SP_FETCH
     }
-    // one block scan gives the ranks and the neuron's count
-    const uint32_t incl = fv_wave_inclusive_scan_u32(eq);
+    // anti-Hebbian form: the second neurons' activations, times -delta (flyvec/src/cuda_funcs.cu:726-734), summed
+    // like the others; a thread's group in row order, eight loads in flight
+    float part2 = 0.0f;
+    if (DELTA) {
+      uint64_t left = mask2;
+      while (__ballot(left != 0ull)) {
+        float v[8];
+        uint64_t l2 = left;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint32_t r = l2 ? r0 + (uint32_t)__ffsll((long long)l2) - 1 : r0;
+          l2 &= l2 - 1;
+          v[e] = a.sc2[min(r, n - 1)];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if (left) part2 = __fadd_rn(part2, __fmul_rn(-a.delta, v[e]));
+          left &= left - 1;
+        }
+      }
+    }
+    // one block scan gives the ranks and the neuron's count (both lists' as the halves of a word: a step of this
+    // form has fewer than 2^16 windows)
+    const uint32_t both = eq | (eq2 << 16);
+    const uint32_t incl = fv_wave_inclusive_scan_u32(both);
     if ((tid & 63u) == 63u) red[tid >> 6] = incl;
     fv_lds_barrier();
     uint32_t before = 0, total = 0;
@@ -329,8 +387,10 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       before += i < (tid >> 6) ? t : 0u;
       total += t;
     }
-    c_h = total;
-    my_off = before + incl - eq;
+    c_h = total & 0xffffu;
+    c2_grouped = total >> 16;
+    my_off = ((before + incl - both) & 0xffffu);
+    my_off2 = (before + incl - both) >> 16;
     // The launch lasts as long as its few heaviest blocks: their waves go first wherever they share a
     // SIMD with the waves of light blocks.
     if (c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
@@ -361,6 +421,8 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
         }
       }
       x_h = fv_block_tree_sum(part, wave_max);
+      // the second neurons' total is added to the winners' (the checker's order)
+      if (DELTA) x_h = __fadd_rn(x_h, fv_block_tree_sum(part2, wave_max));
     }
     base = 0;
     if (c_h != 0 && a.slot_region == 0) {
@@ -397,11 +459,15 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       a.group_base_out[h] = base;  // used where it was counted
       a.group_count_out[h] = c_h;
       a.xx_out[h] = x_h;  // (+0 for a neuron without a window)
+      if (DELTA) {
+        a.group_base2_out[h] = 0;
+        a.group_count2_out[h] = c2_grouped;
+      }
     }
   } else {
     c_h = a.group_count[h];
   }
-  const uint32_t c2_h = DELTA ? a.group_count2[h] : 0u;
+  const uint32_t c2_h = DELTA ? (GROUPING ? c2_grouped : a.group_count2[h]) : 0u;
   if (c_h == 0 && c2_h == 0) {
     if (tid == 0) {
       a.bmax_sparse[blk] = 0.0f;
@@ -413,8 +479,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   if (GROUPING) {
     // a neuron with no more window positions than the block has threads: all of it in the class-0 block
     const uint32_t class_cols0 = (2 * a.V + FV_NB_CLASSES - 1) >> FV_NB_CLASS_SHIFT;
-    const bool light = a.light && a.slot_region != 0 && c_h * a.stride <= T &&
-                       class_cols0 <= 2u * CW;  // (the same answer in the neuron's four blocks)
+    // (the same answer in the neuron's four blocks; both forms have a counter for every column of a class: halves
+    // of CW words, or, with two counts per column, 2 CW words)
+    const bool light = a.light && a.slot_region != 0 && (c_h + c2_h) * a.stride <= T && class_cols0 <= 2u * CW;
     if (light) {
       if (q != 0) {
         if (tid == 0) {
@@ -428,8 +495,12 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
 #pragma unroll
         for (int i = 0; i < NW; ++i)
           for (uint64_t mm = mask[i]; mm; mm &= mm - 1) ord[at++] = (ord_t)(r0 + 64 * i + (uint32_t)__ffsll((long long)mm) - 1);
+        if (DELTA) {
+          at = c_h + my_off2;  // behind them those in which the neuron came second
+          for (uint64_t mm = mask2; mm; mm &= mm - 1) ord[at++] = (ord_t)(r0 + (uint32_t)__ffsll((long long)mm) - 1);
+        }
       }
-      fv_sparse_light<ord_t>(a, h, blk, c_h, x_h, cnt, ord, red2, sh_hits, wave_max);
+      fv_sparse_light<DELTA, ord_t>(a, h, blk, c_h, c2_h, x_h, cnt, ord, red2, sh_hits, wave_max);
       return;
     }
   }
@@ -440,7 +511,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   // (GROUPING: done as soon as the count was known) the waves of the few heaviest blocks go first
   if (!GROUPING && c_h > FV_SP_HEAVY) __builtin_amdgcn_s_setprio(3);
   if (!GROUPING) base = a.group_base[h];
-  const uint32_t base2 = DELTA ? a.group_base2[h] : 0u;
+  const uint32_t base2 = DELTA && !GROUPING ? a.group_base2[h] : 0u;
   if (!GROUPING) x_h = a.xx[h];
   float ds_max = 0.0f;
   const uint32_t *order = (GROUPING ? a.order_out : a.order) + base;  // GROUPING: also written here, through order_out
@@ -462,13 +533,13 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   // GROUPING: the window ids of ranks [j0, j0 + FV_SP_STAGE) into LDS, every thread those of its own matches (its
   // ranks start at my_off; a neuron with more windows than LDS stages is staged part by part, each time
   // from the bit row's words in registers)
-  auto stage_ids = [&](uint32_t j0) {
-    uint32_t at = my_off - j0;  // wraps below 0 for the ranks in front of the part
+  auto stage_ids = [&](uint32_t j0, int second = 0) {
+    uint32_t at = (second ? my_off2 : my_off) - j0;  // wraps below 0 for the ranks in front of the part
     // the two halves of a word one after the other, four matches between two branches, as many rounds as the
     // wave's busiest thread needs (a taken branch costs a lone wave as much as four or five instructions)
 #pragma unroll
     for (int half = 0; half < 2 * NW; ++half) {
-      uint32_t mm = (uint32_t)(mask[half >> 1] >> (32 * (half & 1)));
+      uint32_t mm = (uint32_t)((second ? mask2 : mask[half >> 1]) >> (32 * (half & 1)));
       const uint32_t first = r0 + 32u * half;
       const uint32_t rounds = (fv_wave_max_u32((uint32_t)__popc(mm)) + 3u) >> 2;
       for (uint32_t it = 0; it < rounds; ++it) {
@@ -511,7 +582,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
         if (!staged_once) {
           fv_lds_barrier();  // the previous part has been counted
           if (GROUPING) {
-            stage_ids(j0);
+            stage_ids(j0, l);
           } else {
             for (uint32_t i = tid; i < n_staged; i += T) ord[i] = (ord_t)ids[j0 + i];
           }
@@ -670,4 +741,12 @@ __global__ __launch_bounds__(FV_SP_THREADS) __attribute__((amdgpu_waves_per_eu(6
 
 __global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_grouping_wide_kernel(fv_sparse_args a) {
   fv_sparse_block<false, true, FV_NB_CNT_WORDS_WIDE>(a);
+}
+
+// The anti-Hebbian form that groups for itself: both of a neuron's window lists from bit rows. With two counter
+// arrays of full length it takes 47 KB of LDS and three blocks share a compute unit (arrays of half the length, six
+// blocks, two counting passes per class measured 3 us slower at 10000 windows of 11 over 400 neurons).
+template <int CW>
+__global__ __launch_bounds__(FV_SP_THREADS) void fv_sparse_grouping_delta_kernel(fv_sparse_args a) {
+  fv_sparse_block<true, true, CW>(a);
 }

@@ -63,6 +63,14 @@ struct fv_trainer {
   uint32_t *won[2];        // K rows of won_words words each
   uint32_t won_words;      // words per row (even)
   uint32_t won_parity;     // the pair the last such step used
+  // the same for the second neurons of the anti-Hebbian form (allocated with its other buffers; its own parity: it
+  // changes only with the steps that use the rows)
+  uint32_t *won2[2];
+  uint32_t won2_parity;
+  // records per block of the sparse launch when that form groups for itself (like slots_blocks) and their second counts
+  fv_slot *slots2_blocks;
+  uint32_t *slot_n2_blocks;
+  bool last_delta_grouped;  // the form the last whole anti-Hebbian step took
   // anti-Hebbian form (delta != 0), allocated with the first such step: the second neuron of every
   // window, its scaled activation, the windows grouped by it, the second count of every slot record
   int32_t *win2;

@@ -616,22 +616,28 @@ def test_large_config_shape(gpu, oracle_lib):
 
 # ---- anti-Hebbian term (delta != 0) -----------------------------------------------------------------
 
-def run_both_delta(to, V, K, w, B, steps, delta, tie=0, n_tokens=60000, W0=None, sigma=0.02, seed=0):
+def run_both_delta(to, V, K, w, B, steps, delta, tie=0, n_tokens=60000, W0=None, sigma=0.02, seed=0, separate=False,
+                   launches=0, mixed=False):
+    """separate: the two lists of a neuron's windows grouped by launches of their own (else inside the sparse launch
+    wherever the trainer has the bit rows and the regions for it); mixed: every third step without the term."""
     from flyvec_amd import synthetic
     tokens, offsets = small_corpus(n_tokens, V, seed=seed)
     if W0 is None:
         W0 = synthetic.synapses(K, V, seed=5 + seed, sigma=sigma)
-    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, tie=tie)
+    t, perm = make_trainer(tokens, offsets, V, K, w, B, W0, tie=tie, launches=launches)
+    t.set_grouping_launch(separate)
     starts, invf = oracle_inputs(to, tokens, offsets, V, w)
     eps = t.epoch_eps(0, 15)
     steps = min(steps, t.num_windows // B)
     Wo = W0.copy()
     for s in range(steps):
-        t.step(s * B, B, eps, delta=delta)
+        d = 0.0 if mixed and s % 3 == 1 else delta
+        t.step(s * B, B, eps, delta=d)
         idx = to.inflate(tokens, starts, perm, s * B, B, w, V)
-        ref = to.train_step(Wo, idx, invf, eps, tie_rule=tie, delta=delta)
+        ref = to.train_step(Wo, idx, invf, eps, tie_rule=tie, delta=d)
         assert np.array_equal(t.winners(B), ref["winners"]), f"winners, step {s}"
-        assert np.array_equal(t.second_winners(B), ref["seconds"]), f"second neurons, step {s}"
+        if d:
+            assert np.array_equal(t.second_winners(B), ref["seconds"]), f"second neurons, step {s}"
         xx, nc = t.step_stats()
         assert np.array_equal(xx, ref["xx"]) and nc == ref["nc"], f"xx / max|ds|, step {s}"
     Wg = t.get_weights()
@@ -639,18 +645,52 @@ def run_both_delta(to, V, K, w, B, steps, delta, tie=0, n_tokens=60000, W0=None,
     return Wg, Wo
 
 
+@pytest.mark.parametrize("separate", [False, True])
 @pytest.mark.parametrize("tie", [0, 1])
-def test_delta_small_config_bit_exact(gpu, oracle_lib, tie):
-    Wg, Wo = run_both_delta(oracle_lib, V=500, K=400, w=11, B=512, steps=10, delta=0.4, tie=tie)
+def test_delta_small_config_bit_exact(gpu, oracle_lib, tie, separate):
+    Wg, Wo = run_both_delta(oracle_lib, V=500, K=400, w=11, B=512, steps=10, delta=0.4, tie=tie, separate=separate)
     assert np.array_equal(Wg, Wo)
 
 
+@pytest.mark.parametrize("separate", [False, True])
 @pytest.mark.parametrize("K,w,V,B", [(1, 1, 5, 1), (2, 3, 9, 7), (65, 15, 200, 256), (130, 64, 300, 64),
-                                     (30, 11, 30000, 700), (20, 7, 22000, 500)])  # the last: the wider counter arrays
-def test_delta_shapes_bit_exact(gpu, oracle_lib, K, w, V, B):
+                                     (30, 11, 30000, 700), (20, 7, 22000, 500),   # the wider counter arrays
+                                     (400, 11, 3000, 4000), (96, 9, 500, 16384)])
+def test_delta_shapes_bit_exact(gpu, oracle_lib, K, w, V, B, separate):
     n_tokens = 40000 if V < 20000 else 120000
-    Wg, Wo = run_both_delta(oracle_lib, V=V, K=K, w=w, B=B, steps=4, delta=0.25, n_tokens=n_tokens)
+    n_tokens = max(n_tokens, 8 * B)
+    Wg, Wo = run_both_delta(oracle_lib, V=V, K=K, w=w, B=B, steps=4, delta=0.25, n_tokens=n_tokens, separate=separate)
     assert np.array_equal(Wg, Wo)
+
+
+@pytest.mark.parametrize("launches", [1, 2, 3])
+def test_delta_grouped_inside_the_sparse_launch(gpu, oracle_lib, launches):
+    """The anti-Hebbian step whose sparse launch takes both of a neuron's window lists from bit rows (no grouping
+    launches), at a shape where every block of that launch has a slot region of its own: every dense-launch form,
+    steps with and without the term in turn (the second neurons' bit rows keep a parity of their own), and the
+    epoch driver with the schedule."""
+    from flyvec_amd import Trainer, synthetic
+    to = oracle_lib
+    V, K, w, B = 1500, 130, 11, 3000
+    Wg, Wo = run_both_delta(to, V=V, K=K, w=w, B=B, steps=7, delta=0.4, n_tokens=90000, launches=launches, mixed=True)
+    assert np.array_equal(Wg, Wo)
+    tokens, offsets = small_corpus(30000, V, seed=4)
+    W0 = synthetic.synapses(K, V, seed=2, sigma=0.02)
+    t = Trainer(V, K, w, B, initial_learning_rate=1e-3, delta=0.3)
+    t.set_dense_launches(launches)
+    t.set_corpus(tokens, offsets)
+    t.set_weights(W0)
+    t.shuffle(3)
+    perm = t.get_permutation()
+    starts, invf = oracle_inputs(to, tokens, offsets, V, w)
+    assert len(starts) % B != 0 and len(starts) > 2 * B
+    Wo = W0.copy()
+    for ep in (0, 9):
+        t.run_epoch(ep, 15)
+        to.train_steps(Wo, tokens, starts, perm, 0, B, len(starts) // B + 1, w, invf, to.epoch_eps(1e-3, ep, 15),
+                       delta=to.epoch_delta(0.3, ep, 15))
+        assert np.array_equal(t.get_weights().view(np.uint32), Wo.view(np.uint32)), ep
+    t.close()
 
 
 def test_delta_with_ties_and_heavy_neurons(gpu, oracle_lib):
