@@ -61,6 +61,7 @@ SIGNATURES = {
     "fv_build_window_starts": [_vp, _u64, _u64, _vp, _u64],
     "fv_inverse_frequency": [_vp, _u64, _u64, _vp],
     "fv_inverse_frequency_static": [_vp, _u64, _u64, _vp],
+    "fv_histogram_stops_from": [_u64],
     "fv_mask_tokens": [_vp, _u64, _vp, _u64, _u64],
     "fv_prune_windows": [_vp, _u64, _u64],
     "fv_trainer_create": [C.POINTER(TrainConfig), _pp],

@@ -10,6 +10,8 @@
 //     histogram clamped to 2^24 gives the same value. The counters saturate (at 2^31) instead of wrapping,
 //     so a corpus of any length is counted right: the reference indexes its corpus with uint64_t
 //     (flyvec/src/model_arrays.cu:396-424) and was run on 5.8 G tokens (flyvec/src/test_inv.cpp:10-11).
+#include <atomic>
+
 #include "fv_internal.h"
 #include "fv_histogram.h"
 
@@ -176,6 +178,10 @@ __device__ __forceinline__ void fv_saturating_add(uint32_t *counter, uint32_t ad
   }
 }
 
+// STOPS: the counters in HBM stop at FV_HIST_SATURATED instead of wrapping, for a corpus long enough that one could
+// get there; the block's additions are then compare-and-swap loops, which under the contention of 2048 blocks on the
+// same few thousand counters take some 10 ms in all, against 0.2 ms for the plain additions of the other form.
+template <bool STOPS>
 __global__ __launch_bounds__(256) void fv_histogram_kernel(const int32_t *__restrict__ corpus,
                                                            uint64_t n_tokens, uint32_t vocab,
                                                            uint32_t *__restrict__ counts,
@@ -192,6 +198,8 @@ __global__ __launch_bounds__(256) void fv_histogram_kernel(const int32_t *__rest
     if (t >= 0 && (uint32_t)t < vocab) {
       if (t < FV_HIST_LDS) {
         atomicAdd(&hist[t], 1u);
+      } else if (!STOPS) {
+        atomicAdd(&counts[t], 1u);
       } else if (atomicAdd(&counts[t], 1u) >= FV_HIST_SATURATED + (1u << 30)) {
         // far beyond the stop: back to it. Every thread that sees this writes the same value, and between the
         // stop and the wrap lie 2^30 more additions than there are threads in flight.
@@ -202,7 +210,12 @@ __global__ __launch_bounds__(256) void fv_histogram_kernel(const int32_t *__rest
   __syncthreads();
   const uint32_t lim = vocab < FV_HIST_LDS ? vocab : FV_HIST_LDS;
   for (uint32_t i = threadIdx.x; i < lim; i += 256)
-    if (hist[i]) fv_saturating_add(&counts[i], hist[i]);
+    if (hist[i]) {
+      if (STOPS)
+        fv_saturating_add(&counts[i], hist[i]);
+      else
+        atomicAdd(&counts[i], hist[i]);
+    }
   for (int d = 32; d >= 1; d >>= 1) {
     int32_t ol = __shfl_down(lo, d, 64), oh = __shfl_down(hi, d, 64);
     lo = ol < lo ? ol : lo;
@@ -212,6 +225,25 @@ __global__ __launch_bounds__(256) void fv_histogram_kernel(const int32_t *__rest
     atomicMin(&minmax[0], lo);
     atomicMax(&minmax[1], hi);
   }
+}
+
+// A corpus shorter than the stop cannot bring a counter there: plain additions. fv_histogram_stops_from (a test
+// hook) lowers the length from which the other form is taken.
+static std::atomic<uint64_t> fv_hist_stops_from{FV_HIST_SATURATED};
+
+extern "C" int fv_histogram_stops_from(uint64_t n_tokens) {
+  fv_hist_stops_from.store(n_tokens ? n_tokens : (uint64_t)FV_HIST_SATURATED);
+  return FV_OK;
+}
+
+static void fv_launch_histogram(unsigned blocks, hipStream_t stream, const int32_t *corpus_dev, uint64_t n_tokens,
+                                uint32_t vocab, uint32_t *counts, int32_t *minmax) {
+  if (n_tokens >= fv_hist_stops_from.load())
+    hipLaunchKernelGGL(fv_histogram_kernel<true>, dim3(blocks), dim3(256), 0, stream, corpus_dev, n_tokens, vocab, counts,
+                       minmax);
+  else
+    hipLaunchKernelGGL(fv_histogram_kernel<false>, dim3(blocks), dim3(256), 0, stream, corpus_dev, n_tokens, vocab, counts,
+                       minmax);
 }
 
 __global__ void fv_invert_counts_kernel(const uint32_t *__restrict__ counts, uint32_t vocab,
@@ -237,8 +269,7 @@ int fv_dev_inverse_frequency(const int32_t *corpus_dev, uint64_t n_tokens, uint6
     e = hipMemcpyAsync(minmax, init, sizeof init, hipMemcpyHostToDevice, stream);
   if (e == hipSuccess && n_tokens) {
     const unsigned blocks = fv_hist_blocks(n_tokens);
-    hipLaunchKernelGGL(fv_histogram_kernel, dim3(blocks), dim3(256), 0, stream, corpus_dev, n_tokens,
-                       (uint32_t)vocab, counts, minmax);
+    fv_launch_histogram(blocks, stream, corpus_dev, n_tokens, (uint32_t)vocab, counts, minmax);
     e = hipGetLastError();
   }
   if (e == hipSuccess) {
@@ -396,8 +427,7 @@ extern "C" int fv_inverse_frequency_static(const int32_t *corpus_dev, uint64_t n
   hipLaunchKernelGGL(fv_static_clear_kernel, dim3(clear_blocks), dim3(256), 0, stream, counts, (uint32_t)vocab, minmax);
   if (n_tokens) {
     const unsigned blocks = fv_hist_blocks(n_tokens);
-    hipLaunchKernelGGL(fv_histogram_kernel, dim3(blocks), dim3(256), 0, stream, corpus_dev, n_tokens, (uint32_t)vocab,
-                       counts, minmax);
+    fv_launch_histogram(blocks, stream, corpus_dev, n_tokens, (uint32_t)vocab, counts, minmax);
   }
   hipLaunchKernelGGL(fv_invert_counts_kernel, dim3((unsigned)((vocab + 255) / 256)), dim3(256), 0, stream, counts,
                      (uint32_t)vocab, out_invf_dev);

@@ -94,6 +94,12 @@ int fv_inverse_frequency(const int32_t *corpus, uint64_t n_tokens, uint64_t voca
 int fv_inverse_frequency_static(const int32_t *corpus_dev, uint64_t n_tokens, uint64_t vocab,
                                 float *out_invf_dev);
 
+/* Test hook. The token histogram behind 1/frequency keeps 32-bit counters in HBM. A corpus of fewer than 2^31
+ * tokens cannot bring one to 2^31 and is counted with plain additions; a longer one is counted by a form whose
+ * counters stop at 2^31 instead of wrapping (the result is clamped to 2^24 either way). n_tokens > 0: corpora of
+ * at least that many tokens take the second form; 0 restores 2^31. Process-wide. No counterpart in the reference. */
+int fv_histogram_stops_from(uint64_t n_tokens);
+
 /* flyvec/src/remove_words.cpp:28-37 (an off-line tool of the reference: for every id of a stop list,
  * data[w] == id ? -1): rewrites `tokens` in place, every occurrence of an id of `remove_ids`
  * becomes -1 (masked: such a position contributes nothing to a window). One pass on the device,
@@ -243,10 +249,11 @@ int fv_trainer_set_slot_regions(fv_trainer *t, uint32_t per_block);
  * default; 0 keeps the four class blocks for every neuron. Results are bit-identical either way. No counterpart
  * in the reference. */
 int fv_trainer_set_light_blocks(fv_trainer *t, uint32_t on);
-/* Test hook. A block of the single dense launch notes the sparse elements it meets (their sentinels) in an LDS
- * list and finishes them when its dense elements are done; an element that finds the list full is finished on
- * the spot. entries > 0 makes the list count as full after that many (no more than it holds: 2048, or 8192 in
- * the streaming form), 0 restores its size. Results are bit-identical. No counterpart in the reference. */
+/* Test hook. The single dense launch notes the sparse elements it meets (their sentinels) in LDS lists, one of
+ * 256 entries per wave in the register form, one of 8192 per block in the streaming form, and finishes them when
+ * its dense elements are done; an element that finds its list full is finished by its own thread. entries > 0
+ * makes a list count as full after that many (no more than it holds), 0 restores its size. Results are
+ * bit-identical. No counterpart in the reference. */
 int fv_trainer_set_sentinel_list(fv_trainer *t, uint32_t entries);
 /* Test hook: between its two passes a single-launch dense pass waits for all its blocks, at most
  * `rounds` polling rounds (2^14 by default, tens of milliseconds); 0 makes every block give up at once, which

@@ -60,6 +60,27 @@ def test_inverse_frequency_saturation(gpu, oracle_lib):
     assert got[0] == np.float32(1.0 / float(1 << 24)) and got[1] == np.float32(1.0 / 7.0)
 
 
+def test_inverse_frequency_in_the_form_whose_counters_stop(gpu, oracle_lib):
+    """A corpus of 2^31 tokens or more is counted by a kernel whose counters in HBM stop instead of wrapping; the test
+    hook sends a small corpus through it: same result as the plain form and as the oracle, ids above and below
+    the part of the vocabulary a block counts in LDS."""
+    from flyvec_amd import inverse_frequency, _lib
+    lib = _lib.load()
+    V = 30000
+    rng = np.random.default_rng(11)
+    corpus = np.minimum(rng.zipf(1.2, size=1_500_000) - 1, V - 1).astype(np.int32)
+    corpus[::7] = V - 1 - (np.arange(len(corpus[::7])) % 9000).astype(np.int32)   # counted in HBM directly
+    corpus[5::1001] = -1
+    plain = inverse_frequency(corpus, V)
+    try:
+        assert lib.fv_histogram_stops_from(1) == 0
+        stops = inverse_frequency(corpus, V)
+    finally:
+        assert lib.fv_histogram_stops_from(0) == 0
+    want = oracle_lib.inverse_frequency(corpus, V)
+    assert np.array_equal(plain, want) and np.array_equal(stops, want)
+
+
 def test_trainer_tables_match_the_standalone_functions(gpu, oracle_lib):
     from flyvec_amd import Trainer
     V = 300
