@@ -370,9 +370,9 @@ __device__ __forceinline__ void fv_finish_sparse_element(const fv_dense_args &a,
   const uint32_t col = p / a.ldk, h = p - col * a.ldk;
   // the sentinel's number counts from the start of the slots, or of the region of the sparse launch's block
   // that owns the element
-  const uint64_t at = a.slot_region
-                          ? (uint64_t)((h << FV_NB_CLASS_SHIFT) | (col & (FV_NB_CLASSES - 1))) * a.slot_region + number
-                          : number;
+  const uint64_t at = a.slot_region ? fv_slot_place((h << FV_NB_CLASS_SHIFT) | (col & (FV_NB_CLASSES - 1)), number,
+                                                    a.slot_region, a.K * FV_NB_CLASSES)
+                                    : number;
   const fv_slot sl = a.slots[at];
   if (sl.p != p) return;
   const float x = xs[h];
@@ -406,9 +406,9 @@ __device__ __forceinline__ void fv_finish_sparse_elements(const fv_dense_args &a
       const uint32_t number = (hit[u].x & FV_SENTINEL_MAX) - 1u;
       mine[u] = i0 + u * width < n && number < a.n_slots;  // a NaN of another origin stays what it is
       const uint32_t p = hit[u].y, col = p / a.ldk, h = p - col * a.ldk;
-      const uint64_t at = a.slot_region
-                              ? (uint64_t)((h << FV_NB_CLASS_SHIFT) | (col & (FV_NB_CLASSES - 1))) * a.slot_region + number
-                              : number;
+      const uint64_t at = a.slot_region ? fv_slot_place((h << FV_NB_CLASS_SHIFT) | (col & (FV_NB_CLASSES - 1)), number,
+                                                        a.slot_region, a.K * FV_NB_CLASSES)
+                                        : number;
       sl[u] = a.slots[mine[u] ? at : 0];
       n2[u] = DELTA ? a.slot_n2[mine[u] ? at : 0] : 0u;
     }
@@ -1089,9 +1089,12 @@ __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
   }
   float m1 = 0.0f, m2 = 0.0f;
   const uint64_t slot_first =
-      a.slot_region ? (uint64_t)blockIdx.x * a.slot_region
+      a.slot_region ? 0ull
                     : (uint64_t)q * a.slot_stride + (uint64_t)(a.group_base[h] + (DELTA ? a.group_base2[h] : 0u)) * a.w;
-  const fv_slot *slots = a.slots + slot_first;
+  // record `number` of the block
+  auto place_of = [&](uint32_t number) {
+    return a.slot_region ? fv_slot_place(blockIdx.x, number, a.slot_region, gridDim.x) : slot_first + number;
+  };
   const float x = a.xx[h];
   const float nc = a.scalars[0];
   const float s = a.prec > nc ? a.eps / a.prec : a.eps / nc;
@@ -1100,8 +1103,9 @@ __global__ __launch_bounds__(256) void fv_slot_update_kernel(fv_dense_args a) {
     uint32_t n2[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      sl[u] = slots[min(eb + u * 256, count - 1)];
-      n2[u] = DELTA ? a.slot_n2[slot_first + min(eb + u * 256, count - 1)] : 0u;
+      const uint64_t place = place_of(min(eb + u * 256, count - 1));
+      sl[u] = a.slots[place];
+      n2[u] = DELTA ? a.slot_n2[place] : 0u;
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {

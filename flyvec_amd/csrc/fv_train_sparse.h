@@ -19,8 +19,8 @@ struct fv_sparse_args {
   float *Wt;
   fv_slot *slots;  // FV_NB_CLASSES regions of slot_stride records
   uint64_t slot_stride;
-  // Not 0 (grouping form only): every block has a region of slot_region records of its own in slots[], at
-  // blockIdx * slot_region, and a sentinel names a record by its place in the block's region. A block has no
+  // Not 0 (grouping form only): every block has a region of slot_region records of its own in slots[]
+  // (fv_slot_place), and a sentinel names a record by its number in the block's region. A block has no
   // more records than its class has columns, so no block needs to know what the others write.
   uint32_t slot_region;
   const float *xx;
@@ -217,7 +217,7 @@ __device__ __forceinline__ void fv_sparse_light(const fv_sparse_args &a, uint32_
       rec.n = n;
       rec.wv = wv;
       rec.f = f;
-      const uint64_t place = (uint64_t)((h << FV_NB_CLASS_SHIFT) | q) * a.slot_region + number;
+      const uint64_t place = fv_slot_place((h << FV_NB_CLASS_SHIFT) | q, number, a.slot_region, gridDim.x);
       a.slots[place] = rec;
       if (DELTA) a.slot_n2[place] = n2;
       a.Wt[p] = fv_sentinel(number);
@@ -519,9 +519,12 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   const uint32_t m_ent = max(c_h, c2_h) * a.w;
   // the block's records: no more than (c_h + c2_h) * w of them, behind those of the lower neurons
   const bool regions = GROUPING && a.slot_region != 0;
-  const uint64_t slot_first = regions ? (uint64_t)blk * a.slot_region
-                                      : (uint64_t)q * a.slot_stride + (uint64_t)(base + base2) * a.w;
-  fv_slot *slots = a.slots + slot_first;
+  // (without regions of their own: behind the records of the lower neurons in the class's part)
+  const uint64_t slot_first = regions ? 0ull : (uint64_t)q * a.slot_stride + (uint64_t)(base + base2) * a.w;
+  // where the block's records lie (fv_slot_place, the block's part of it formed once)
+  const uint32_t slot_primary = min(a.slot_region, FV_SLOT_PRIMARY);
+  const uint64_t place_low = regions ? (uint64_t)blk * slot_primary : slot_first;
+  const uint64_t place_high = regions ? fv_slot_place(blk, slot_primary, a.slot_region, gridDim.x) - slot_primary : slot_first;
 
   const uint32_t stage_cap = fv_sparse_stage_cap(a.stride);  // window ids staged in LDS at a time
   const bool staged_once = !DELTA && c_h <= stage_cap;  // the usual case: the neuron's window ids are staged here
@@ -695,8 +698,10 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
             rec.n = ne[u];
             rec.wv = wv[u];
             rec.f = fe[u];
-            slots[emitted + eb + u * T] = rec;
-            if (DELTA) a.slot_n2[slot_first + emitted + eb + u * T] = n2e[u];
+            const uint32_t number = emitted + eb + u * T;
+            const uint64_t place = (number < slot_primary ? place_low : place_high) + number;
+            a.slots[place] = rec;
+            if (DELTA) a.slot_n2[place] = n2e[u];
             a.Wt[pe[u]] = fv_sentinel(record0 + eb + u * T);
             // counted per wave from lane masks: the counts stay in scalar registers
             const float aw = fabsf(wv[u]);
