@@ -15,6 +15,12 @@
 
 #define FV_PAD_ROWS 2
 
+#if defined(__HIPCC__)
+#define FV_LAYOUT_HD __host__ __device__ __forceinline__
+#else
+#define FV_LAYOUT_HD static inline
+#endif
+
 static inline uint32_t fv_ldk(uint32_t K) { return (K + 3u) & ~3u; }
 
 // 64-float registers per lane of a wave that holds K values.
@@ -35,3 +41,19 @@ static inline uint64_t fv_matrix_alloc_elems(uint32_t K, uint64_t N) {
 static inline uint64_t fv_matrix_gather_reach(uint32_t K, uint64_t N) {
   return N * fv_ldk(K) + 64ull * fv_lane_values(K);
 }
+
+// Where record `number` of block `blk` of the sparse launch lies when every block has a region of `region` records
+// of its own (n_blocks blocks): the first FV_SLOT_PRIMARY records of all blocks side by side, the others in a second
+// part with the rest of every region. Nearly every block has fewer records than that, so a step's records lie
+// within n_blocks * FV_SLOT_PRIMARY records (26 MB at 1600 blocks) instead of being strewn over all regions (256 MB at
+// 10000 records each: the sparse launch then took 16.8 us instead of 14.8 in some processes, the address
+// translation's reach being the difference), and only the few heaviest neurons' blocks touch the second part.
+#define FV_SLOT_PRIMARY 1024u
+FV_LAYOUT_HD uint64_t fv_slot_place(uint32_t blk, uint32_t number, uint32_t region, uint32_t n_blocks) {
+  const uint32_t first = region < FV_SLOT_PRIMARY ? region : FV_SLOT_PRIMARY;
+  return number < first ? (uint64_t)blk * first + number
+                        : (uint64_t)n_blocks * first + (uint64_t)blk * (region - first) + (number - first);
+}
+
+// Records the regions of n_blocks blocks take together.
+static inline uint64_t fv_slot_regions_records(uint32_t region, uint32_t n_blocks) { return (uint64_t)region * n_blocks; }

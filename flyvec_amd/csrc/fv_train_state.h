@@ -14,21 +14,6 @@
 #include "fv_permute.h"
 #include "fv_repeat_add.h"
 
-// Where record `number` of block `blk` of the sparse launch lies when every block has a region of `region` records
-// of its own (n_blocks blocks): the first FV_SLOT_PRIMARY records of all blocks side by side, the others in a second
-// part with the rest of every region. Nearly every block has fewer records than that, so a step's records lie
-// within n_blocks * FV_SLOT_PRIMARY records (26 MB at 1600 blocks) instead of being strewn over all regions (256 MB at
-// 10000 records each: the sparse launch then took 16.8 us instead of 14.8 in some processes, the address
-// translation's reach being the difference), and only the few heaviest neurons' blocks touch the second part.
-#ifndef FV_SLOT_PRIMARY
-#define FV_SLOT_PRIMARY 1024u
-#endif
-__host__ __device__ __forceinline__ uint64_t fv_slot_place(uint32_t blk, uint32_t number, uint32_t region, uint32_t n_blocks) {
-  const uint32_t first = region < FV_SLOT_PRIMARY ? region : FV_SLOT_PRIMARY;
-  return number < first ? (uint64_t)blk * first + number
-                        : (uint64_t)n_blocks * first + (uint64_t)blk * (region - first) + (number - first);
-}
-
 // Written over W[p] while the true weight of a sparse element waits in its slot record: a NaN whose
 // 23 mantissa bits hold the number of that record plus one (so they are never all zero, which would
 // be an infinity), saturated at the largest value. A step whose record numbers all fit takes the

@@ -56,3 +56,31 @@ def test_small_hid_needs_more_than_two_pad_rows(shim):
         assert shim.fvt_pad_elems(K) == 2 * shim.fvt_ldk(K) >= 64 * -(-K // 64)
     # the case a page-aligned allocation exposes: K = 4, V = 127 (N = 254)
     assert shim.fvt_alloc_elems(4, 254) * 4 > (254 * 4 + 63 + 1) * 4 - 1
+
+
+def test_slot_records_of_all_blocks_have_places_of_their_own_inside_the_allocation(shim):
+    """fv_slot_place: record `number` of block `blk` when every block of the sparse launch has a region of `region`
+    records. Every (block, number) gets a place of its own below region * n_blocks, and the first records of all
+    blocks lie side by side at the front."""
+    shim.fvt_slot_place.restype = C.c_uint64
+    shim.fvt_slot_place.argtypes = [C.c_uint32] * 4
+    shim.fvt_slot_regions_records.restype = C.c_uint64
+    shim.fvt_slot_regions_records.argtypes = [C.c_uint32] * 2
+    shim.fvt_slot_primary.restype = C.c_uint32
+    primary = shim.fvt_slot_primary()
+    for region, n_blocks in ((1, 4), (7, 8), (primary - 1, 12), (primary, 12), (primary + 1, 12), (3 * primary + 5, 20)):
+        total = shim.fvt_slot_regions_records(region, n_blocks)
+        assert total == region * n_blocks
+        seen = set()
+        for blk in range(n_blocks):
+            for number in range(region):
+                place = shim.fvt_slot_place(blk, number, region, n_blocks)
+                assert place < total
+                seen.add(place)
+                if number < min(region, primary):
+                    assert place == blk * min(region, primary) + number
+        assert len(seen) == total          # no two records share a place
+    # the shapes the trainer meets: 1600 blocks of 10000 records, 8192 blocks of 2^23 - 2 (beyond 32 bits)
+    assert shim.fvt_slot_place(1599, 9999, 10000, 1600) == 1600 * 10000 - 1
+    big = (1 << 23) - 2
+    assert shim.fvt_slot_place(8191, big - 1, big, 8192) == 8192 * big - 1
