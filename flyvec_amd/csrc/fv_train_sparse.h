@@ -548,11 +548,11 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       for (uint32_t it = 0; it < rounds; ++it) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          if (mm) {
-            if (at < stage_cap) ord[at] = (ord_t)(first + (uint32_t)__ffs((int)mm) - 1u);
-            ++at;
-            mm &= mm - 1;
-          }
+          // (no branch around a match: one masked store, the rest by selects; a thread out of matches adds nothing)
+          const bool more = mm != 0;
+          if (more && at < stage_cap) ord[at] = (ord_t)(first + (uint32_t)__ffs((int)mm) - 1u);
+          at += more ? 1u : 0u;
+          mm &= mm - 1;
         }
       }
     }
