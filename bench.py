@@ -192,24 +192,36 @@ def bench_train(steps, warmup, cpu_seconds, c=TRAIN, which="step", dense_launche
     # the same number of steps again, timed by two HIP events on the trainer's stream
     total_ms, _ = t.time_steps((warmup + steps) * c["B"], steps, eps, per_kernel=False)
     ev_ms_per_step = total_ms / steps
-    # and as HIP graphs (a graph per step, then one graph for all), on the windows that are left
-    graph = None
-    g_steps = min(steps, (nwin // c["B"] - warmup - 2 * steps) // 2)
-    if graphs and g_steps >= 5:
-        g0 = warmup + 2 * steps
-        per_step_ms = t.time_steps_graph(g0 * c["B"], g_steps, eps, 1) / g_steps
-        whole_ms = t.time_steps_graph((g0 + g_steps) * c["B"], g_steps, eps, g_steps) / g_steps
-        graph = {"steps": g_steps, "stream_launches_ms_per_step": ev_ms_per_step,
-                 "graph_per_step_ms_per_step": per_step_ms, "one_graph_ms_per_step": whole_ms,
-                 "note": "the same kernels with the same arguments captured into HIP graphs, instantiated before "
-                         "the clock starts; HIP events on the trainer's stream"}
     # per-kernel durations: each kernel of the last step launched back to back between two HIP
-    # events on that stream (bracketing every kernel inside a step would add ~3 us of event
-    # overhead to each); this destroys W, so it comes last
+    # events on that stream (bracketing every kernel inside a step would add 3 to 5 us of event
+    # overhead to each); this destroys W, so it is the last thing this trainer does
     kern_ms = t.time_kernels(reps=50)
     launches = t.dense_launches
     grouping_separate = t.grouping_launch
     t.close()
+    # the same steps as HIP graphs (a graph per step, then one graph for all) against stream launches, in a trainer
+    # of its own: the three forms on one matrix in one state, one after the other
+    graph = None
+    g_steps = min(steps, (nwin // c["B"] - warmup) // 3)
+    if graphs and g_steps >= 5:
+        g = Trainer(c["V"], c["K"], c["w"], c["B"], initial_learning_rate=c["lr0"], prec=c["prec"])
+        g.set_dense_launches(dense_launches)
+        g.set_grouping_launch(separate_grouping)
+        g.set_corpus(tokens, offsets)
+        g.set_permutation(perm)
+        g.set_weights(W0)
+        for s in range(warmup):
+            g.step(s * c["B"], c["B"], eps)
+        g.sync()
+        stream_ms = g.time_steps(warmup * c["B"], g_steps, eps, per_kernel=False)[0] / g_steps
+        per_step_ms = g.time_steps_graph((warmup + g_steps) * c["B"], g_steps, eps, 1) / g_steps
+        whole_ms = g.time_steps_graph((warmup + 2 * g_steps) * c["B"], g_steps, eps, g_steps) / g_steps
+        g.close()
+        graph = {"steps": g_steps, "stream_launches_ms_per_step": stream_ms,
+                 "graph_per_step_ms_per_step": per_step_ms, "one_graph_ms_per_step": whole_ms,
+                 "note": "a trainer of its own, the three forms one after the other on consecutive windows: the same "
+                         "kernels with the same arguments, as stream launches and captured into HIP graphs that are "
+                         "instantiated before the clock starts; HIP events on the trainer's stream"}
 
     N = 2 * c["V"]
     per_kernel = kernel_bytes(c["K"], N, c["w"], c["B"], single_dense_launch=launches == 1)
