@@ -48,7 +48,9 @@ static inline uint64_t fv_matrix_gather_reach(uint32_t K, uint64_t N) {
 // within n_blocks * FV_SLOT_PRIMARY records (26 MB at 1600 blocks) instead of being strewn over all regions (256 MB at
 // 10000 records each: the sparse launch then took 16.8 us instead of 14.8 in some processes, the address
 // translation's reach being the difference), and only the few heaviest neurons' blocks touch the second part.
+#ifndef FV_SLOT_PRIMARY
 #define FV_SLOT_PRIMARY 1024u
+#endif
 FV_LAYOUT_HD uint64_t fv_slot_place(uint32_t blk, uint32_t number, uint32_t region, uint32_t n_blocks) {
   const uint32_t first = region < FV_SLOT_PRIMARY ? region : FV_SLOT_PRIMARY;
   return number < first ? (uint64_t)blk * first + number
