@@ -53,7 +53,13 @@ static inline uint64_t fv_matrix_gather_reach(uint32_t K, uint64_t N) {
 #endif
 FV_LAYOUT_HD uint64_t fv_slot_place(uint32_t blk, uint32_t number, uint32_t region, uint32_t n_blocks) {
   const uint32_t first = region < FV_SLOT_PRIMARY ? region : FV_SLOT_PRIMARY;
-  return number < first ? (uint64_t)blk * first + number
+  // (the usual case in 32 bits: n_blocks * first is at most 2^13 * 2^10; on the device the other case is a branch
+  // the wave takes only if one of its lanes has such a record, so that the usual one stays one instruction)
+  const uint32_t low = blk * first + number;
+#if defined(__HIP_DEVICE_COMPILE__)
+  if (!__any(number >= first)) return low;
+#endif
+  return number < first ? (uint64_t)low
                         : (uint64_t)n_blocks * first + (uint64_t)blk * (region - first) + (number - first);
 }
 

@@ -817,6 +817,7 @@ static int fv_enqueue_step(fv_trainer *t, uint64_t first, uint32_t n, float eps,
   sp.Wt = t->Wt;
   sp.slots = anti ? (slot_region ? t->slots2_blocks : t->slots2) : slot_region ? t->slots_blocks : t->slots;
   sp.slot_region = slot_region;
+  sp.n_blocks = t->K * FV_NB_CLASSES;
   sp.slot_stride = (uint64_t)t->B * t->w * (anti ? 2 : 1);
   sp.order2 = t->order2;
   sp.group_base2 = t->group_base2;

@@ -23,6 +23,7 @@ struct fv_sparse_args {
   // (fv_slot_place), and a sentinel names a record by its number in the block's region. A block has no
   // more records than its class has columns, so no block needs to know what the others write.
   uint32_t slot_region;
+  uint32_t n_blocks;  // blocks of the launch (what fv_slot_place needs; read from the arguments, not from the dispatch packet)
   const float *xx;
   const float *invf;
   float *bmax_sparse;    // one maximum of |ds| per block
@@ -217,7 +218,8 @@ __device__ __forceinline__ void fv_sparse_light(const fv_sparse_args &a, uint32_
       rec.n = n;
       rec.wv = wv;
       rec.f = f;
-      const uint64_t place = fv_slot_place((h << FV_NB_CLASS_SHIFT) | q, number, a.slot_region, gridDim.x);
+      // (fv_slot_place for a number below the block's threads, which is below FV_SLOT_PRIMARY or below the region)
+      const uint64_t place = ((h << FV_NB_CLASS_SHIFT) | q) * min(a.slot_region, FV_SLOT_PRIMARY) + number;
       a.slots[place] = rec;
       if (DELTA) a.slot_n2[place] = n2;
       a.Wt[p] = fv_sentinel(number);
@@ -524,7 +526,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
   // where the block's records lie (fv_slot_place, the block's part of it formed once)
   const uint32_t slot_primary = min(a.slot_region, FV_SLOT_PRIMARY);
   const uint64_t place_low = regions ? (uint64_t)blk * slot_primary : slot_first;
-  const uint64_t place_high = regions ? fv_slot_place(blk, slot_primary, a.slot_region, gridDim.x) - slot_primary : slot_first;
+  const uint64_t place_high = regions ? fv_slot_place(blk, slot_primary, a.slot_region, a.n_blocks) - slot_primary : slot_first;
 
   const uint32_t stage_cap = fv_sparse_stage_cap(a.stride);  // window ids staged in LDS at a time
   const bool staged_once = !DELTA && c_h <= stage_cap;  // the usual case: the neuron's window ids are staged here
@@ -660,6 +662,10 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
       // number of the round's first record, for the sentinels (saturated: a step with more records than a
       // sentinel can name is not finished by the launch that reads the numbers)
       const uint32_t record0 = (uint32_t)min((regions ? 0ull : slot_first) + emitted, (uint64_t)FV_SENTINEL_MAX);
+      // a round's records are numbered from a multiple of the list's length: all in the first part of the block's
+      // region or all in the second (fv_slot_place)
+      static_assert(FV_SLOT_PRIMARY % FV_SP_LIST_CAP == 0, "a round of records does not straddle the two parts of a region");
+      const uint64_t round_place = emitted < slot_primary ? place_low : place_high;
       // the row's two largest weights: the same address in the whole block, fetched where they are used
       const float2 top2 = a.top2_known ? a.row_top2[h] : make_float2(0.0f, 0.0f);
       for (uint32_t eb = tid; eb < take; eb += 4 * T) {
@@ -699,7 +705,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
             rec.wv = wv[u];
             rec.f = fe[u];
             const uint32_t number = emitted + eb + u * T;
-            const uint64_t place = (number < slot_primary ? place_low : place_high) + number;
+            const uint64_t place = round_place + number;
             a.slots[place] = rec;
             if (DELTA) a.slot_n2[place] = n2e[u];
             a.Wt[pe[u]] = fv_sentinel(record0 + eb + u * T);
