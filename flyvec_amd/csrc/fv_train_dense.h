@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256) void fv_absmax_kernel(fv_dense_args a) {
     p4 += FV_ABSMAX_UNROLL * stride;
     if (p4 < a.total4) fv_dense_load(a, p4, stride, w);
   }
-  const float bm = fv_block_max_nonneg(m, smem4);
+  const float bm = fv_block_max_nonneg<4>(m, smem4);
   if (threadIdx.x == 0) a.bmax[blockIdx.x] = bm;
 }
 
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(TB) void fv_update_kernel(fv_dense_args a) {
     }
     for (uint32_t i = 4 * n4 + tid; i < a.n_bmax; i += TB) nc = fmaxf(nc, a.bmax[i]);
   }
-  nc = fv_block_max_nonneg(nc, smem16);
+  nc = fv_block_max_nonneg<TB / 64>(nc, smem16);
   if (tid == 0) {
     sh_s = a.prec > nc ? a.eps / a.prec : a.eps / nc;  // flyvec/src/cuda_funcs.cu:1797-1799
     if (blockIdx.x == 0) a.scalars[0] = nc;

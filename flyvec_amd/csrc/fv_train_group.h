@@ -63,20 +63,26 @@ __device__ __forceinline__ float fv_sparse_ds2(float xx, float wv, float f, uint
 }
 
 // Block-wide maximum of non-negative floats (blocks of up to 16 waves; smem holds one float per wave).
+// WAVES: the block's waves where the caller knows them at compile time. blockDim.x is one of the launch's hidden
+// arguments: the compiler fetches it where it is first used, and that first use then waits for a trip to memory
+// in the middle of the kernel (0: read it).
+template <uint32_t WAVES = 0>
 __device__ __forceinline__ float fv_block_max_nonneg(float m, float *smem) {
   const uint32_t wm = fv_wave_max_u32(__float_as_uint(m));
   __syncthreads();
   if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = __uint_as_float(wm);
   __syncthreads();
   float r = smem[0];
-  for (uint32_t i = 1; i < (blockDim.x >> 6); ++i) r = fmaxf(r, smem[i]);
+  const uint32_t n_waves = WAVES ? WAVES : blockDim.x >> 6;
+  for (uint32_t i = 1; i < n_waves; ++i) r = fmaxf(r, smem[i]);
   return r;
 }
 
 // Sum over the block of one value per thread (result in every thread).
+template <uint32_t WAVES = 0>
 __device__ __forceinline__ uint32_t fv_block_sum_u32(uint32_t v, uint32_t *smem /*17*/) {
   v = fv_wave_sum_u32(v);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = WAVES ? (int)WAVES : (int)(blockDim.x >> 6);
   __syncthreads();
   if (lane == 0) smem[wave] = v;
   __syncthreads();
@@ -118,9 +124,10 @@ __device__ __forceinline__ float fv_wave_tree_sum(float v) {
 // sums meet in smem (16 floats) and every thread adds them up, the waves a block does not have counting as +0
 // (no value here is -0, so that changes no bit). LDS-only barriers.
 __device__ __forceinline__ void fv_lds_barrier();
+template <uint32_t WAVES = 0>
 __device__ __forceinline__ float fv_block_tree_sum(float v, float *smem /*16*/) {
   const float ws = fv_wave_tree_sum(v);
-  const uint32_t wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+  const uint32_t wave = threadIdx.x >> 6, n_waves = WAVES ? WAVES : blockDim.x >> 6;
   fv_lds_barrier();  // whoever still reads smem from an earlier use has done so
   if ((threadIdx.x & 63u) == 0) smem[wave] = ws;
   fv_lds_barrier();

@@ -235,7 +235,7 @@ __device__ __forceinline__ void fv_sparse_light(const fv_sparse_args &a, uint32_
     atomicAdd(&sh_hits[0], hits1);
     atomicAdd(&sh_hits[1], hits2);
   }
-  const float bm = fv_block_max_nonneg(ds_max, wave_max);  // behind its barriers every wave's hits are counted
+  const float bm = fv_block_max_nonneg<FV_SP_THREADS / 64>(ds_max, wave_max);  // behind its barriers every wave's hits are counted
   if (tid == 0) {
     a.bmax_sparse[blk] = bm;
     a.row_hits[blk] = min(sh_hits[0], 3u) | (min(sh_hits[1], 3u) << 2);
@@ -422,9 +422,9 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
           }
         }
       }
-      x_h = fv_block_tree_sum(part, wave_max);
+      x_h = fv_block_tree_sum<T / 64>(part, wave_max);
       // the second neurons' total is added to the winners' (the checker's order)
-      if (DELTA) x_h = __fadd_rn(x_h, fv_block_tree_sum(part2, wave_max));
+      if (DELTA) x_h = __fadd_rn(x_h, fv_block_tree_sum<T / 64>(part2, wave_max));
     }
     base = 0;
     if (c_h != 0 && a.slot_region == 0) {
@@ -455,7 +455,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
           }
         }
       }
-      base = fv_block_sum_u32((uint32_t)(-((int)below.x + (int)below.y)), red2);
+      base = fv_block_sum_u32<T / 64>((uint32_t)(-((int)below.x + (int)below.y)), red2);
     }
     if (q == 0 && tid == 0) {
       a.group_base_out[h] = base;  // used where it was counted
@@ -726,7 +726,7 @@ __device__ __forceinline__ void fv_sparse_block(const fv_sparse_args &a) {
     atomicAdd(&sh_hits[0], hits1);
     atomicAdd(&sh_hits[1], hits2);
   }
-  const float bm = fv_block_max_nonneg(ds_max, wave_max);  // behind its barriers every wave's hits are counted
+  const float bm = fv_block_max_nonneg<FV_SP_THREADS / 64>(ds_max, wave_max);  // behind its barriers every wave's hits are counted
   if (tid == 0) {
     a.bmax_sparse[blk] = bm;
     a.slot_count[blk] = emitted;
