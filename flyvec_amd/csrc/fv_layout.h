@@ -46,8 +46,8 @@ static inline uint64_t fv_matrix_gather_reach(uint32_t K, uint64_t N) {
 // of its own (n_blocks blocks): the first FV_SLOT_PRIMARY records of all blocks side by side, the others in a second
 // part with the rest of every region. Nearly every block has fewer records than that, so a step's records lie
 // within n_blocks * FV_SLOT_PRIMARY records (26 MB at 1600 blocks) instead of being strewn over all regions (256 MB at
-// 10000 records each: the sparse launch then took 16.8 us instead of 14.8 in some processes, the address
-// translation's reach being the difference), and only the few heaviest neurons' blocks touch the second part.
+// 10000 records each; with that layout the sparse launch was measured at 16.8 us instead of 14.8 in some processes
+// and not in others), and only the few heaviest neurons' blocks touch the second part.
 #ifndef FV_SLOT_PRIMARY
 #define FV_SLOT_PRIMARY 1024u
 #endif
