@@ -703,12 +703,14 @@ def test_delta_with_ties_and_heavy_neurons(gpu, oracle_lib):
     for tie in (0, 1):
         Wg, Wo = run_both_delta(oracle_lib, V=V, K=K, w=5, B=256, steps=4, delta=0.5, tie=tie, W0=W0)
         assert np.array_equal(Wg, Wo)
-    V, K, B = 300, 6, 7000
-    W0 = synthetic.synapses(K, V, sigma=0.01)
-    W0[2] = np.abs(W0[2]) + 1.0
-    W0[4] = np.abs(W0[4]) + 0.5
-    Wg, Wo = run_both_delta(oracle_lib, V=V, K=K, w=11, B=B, steps=2, delta=0.3, W0=W0, n_tokens=120000)
-    assert np.array_equal(Wg, Wo)
+    # (V = 12000: each of the two neurons' class blocks has more records than the first part of its slot region holds)
+    for V in (300, 12000):
+        K, B = 6, 7000
+        W0 = synthetic.synapses(K, V, sigma=0.01)
+        W0[2] = np.abs(W0[2]) + 1.0
+        W0[4] = np.abs(W0[4]) + 0.5
+        Wg, Wo = run_both_delta(oracle_lib, V=V, K=K, w=11, B=B, steps=2, delta=0.3, W0=W0, n_tokens=120000)
+        assert np.array_equal(Wg, Wo)
 
 
 def test_delta_epoch_schedule_and_driver(gpu, oracle_lib):
